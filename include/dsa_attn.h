@@ -1,0 +1,104 @@
+/*
+ * dsa_attn.h - C ABI of the MI355X (gfx950) packed-sequence DSA attention library.
+ *
+ * The library replaces the one device routine the reference's attention layers call,
+ *   torch.nn.attention.varlen.varlen_attn(q, k, v, cu_seq_q, cu_seq_k, max_q, max_k, window_size=(-1, 0))
+ * reached from train/model_attention.py:123-132, models/qwen3_vl/model.py:41-46 and
+ * models/qwen3_5/model.py:93-98, and extends it with the four DSA stages
+ * (indexer score -> top-k -> sparse forward -> sparse backward).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless it says "host"; tensors are row-major contiguous;
+ *   - q (T,Hq,D), k/v (T,Hkv,D), q_idx (T,Hi,Di), k_idx (T,Di), w_idx (T,Hi): bf16 (dtype code below);
+ *   - cu_seqlens (N+1) int32, cu[0]=0, cu[N]=T, non-decreasing (zero-length segments allowed, the pad
+ *     tail is one more segment: data/energon_dataloader.py:431-464, models/qwen3_vl/model.py:757-765);
+ *   - idx (T,K) int32: global packed row ids of the selected keys, ascending, padded with -1;
+ *     n (T) int32: how many are valid.  idx == NULL and n == NULL select every causal key of the
+ *     token's own segment (the reference's dense causal semantics);
+ *   - lse (Hq,T) fp32 natural-log softmax normaliser (what the flash kernel behind varlen_attn saves);
+ *   - stream is a hipStream_t passed as void*; all work is enqueued on it, nothing synchronises;
+ *   - every entry returns 0 on success or a negative dsa_status; dsa_last_error() gives the text
+ *     (thread-local).  No exception crosses the boundary.
+ */
+#ifndef DSA_ATTN_H
+#define DSA_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    DSA_OK = 0,
+    DSA_ERR_ARG = -1,          /* bad shape / null pointer / inconsistent sizes */
+    DSA_ERR_UNSUPPORTED = -2,  /* dtype or head geometry the kernels do not cover */
+    DSA_ERR_WORKSPACE = -3,    /* workspace too small */
+    DSA_ERR_HIP = -4           /* a HIP call or launch failed */
+} dsa_status;
+
+#define DSA_DTYPE_BF16 0
+#define DSA_DTYPE_FP32 1 /* accepted by the Python host only (it rounds to bf16 first) */
+
+/* Library identification, e.g. "dsa-attn-gfx950 0.1".  (no reference counterpart) */
+const char *dsa_version(void);
+/* Text of the last error raised on the calling thread ("" if none). */
+const char *dsa_last_error(void);
+
+/*
+ * Stage D1 - lightning-indexer scores for the query rows [row_begin,row_end).
+ *   scores[(t-row_begin)*ld + (s - seg_start(t))] = scale * sum_j w[t,j] * relu(q_idx[t,j,:] . k_idx[s,:])
+ * for s in [seg_start(t), t].  Columns beyond the row's own position are left untouched.
+ * Rows with pos(t)+1 <= skip_dense_k are skipped (their top-k is the whole causal window).
+ * No reference counterpart (the reference has no indexer); formula of the DSA operator.
+ */
+int dsa_indexer_scores(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu_seqlens,
+                       int T, int N, int Hi, int Di, float scale, int dtype, int row_begin, int row_end,
+                       int skip_dense_k, float *scores, int64_t ld, void *stream);
+
+/*
+ * Stage D2 - per-query top-k of materialised scores (also the bit-exactness test hook).
+ * Row t keeps the min(K, pos+1) columns first under (score descending, column ascending); -0.0 == +0.0.
+ * Writes global row ids ascending into idx[t*K ...], -1 padded, and n[t].
+ */
+int dsa_topk_from_scores(const float *scores, int64_t ld, int row_begin, int row_end, const int32_t *cu_seqlens,
+                         int T, int N, int K, int32_t *idx, int32_t *n, void *stream);
+
+/* Bytes of workspace dsa_index_topk needs (score rows are produced in chunks that fit). */
+size_t dsa_index_topk_workspace_bytes(int T, int max_seqlen, int K);
+
+/*
+ * Stages D1+D2 over the whole packed batch.  ws must hold dsa_index_topk_workspace_bytes().
+ * Stands where a DSA layer would call its indexer before attention; no reference counterpart.
+ */
+int dsa_index_topk(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu_seqlens,
+                   int T, int N, int Hi, int Di, int K, float scale, int dtype, int max_seqlen,
+                   int32_t *idx, int32_t *n, void *ws, size_t ws_bytes, void *stream);
+
+/*
+ * Stage D3 - attention forward over the selected keys (idx/n), or over every causal key of the own
+ * segment when idx == NULL: that case is the drop-in for varlen_attn(..., window_size=(-1,0))
+ * (train/model_attention.py:123-132; models/qwen3_vl/model.py:41-46; models/qwen3_5/model.py:93-98).
+ * q head h reads kv head h / (Hq/Hkv) (models/qwen3/model.py:125-129).  softmax in fp32.
+ */
+int dsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
+                 const int32_t *cu_seqlens, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
+                 int dtype, void *out, float *lse, void *stream);
+
+/* Bytes of workspace dsa_attn_bwd needs (softmax row terms + the inverted selection bitmap). */
+size_t dsa_attn_bwd_workspace_bytes(int T, int Hq, int max_seqlen, int has_idx);
+
+/*
+ * Stage D4 - gradients of D3 (the autograd backward of varlen_attn restricted to the selected keys;
+ * aten::_flash_attention_backward in the reference's stack).  Deterministic: no atomics on dq/dk/dv.
+ */
+int dsa_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out, const float *lse,
+                 const int32_t *idx, const int32_t *n, const int32_t *cu_seqlens, int T, int N, int Hq, int Hkv,
+                 int D, int K, float softmax_scale, int dtype, int max_seqlen, void *dq, void *dk, void *dv,
+                 void *ws, size_t ws_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DSA_ATTN_H */

@@ -1,0 +1,251 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on the same seeded inputs.
+
+Bars: top-k index sets bit-exact given identical fp32 scores; outputs and gradients within
+max-abs 2e-2 and cosine > 0.9995 of the fp32 oracle."""
+import math
+
+import pytest
+import torch
+
+from oracle import dsa_ref as R
+from tests.util import assert_close_bf16, oracle_topk_from_gpu_scores
+from vlm_training_amd import ops, workloads as W
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _log(msg):
+    print(msg, flush=True)
+
+
+# ------------------------------------------------------------------------------------------ D2
+def _topk_case(scores, cu, K):
+    T = scores.shape[0]
+    idx, n = ops.topk_from_scores(scores.to(DEV).contiguous(), torch.tensor(cu, dtype=torch.int32, device=DEV), K)
+    torch.cuda.synchronize()
+    want_idx, want_n = oracle_topk_from_gpu_scores(scores, cu, K)
+    assert torch.equal(n.cpu(), want_n)
+    bad = (idx.cpu() != want_idx).any(dim=1).nonzero().flatten()
+    assert bad.numel() == 0, f"rows differ: {bad[:8].tolist()} got {idx[bad[0]].tolist()[:16]} want {want_idx[bad[0]].tolist()[:16]}"
+
+
+@pytest.mark.parametrize("K", [1, 7, 64, 300])
+def test_topk_bit_exact_random_and_ties(K):
+    _log(f"topk K={K}")
+    g = torch.Generator().manual_seed(K)
+    cu = [0, 130, 130, 700, 1000]
+    T, ld = cu[-1], 576
+    for kind in ("normal", "quantised", "all_equal", "signed_zero", "relu_like"):
+        sc = torch.randn(T, ld, generator=g)
+        if kind == "quantised":
+            sc = torch.round(sc * 4) / 4
+        elif kind == "all_equal":
+            sc = torch.full((T, ld), 0.125)
+        elif kind == "signed_zero":
+            sc = torch.zeros(T, ld)
+            sc[:, 1::2] = -0.0
+            sc[:, ::7] = torch.randn(T, len(range(0, ld, 7)), generator=g).clamp(min=0) * 0.0
+        elif kind == "relu_like":
+            sc = torch.relu(sc) * torch.randn(T, 1, generator=g)
+        _topk_case(sc, cu, K)
+
+
+def test_topk_long_rows_uncached_path():
+    _log("topk long rows")
+    g = torch.Generator().manual_seed(3)
+    L = 9000                                    # longer than the LDS key cache
+    rows = [8191, 8192, 8193, L - 1]
+    cu = [0, L]
+    sc = torch.full((L, L), float("nan"))       # only a few rows are filled and checked
+    K = 2048
+    scd = torch.zeros(L, L)
+    for r in rows:
+        scd[r] = torch.round(torch.randn(L, generator=g) * 64) / 64
+    idx, n = ops.topk_from_scores(scd.to(DEV), torch.tensor(cu, dtype=torch.int32, device=DEV), K)
+    for r in rows:
+        want = R.topk_from_score_rows([scd[r, :r + 1]], K)[0]
+        assert idx[r].cpu().tolist() == want, r
+        assert int(n[r]) == K
+
+
+# ------------------------------------------------------------------------------------------ D1
+@pytest.mark.parametrize("Hi,Di", [(4, 32), (32, 64), (64, 128), (32, 128), (20, 64)])
+def test_indexer_scores_match_oracle(Hi, Di):
+    _log(f"indexer Hi={Hi} Di={Di}")
+    g = torch.Generator().manual_seed(Hi * 1000 + Di)
+    cu = [0, 70, 70, 333, 520]
+    T = cu[-1]
+    qi = (torch.randn(T, Hi, Di, generator=g) * 0.5).bfloat16()
+    ki = (torch.randn(T, Di, generator=g) * 0.5).bfloat16()
+    w = (torch.randn(T, Hi, generator=g) * 0.5).bfloat16()
+    sc = ops.indexer_scores(qi.to(DEV), ki.to(DEV), w.to(DEV), torch.tensor(cu, dtype=torch.int32, device=DEV), 263).cpu()
+    for a, b in R.segments(cu):
+        L = b - a
+        if L == 0:
+            continue
+        want = R.indexer_scores_segment(qi[a:b], ki[a:b], w[a:b])
+        low = torch.tril(torch.ones(L, L, dtype=torch.bool))
+        got = sc[a:b, :L]
+        err = (got[low] - want[low]).abs().max().item()
+        assert err < 2e-5 * max(1.0, want[low].abs().max().item()), err
+        assert torch.isneginf(sc[a:b, :L][~low]).all()      # untouched above the diagonal
+
+
+# ------------------------------------------------------------------------------------------ whole operator
+def _run_case(w, check_bwd=True):
+    t = W.make_inputs(w, device="cpu")
+    cu = t["cu_seqlens"]
+    d = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in t.items()}
+    q = d["q"].clone().requires_grad_(True)
+    k = d["k"].clone().requires_grad_(True)
+    v = d["v"].clone().requires_grad_(True)
+    out, idx, n = ops.dsa_varlen_attn(q, k, v, d["cu_seqlens"], w.max_seqlen, indexer_q=d["q_idx"], indexer_k=d["k_idx"],
+                                      indexer_w=d["w_idx"], top_k=w.top_k, return_indices=True)
+    # (1) top-k bit-exact given the GPU's own fp32 scores
+    sc = ops.indexer_scores(d["q_idx"], d["k_idx"], d["w_idx"], d["cu_seqlens"], w.max_seqlen).cpu()
+    want_idx, want_n = oracle_topk_from_gpu_scores(sc, cu.tolist(), w.top_k)
+    assert torch.equal(n.cpu(), want_n)
+    assert torch.equal(idx.cpu(), want_idx), "top-k index sets differ from the oracle on identical scores"
+    # (2) outputs / gradients against the fp32 oracle on the same selection
+    if check_bwd:
+        ref_out, rdq, rdk, rdv = R.sparse_attention_grads(t["q"], t["k"], t["v"], want_idx, want_n, cu, t["dout"])
+        out.backward(d["dout"])
+        torch.cuda.synchronize()
+        res = [assert_close_bf16(out, ref_out, "out"), assert_close_bf16(q.grad, rdq, "dq"),
+               assert_close_bf16(k.grad, rdk, "dk"), assert_close_bf16(v.grad, rdv, "dv")]
+    else:
+        ref_out = R.sparse_attention(t["q"], t["k"], t["v"], want_idx, want_n, cu)
+        res = [assert_close_bf16(out, ref_out, "out")]
+    _log(f"  {w.name}: " + " ".join(f"({e:.2e},{c:.6f})" for e, c in res))
+    return out
+
+
+def test_c1_toy_fp32_full():
+    _log("C1 full")
+    _run_case(W.C1)
+
+
+@pytest.mark.parametrize("name,segs,K", [
+    ("C2", (700, 333, 40, 0, 515, 204), 256),
+    ("C3", (1100, 64, 600, 284), 512),
+    ("C5", (300, 65, 73, 107, 500, 33, 74), 128),
+])
+def test_scaled_configs(name, segs, K):
+    _log(f"scaled {name}")
+    _run_case(W.scaled(W.WORKLOADS[name], segs, top_k=K, name=name + "-scaled"))
+
+
+def test_dense_path_equals_reference_semantics():
+    _log("dense path")
+    g = torch.Generator().manual_seed(11)
+    cu = [0, 190, 190, 400, 431]
+    T = cu[-1]
+    for Hq, Hkv, D in ((8, 2, 64), (4, 4, 128), (16, 2, 256), (6, 2, 128)):
+        q = (torch.randn(T, Hq, D, generator=g) * 0.7).bfloat16()
+        k = (torch.randn(T, Hkv, D, generator=g) * 0.7).bfloat16()
+        v = (torch.randn(T, Hkv, D, generator=g) * 0.7).bfloat16()
+        do = torch.randn(T, Hq, D, generator=g).bfloat16()
+        qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+        out = ops.dsa_varlen_attn(qd, kd, vd, torch.tensor(cu, dtype=torch.int32, device=DEV), 210)
+        out.backward(do.to(DEV))
+        qr, kr, vr = (x.float().requires_grad_(True) for x in (q, k, v))
+        ref = R.dense_varlen_causal(qr, kr, vr, cu)
+        ref.backward(do.float())
+        assert_close_bf16(out, ref, f"out {Hq}/{Hkv}/{D}")
+        assert_close_bf16(qd.grad, qr.grad, "dq")
+        assert_close_bf16(kd.grad, kr.grad, "dk")
+        assert_close_bf16(vd.grad, vr.grad, "dv")
+
+
+def test_topk_at_least_longest_segment_is_dense():
+    _log("K >= L")
+    w = W.scaled(W.C2, (300, 120, 77), top_k=512, name="C2-dense")
+    t = W.make_inputs(w, device=DEV)
+    out, idx, n = ops.dsa_varlen_attn(t["q"], t["k"], t["v"], t["cu_seqlens"], w.max_seqlen, indexer_q=t["q_idx"],
+                                      indexer_k=t["k_idx"], indexer_w=t["w_idx"], top_k=512, return_indices=True)
+    dense = ops.dsa_varlen_attn(t["q"], t["k"], t["v"], t["cu_seqlens"], w.max_seqlen)
+    assert torch.equal(out, dense)                       # same kernel, same key order -> bit-identical
+    cu = w.cu
+    for a, b in zip(cu[:-1], cu[1:]):
+        for r in (a, (a + b) // 2, b - 1):
+            assert idx[r, : r - a + 1].cpu().tolist() == list(range(a, r + 1)) and int(n[r]) == r - a + 1
+            assert (idx[r, r - a + 1:] == -1).all()
+
+
+def test_packing_equivalence_pad_independence_determinism():
+    _log("invariants")
+    w = W.scaled(W.C2, (400, 150, 290), top_k=96, name="C2-inv")
+    t = W.make_inputs(w, device=DEV)
+    kw = dict(indexer_q=t["q_idx"], indexer_k=t["k_idx"], indexer_w=t["w_idx"], top_k=96, return_indices=True)
+    out, idx, n = ops.dsa_varlen_attn(t["q"], t["k"], t["v"], t["cu_seqlens"], w.max_seqlen, **kw)
+    out2, idx2, _ = ops.dsa_varlen_attn(t["q"], t["k"], t["v"], t["cu_seqlens"], w.max_seqlen, **kw)
+    assert torch.equal(out, out2) and torch.equal(idx, idx2)            # I4 bitwise determinism
+    cu = w.cu
+    for a, b in zip(cu[:-1], cu[1:]):                                   # I2 packed == solo
+        sl = slice(a, b)
+        solo, sidx, _ = ops.dsa_varlen_attn(t["q"][sl], t["k"][sl], t["v"][sl], torch.tensor([0, b - a], dtype=torch.int32, device=DEV),
+                                            b - a, indexer_q=t["q_idx"][sl], indexer_k=t["k_idx"][sl], indexer_w=t["w_idx"][sl],
+                                            top_k=96, return_indices=True)
+        assert torch.equal(torch.where(idx[sl] >= 0, idx[sl] - a, idx[sl]), sidx)
+        assert torch.equal(out[sl], solo)
+    pad = 100                                                           # I3 pad tail as one more segment
+    ext = {name: torch.cat([t[name], torch.zeros(pad, *t[name].shape[1:], dtype=t[name].dtype, device=DEV)])
+           for name in ("q", "k", "v", "q_idx", "k_idx", "w_idx")}
+    cu_pad = torch.tensor(cu + [cu[-1] + pad], dtype=torch.int32, device=DEV)
+    outp = ops.dsa_varlen_attn(ext["q"], ext["k"], ext["v"], cu_pad, w.max_seqlen, indexer_q=ext["q_idx"],
+                               indexer_k=ext["k_idx"], indexer_w=ext["w_idx"], top_k=96)
+    assert torch.equal(outp[: cu[-1]], out) and torch.isfinite(outp).all()
+
+
+def test_backward_is_deterministic_and_unselected_keys_get_zero():
+    _log("bwd determinism")
+    w = W.scaled(W.C3, (500, 260), top_k=32, name="C3-det")
+    t = W.make_inputs(w, device=DEV)
+    grads = []
+    for _ in range(2):
+        q, k, v = (t[x].clone().requires_grad_(True) for x in ("q", "k", "v"))
+        out, idx, n = ops.dsa_varlen_attn(q, k, v, t["cu_seqlens"], w.max_seqlen, indexer_q=t["q_idx"], indexer_k=t["k_idx"],
+                                          indexer_w=t["w_idx"], top_k=32, return_indices=True)
+        out.backward(t["dout"])
+        grads.append((q.grad.clone(), k.grad.clone(), v.grad.clone()))
+    for a, b in zip(*grads):
+        assert torch.equal(a, b)
+    used = torch.zeros(w.T, dtype=torch.bool, device=DEV)
+    used[idx[idx >= 0].long()] = True
+    assert (grads[0][1][~used] == 0).all() and (grads[0][2][~used] == 0).all()
+
+
+def test_reference_named_entry_points():
+    _log("entry points")
+    import vlm_training_amd as M
+    g = torch.Generator().manual_seed(5)
+    cu = torch.tensor([0, 100, 260], dtype=torch.int32, device=DEV)
+    q = torch.randn(260, 8, 64, generator=g).bfloat16().to(DEV)
+    k = torch.randn(260, 2, 64, generator=g).bfloat16().to(DEV)
+    v = torch.randn(260, 2, 64, generator=g).bfloat16().to(DEV)
+    a = M.dispatch_varlen_attention(q, k, v, cu, 160)
+    b = M.run_varlen_attn(q, k, v, cu, 160)
+    c = M.varlen_attn(q, k, v, cu, cu, 160, 160, is_causal=True)
+    hf, none = M.varlen_attention_forward(q.transpose(0, 1).unsqueeze(0), k.transpose(0, 1).unsqueeze(0),
+                                          v.transpose(0, 1).unsqueeze(0), cu.unsqueeze(0))
+    assert none is None and hf.shape == (1, 260, 8, 64)
+    assert torch.equal(a, b) and torch.equal(a, c) and torch.equal(a, hf[0])
+    ref = R.dense_varlen_causal(q.cpu(), k.cpu(), v.cpu(), cu.cpu())
+    assert_close_bf16(a, ref, "dispatch_varlen_attention")
+
+
+def test_argument_errors_cross_the_boundary_as_exceptions():
+    q = torch.zeros(8, 4, 64, dtype=torch.bfloat16, device=DEV)
+    k = torch.zeros(8, 3, 64, dtype=torch.bfloat16, device=DEV)
+    cu = torch.tensor([0, 8], dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError):
+        ops.dsa_varlen_attn(q, k, k, cu, 8)
+    k = torch.zeros(8, 2, 96, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError):
+        ops.dsa_varlen_attn(q, k, k, cu, 8)
+    q = torch.zeros(8, 4, 96, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError):
+        ops.dsa_varlen_attn(q, k, k, cu, 8)            # head_dim 96 is not covered by the kernels
+    with pytest.raises(RuntimeError):
+        ops.dsa_varlen_attn(q.cpu(), k.cpu(), k.cpu(), cu.cpu(), 8)

@@ -1,0 +1,290 @@
+"""Pins the CPU oracle with checks that do not reuse its formulas: pure-Python loops on tiny
+inputs, library routines (SDPA, numpy einsum), closed-form special cases, fp64 gradcheck and the
+packing invariants the reference's own tests use (models/tests/test_qwen3_5_exhaustive.py:393-498)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import dsa_ref as R
+
+
+def rnd(*shape, seed=0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g, dtype=dtype)
+
+
+# ---------------------------------------------------------------- brute-force restatements
+def brute_dense(q, k, v, cu, scale=None):
+    T, Hq, D = q.shape
+    G = Hq // k.shape[1]
+    scale = scale if scale is not None else 1.0 / math.sqrt(D)
+    out = torch.zeros(T, Hq, D, dtype=torch.float64)
+    for a, b in zip(cu[:-1], cu[1:]):
+        for t in range(a, b):
+            for h in range(Hq):
+                logits = [float(torch.dot(q[t, h].double(), k[s, h // G].double())) * scale for s in range(a, t + 1)]
+                m = max(logits)
+                e = [math.exp(x - m) for x in logits]
+                z = sum(e)
+                for j, s in enumerate(range(a, t + 1)):
+                    out[t, h] += (e[j] / z) * v[s, h // G].double()
+    return out
+
+
+def brute_scores(q_idx, k_idx, w, scale):
+    L, Hi, Di = q_idx.shape
+    sc = [[-math.inf] * L for _ in range(L)]
+    for t in range(L):
+        for s in range(t + 1):
+            acc = 0.0
+            for j in range(Hi):
+                d = float(torch.dot(q_idx[t, j].double(), k_idx[s].double()))
+                acc += float(w[t, j]) * max(d, 0.0)
+            sc[t][s] = acc * scale
+    return sc
+
+
+def brute_topk_row(row, K):
+    """row: list of floats (valid part only)."""
+    order = sorted(range(len(row)), key=lambda i: (-row[i], i))
+    return sorted(order[:K])
+
+
+def brute_sparse(q, k, v, idx, scale=None):
+    T, Hq, D = q.shape
+    G = Hq // k.shape[1]
+    scale = scale if scale is not None else 1.0 / math.sqrt(D)
+    out = torch.zeros(T, Hq, D, dtype=torch.float64)
+    for t in range(T):
+        sel = [int(s) for s in idx[t].tolist() if s >= 0]
+        for h in range(Hq):
+            logits = [float(torch.dot(q[t, h].double(), k[s, h // G].double())) * scale for s in sel]
+            m = max(logits)
+            e = [math.exp(x - m) for x in logits]
+            z = sum(e)
+            for j, s in enumerate(sel):
+                out[t, h] += (e[j] / z) * v[s, h // G].double()
+    return out
+
+
+# ---------------------------------------------------------------- dense semantics
+def test_dense_matches_bruteforce_gqa():
+    cu = [0, 5, 5, 12, 14]                      # includes a zero-length segment
+    q, k, v = rnd(14, 4, 8, seed=1), rnd(14, 2, 8, seed=2), rnd(14, 2, 8, seed=3)
+    got = R.dense_varlen_causal(q, k, v, cu)
+    assert torch.allclose(got.double(), brute_dense(q, k, v, cu), atol=1e-5)
+
+
+def test_dense_first_token_is_v_and_rows_are_convex():
+    cu = [0, 7, 16]
+    q, k, v = rnd(16, 2, 4, seed=4), rnd(16, 2, 4, seed=5), rnd(16, 2, 4, seed=6)
+    o = R.dense_varlen_causal(q, k, v, cu)
+    for a in (0, 7):
+        assert torch.allclose(o[a], v[a], atol=1e-6)          # one valid key -> weight 1
+    v1 = torch.ones_like(v)
+    assert torch.allclose(R.dense_varlen_causal(q, k, v1, cu), torch.ones_like(q), atol=1e-6)
+
+
+def test_gqa_head_mapping_is_h_div_g():
+    # kv head 1 carries a marker value; only q heads 2,3 (G=2) may see it
+    T = 6
+    q, k = rnd(T, 4, 4, seed=7), rnd(T, 2, 4, seed=8)
+    v = torch.zeros(T, 2, 4)
+    v[:, 1] = 1.0
+    o = R.dense_varlen_causal(q, k, v, [0, T])
+    assert torch.all(o[:, :2] == 0) and torch.allclose(o[:, 2:], torch.ones(T, 2, 4), atol=1e-6)
+
+
+# ---------------------------------------------------------------- D1
+def test_scores_match_bruteforce_and_numpy():
+    L, Hi, Di = 9, 3, 5
+    qi, ki, w = rnd(L, Hi, Di, seed=9), rnd(L, Di, seed=10), rnd(L, Hi, seed=11)
+    sc = R.indexer_scores_segment(qi, ki, w, scale=0.37)
+    ref = torch.tensor(brute_scores(qi, ki, w, 0.37))
+    assert torch.allclose(sc.double(), ref.double(), atol=1e-5, rtol=1e-5)
+    ein = np.einsum("tj,tjs->ts", w.numpy(), np.maximum(np.einsum("tjd,sd->tjs", qi.numpy(), ki.numpy()), 0)) * 0.37
+    low = np.tril(np.ones((L, L), bool))
+    assert np.allclose(sc.numpy()[low], ein[low], atol=1e-5)
+    assert np.all(np.isneginf(sc.numpy()[~low]))
+
+
+def test_scores_single_head_unit_weight_and_default_scale():
+    L, Di = 6, 4
+    qi, ki = rnd(L, 1, Di, seed=12), rnd(L, Di, seed=13)
+    sc = R.indexer_scores_segment(qi, ki, torch.ones(L, 1))
+    want = torch.relu(qi[:, 0] @ ki.t()) * (Di ** -0.5)
+    low = torch.tril(torch.ones(L, L, dtype=torch.bool))
+    assert torch.allclose(sc[low], want[low], atol=1e-6)
+    assert R.default_index_scale(64, 128) == pytest.approx(1.0 / (math.sqrt(128) * 8))
+
+
+# ---------------------------------------------------------------- D2
+def _check_rows(scores, K, base=0):
+    idx, n = R.topk_select_segment(scores, K, base=base)
+    L = scores.shape[0]
+    for t in range(L):
+        want = brute_topk_row(scores[t, :t + 1].tolist(), K)
+        got = [int(x) - base for x in idx[t].tolist() if x >= 0]
+        assert got == want, (t, got, want)
+        assert int(n[t]) == min(K, t + 1) == len(got)
+        assert idx[t, len(got):].eq(-1).all()
+
+
+def test_topk_random_rows_match_python_sort():
+    L = 40
+    sc = rnd(L, L, seed=14).masked_fill(torch.triu(torch.ones(L, L, dtype=torch.bool), 1), float("-inf"))
+    for K in (1, 3, 16, 39, 40, 64):
+        _check_rows(sc, K, base=100)
+
+
+def test_topk_ties_take_lowest_index():
+    L = 24
+    low = torch.tril(torch.ones(L, L, dtype=torch.bool))
+    all_equal = torch.full((L, L), 0.25).masked_fill(~low, float("-inf"))
+    idx, n = R.topk_select_segment(all_equal, 5)
+    assert idx[20].tolist() == [0, 1, 2, 3, 4]
+    zeros = torch.zeros(L, L)
+    zeros[:, 1::2] = -0.0                        # +-0.0 must tie; the column decides
+    zeros = zeros.masked_fill(~low, float("-inf"))
+    idx, _ = R.topk_select_segment(zeros, 4)
+    assert idx[23].tolist() == [0, 1, 2, 3]
+    # duplicates straddling the K-th place: values 3,3,2,2,2,2,1 ... keep the two lowest-index 2s
+    row = torch.tensor([2.0, 3.0, 2.0, 1.0, 3.0, 2.0, 2.0, 0.0])
+    sc = torch.full((8, 8), float("-inf"))
+    sc[7] = row
+    for t in range(7):
+        sc[t, :t + 1] = 0.0
+    idx, _ = R.topk_select_segment(sc, 4)
+    assert idx[7].tolist() == [0, 1, 2, 4]
+    _check_rows(sc, 4)
+    _check_rows(zeros, 7)
+
+
+def test_topk_quantised_scores_many_ties():
+    L = 64
+    sc = torch.round(rnd(L, L, seed=15) * 2) / 2          # heavy duplication
+    sc = sc.masked_fill(torch.triu(torch.ones(L, L, dtype=torch.bool), 1), float("-inf"))
+    for K in (2, 8, 31):
+        _check_rows(sc, K)
+    rows = [sc[t, :t + 1] for t in range(L)]
+    rag = R.topk_from_score_rows(rows, 8)
+    idx, _ = R.topk_select_segment(sc, 8)
+    for t in range(L):
+        assert rag[t] == [int(x) for x in idx[t].tolist() if x >= 0]
+
+
+def test_topk_rejects_nan_and_bad_k():
+    sc = torch.zeros(4, 4)
+    sc[3, 1] = float("nan")
+    with pytest.raises(ValueError):
+        R.topk_select_segment(sc, 2)
+    with pytest.raises(ValueError):
+        R.topk_select_segment(torch.zeros(4, 4), 0)
+
+
+# ---------------------------------------------------------------- D3 / D4
+def _toy(seed=20, cu=(0, 11, 11, 30, 37), Hq=4, Hkv=2, D=8, Hi=2, Di=4):
+    T = cu[-1]
+    return dict(q=rnd(T, Hq, D, seed=seed), k=rnd(T, Hkv, D, seed=seed + 1), v=rnd(T, Hkv, D, seed=seed + 2),
+                q_idx=rnd(T, Hi, Di, seed=seed + 3), k_idx=rnd(T, Di, seed=seed + 4), w=rnd(T, Hi, seed=seed + 5),
+                cu=list(cu))
+
+
+def test_sparse_matches_bruteforce():
+    t = _toy()
+    out, idx, n = R.dsa_varlen_attn_ref(t["q"], t["k"], t["v"], t["cu"], t["q_idx"], t["k_idx"], t["w"], 5,
+                                        return_indices=True)
+    assert torch.allclose(out.double(), brute_sparse(t["q"], t["k"], t["v"], idx), atol=1e-5)
+    # I6: selected sets lie inside the causal window of the own segment, ascending, right count
+    for a, b in zip(t["cu"][:-1], t["cu"][1:]):
+        for r in range(a, b):
+            sel = [int(x) for x in idx[r].tolist() if x >= 0]
+            assert sel == sorted(set(sel)) and all(a <= s <= r for s in sel)
+            assert len(sel) == int(n[r]) == min(5, r - a + 1)
+
+
+def test_k_at_least_longest_segment_equals_dense():
+    t = _toy(seed=30)
+    dense = R.dense_varlen_causal(t["q"], t["k"], t["v"], t["cu"])
+    for K in (19, 64):
+        out, idx, n = R.dsa_varlen_attn_ref(t["q"], t["k"], t["v"], t["cu"], t["q_idx"], t["k_idx"], t["w"], K,
+                                            return_indices=True)
+        assert torch.allclose(out, dense, atol=1e-5)
+        for a, b in zip(t["cu"][:-1], t["cu"][1:]):
+            for r in range(a, b):
+                assert [int(x) for x in idx[r].tolist() if x >= 0] == list(range(a, r + 1))
+
+
+def test_lse_and_weights_sum_to_one():
+    t = _toy(seed=40)
+    idx, n = R.dsa_select(t["q_idx"], t["k_idx"], t["w"], t["cu"], 4)
+    ones = torch.ones_like(t["v"])
+    out, lse = R.sparse_attention(t["q"], t["k"], ones, idx, n, t["cu"], return_lse=True)
+    assert torch.allclose(out, torch.ones_like(out), atol=1e-6)
+    assert lse.shape == (4, t["cu"][-1]) and torch.isfinite(lse).all()
+
+
+def test_packing_equivalence_and_pad_independence():
+    t = _toy(seed=50, cu=(0, 13, 29))
+    K = 6
+    out, idx, _ = R.dsa_varlen_attn_ref(t["q"], t["k"], t["v"], t["cu"], t["q_idx"], t["k_idx"], t["w"], K,
+                                        return_indices=True)
+    for a, b in ((0, 13), (13, 29)):
+        solo, sidx, _ = R.dsa_varlen_attn_ref(t["q"][a:b], t["k"][a:b], t["v"][a:b], [0, b - a], t["q_idx"][a:b],
+                                              t["k_idx"][a:b], t["w"][a:b], K, return_indices=True)
+        assert torch.allclose(out[a:b], solo, atol=1e-6)
+        assert torch.equal(torch.where(idx[a:b] >= 0, idx[a:b] - a, idx[a:b]), sidx)
+    # appending a pad segment leaves earlier tokens alone (test_qwen3_5_exhaustive.py:463-498)
+    pad = 7
+    ext = {name: torch.cat([t[name], torch.zeros(pad, *t[name].shape[1:])]) for name in ("q", "k", "v", "q_idx", "k_idx", "w")}
+    out2 = R.dsa_varlen_attn_ref(ext["q"], ext["k"], ext["v"], [0, 13, 29, 29 + pad], ext["q_idx"], ext["k_idx"], ext["w"], K)
+    assert torch.equal(out2[:29], out)
+    assert torch.isfinite(out2).all()
+
+
+def test_gradients_gradcheck_fp64_and_dense_limit():
+    T, Hq, Hkv, D = 10, 2, 1, 3
+    cu = [0, 4, 10]
+    q, k, v = (rnd(T, Hq, D, seed=60, dtype=torch.float64).requires_grad_(True),
+               rnd(T, Hkv, D, seed=61, dtype=torch.float64).requires_grad_(True),
+               rnd(T, Hkv, D, seed=62, dtype=torch.float64).requires_grad_(True))
+    idx, n = R.dsa_select(rnd(T, 2, 3, seed=63), rnd(T, 3, seed=64), rnd(T, 2, seed=65), cu, 3)
+    fn = lambda a, b, c: R.sparse_attention(a, b, c, idx, n, cu)
+    assert torch.autograd.gradcheck(fn, (q, k, v), eps=1e-6, atol=1e-5)
+    # with K >= L the gradients are those of dense causal SDPA
+    t = _toy(seed=70, cu=(0, 9, 20))
+    idx, n = R.dsa_select(t["q_idx"], t["k_idx"], t["w"], t["cu"], 32)
+    dout = rnd(20, 4, 8, seed=71)
+    _, dq, dk, dv = R.sparse_attention_grads(t["q"], t["k"], t["v"], idx, n, t["cu"], dout)
+    qd, kd, vd = (t[x].clone().requires_grad_(True) for x in ("q", "k", "v"))
+    R.dense_varlen_causal(qd, kd, vd, t["cu"]).backward(dout)
+    for a, b in ((dq, qd.grad), (dk, kd.grad), (dv, vd.grad)):
+        assert torch.allclose(a, b, atol=1e-5)
+
+
+def test_unselected_keys_get_zero_gradient():
+    t = _toy(seed=80, cu=(0, 24))
+    idx, n = R.dsa_select(t["q_idx"], t["k_idx"], t["w"], t["cu"], 3)
+    used = set(int(x) for x in idx.flatten().tolist() if x >= 0)
+    _, _, dk, dv = R.sparse_attention_grads(t["q"], t["k"], t["v"], idx, n, t["cu"], rnd(24, 4, 8, seed=81))
+    for s in range(24):
+        if s not in used:
+            assert dk[s].abs().max() == 0 and dv[s].abs().max() == 0
+
+
+def test_hf_layout_adapter_and_pair_counts():
+    x = rnd(1, 3, 5, 4, seed=90)                       # (1,H,T,D)
+    y = R.hf_layout_to_packed(x)
+    assert y.shape == (5, 3, 4) and torch.equal(y, x[0].permute(1, 0, 2))
+    assert R.pair_counts([0, 256, 768, 1152, 2048], 128) == (640000, 229632)
+    P, S = R.pair_counts([0, 4, 10], 3)
+    assert P == 10 + 21 and S == (1 + 2 + 3 + 3) + (1 + 2 + 3 + 3 + 3 + 3)
+
+
+def test_determinism_bitwise():
+    t = _toy(seed=95)
+    a = R.dsa_varlen_attn_ref(t["q"], t["k"], t["v"], t["cu"], t["q_idx"], t["k_idx"], t["w"], 4)
+    b = R.dsa_varlen_attn_ref(t["q"], t["k"], t["v"], t["cu"], t["q_idx"], t["k_idx"], t["w"], 4)
+    assert torch.equal(a, b)

@@ -1,0 +1,7 @@
+"""MI355X-native packed-sequence DSA attention (gfx950 HIP kernels behind a C ABI)."""
+from .model_attention import (dispatch_varlen_attention, run_varlen_attn, varlen_attention_forward,  # noqa: F401
+                              varlen_attn)
+from .ops import dsa_varlen_attn, index_topk  # noqa: F401
+
+__all__ = ["dsa_varlen_attn", "index_topk", "varlen_attn", "dispatch_varlen_attention", "run_varlen_attn",
+           "varlen_attention_forward"]

@@ -1,0 +1,158 @@
+// C ABI of the library (declared in include/dsa_attn.h): argument checks, workspace layout, launches.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/dsa_attn.h"
+
+extern "C" {
+hipError_t dsa_launch_topk(const float *scores, int64_t ld, int row_begin, int row_end, const int32_t *cu, int N,
+                           int K, int max_row, int32_t *idx, int32_t *n, hipStream_t stream);
+hipError_t dsa_launch_indexer(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu, int N,
+                              int T, int Hi, int Di, float scale, int row_begin, int row_end, int skip_dense_k,
+                              float *scores, int64_t ld, hipStream_t stream);
+hipError_t dsa_launch_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
+                               const int32_t *cu, int N, int T, int Hq, int Hkv, int D, int K, float scale, void *out,
+                               float *lse, hipStream_t stream);
+hipError_t dsa_launch_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                               const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu, int N, int T,
+                               int Hq, int Hkv, int D, int K, float scale, int max_seqlen, void *dq, void *dk,
+                               void *dv, float *delta, uint32_t *bitmap, int ldw, hipStream_t stream);
+}
+
+static thread_local char g_err[512] = "";
+
+static int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+static int hip_fail(hipError_t e, const char *what) {
+    return fail(DSA_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+#define SCORE_CHUNK_BYTES ((size_t)1 << 30)
+static inline int64_t score_ld(int max_seqlen) { return (int64_t)align_up((size_t)max_seqlen, 32); }
+
+extern "C" const char *dsa_version(void) { return "dsa-attn-gfx950 0.1"; }
+extern "C" const char *dsa_last_error(void) { return g_err; }
+
+static int check_packed(int T, int N, const int32_t *cu) {
+    if (T < 0 || N < 1) return fail(DSA_ERR_ARG, "T=%d N=%d: need T>=0 and at least one segment", T, N);
+    if (!cu) return fail(DSA_ERR_ARG, "cu_seqlens is null");
+    return DSA_OK;
+}
+
+extern "C" int dsa_indexer_scores(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu, int T,
+                                  int N, int Hi, int Di, float scale, int dtype, int row_begin, int row_end,
+                                  int skip_dense_k, float *scores, int64_t ld, void *stream) {
+    if (int rc = check_packed(T, N, cu)) return rc;
+    if (dtype != DSA_DTYPE_BF16) return fail(DSA_ERR_UNSUPPORTED, "indexer inputs must be bf16 (dtype code %d)", dtype);
+    if (!q_idx || !k_idx || !w_idx || !scores) return fail(DSA_ERR_ARG, "null tensor pointer");
+    if (row_begin < 0 || row_end > T || row_begin > row_end) return fail(DSA_ERR_ARG, "bad row range [%d,%d)", row_begin, row_end);
+    if (Hi < 1 || Hi > 64 || !(Di == 32 || Di == 64 || Di == 128))
+        return fail(DSA_ERR_UNSUPPORTED, "indexer geometry Hi=%d Di=%d: need Hi<=64 and Di in {32,64,128}", Hi, Di);
+    hipError_t e = dsa_launch_indexer(q_idx, k_idx, w_idx, cu, N, T, Hi, Di, scale, row_begin, row_end, skip_dense_k,
+                                      scores, ld, (hipStream_t)stream);
+    return e == hipSuccess ? DSA_OK : hip_fail(e, "indexer launch");
+}
+
+extern "C" int dsa_topk_from_scores(const float *scores, int64_t ld, int row_begin, int row_end, const int32_t *cu,
+                                    int T, int N, int K, int32_t *idx, int32_t *n, void *stream) {
+    if (int rc = check_packed(T, N, cu)) return rc;
+    if (!scores || !idx || !n) return fail(DSA_ERR_ARG, "null tensor pointer");
+    if (K < 1) return fail(DSA_ERR_ARG, "top_k=%d must be >= 1", K);
+    if (row_begin < 0 || row_end > T || row_begin > row_end) return fail(DSA_ERR_ARG, "bad row range [%d,%d)", row_begin, row_end);
+    hipError_t e = dsa_launch_topk(scores, ld, row_begin, row_end, cu, N, K, (int)ld, idx, n, (hipStream_t)stream);
+    return e == hipSuccess ? DSA_OK : hip_fail(e, "top-k launch");
+}
+
+extern "C" size_t dsa_index_topk_workspace_bytes(int T, int max_seqlen, int K) {
+    (void)K;
+    if (T <= 0 || max_seqlen <= 0) return 0;
+    const size_t row_bytes = (size_t)score_ld(max_seqlen) * 4;
+    size_t rows = SCORE_CHUNK_BYTES / row_bytes;
+    if (rows < 64) rows = 64;
+    if (rows > (size_t)T) rows = (size_t)T;
+    return align_up(rows, 4) * row_bytes;
+}
+
+extern "C" int dsa_index_topk(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu, int T, int N,
+                              int Hi, int Di, int K, float scale, int dtype, int max_seqlen, int32_t *idx, int32_t *n,
+                              void *ws, size_t ws_bytes, void *stream) {
+    if (int rc = check_packed(T, N, cu)) return rc;
+    if (K < 1) return fail(DSA_ERR_ARG, "top_k=%d must be >= 1", K);
+    if (max_seqlen < 1 || max_seqlen > T) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
+    if (!idx || !n) return fail(DSA_ERR_ARG, "null output pointer");
+    if (T == 0) return DSA_OK;
+    const int64_t ld = score_ld(max_seqlen);
+    int64_t rows = ws ? (int64_t)(ws_bytes / ((size_t)ld * 4)) : 0;
+    rows &= ~(int64_t)3;
+    if (max_seqlen <= K) rows = T;   // every row is dense: no score is read or written
+    else if (rows < 4) return fail(DSA_ERR_WORKSPACE, "workspace of %zu bytes holds no score chunk (row = %lld bytes)", ws_bytes, (long long)ld * 4);
+    if (rows > T) rows = T;
+    for (int64_t r0 = 0; r0 < T; r0 += rows) {
+        const int r1 = (int)((r0 + rows < T) ? r0 + rows : T);
+        if (max_seqlen > K) {
+            int rc = dsa_indexer_scores(q_idx, k_idx, w_idx, cu, T, N, Hi, Di, scale, dtype, (int)r0, r1, K, (float *)ws, ld, stream);
+            if (rc) return rc;
+        }
+        hipError_t e = dsa_launch_topk((const float *)ws, ld, (int)r0, r1, cu, N, K, max_seqlen, idx, n, (hipStream_t)stream);
+        if (e != hipSuccess) return hip_fail(e, "top-k launch");
+    }
+    return DSA_OK;
+}
+
+static int check_attn(int T, int N, const int32_t *cu, int Hq, int Hkv, int D, int K, int dtype, const int32_t *idx,
+                      const int32_t *n) {
+    if (int rc = check_packed(T, N, cu)) return rc;
+    if (dtype != DSA_DTYPE_BF16) return fail(DSA_ERR_UNSUPPORTED, "q/k/v must be bf16 (dtype code %d)", dtype);
+    if (Hq < 1 || Hkv < 1 || Hq % Hkv) return fail(DSA_ERR_ARG, "Hq=%d must be a positive multiple of Hkv=%d", Hq, Hkv);
+    if (Hq / Hkv > 16) return fail(DSA_ERR_UNSUPPORTED, "Hq/Hkv=%d: at most 16 query heads per kv head", Hq / Hkv);
+    if (!(D == 64 || D == 128 || D == 256)) return fail(DSA_ERR_UNSUPPORTED, "head_dim=%d: need 64, 128 or 256", D);
+    if ((idx == nullptr) != (n == nullptr)) return fail(DSA_ERR_ARG, "idx and n must both be given or both be null");
+    if (idx && K < 1) return fail(DSA_ERR_ARG, "top_k=%d must be >= 1", K);
+    if ((int64_t)T * Hkv >= ((int64_t)1 << 31)) return fail(DSA_ERR_UNSUPPORTED, "T*Hkv too large for one launch");
+    return DSA_OK;
+}
+
+extern "C" int dsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
+                            const int32_t *cu, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
+                            int dtype, void *out, float *lse, void *stream) {
+    if (int rc = check_attn(T, N, cu, Hq, Hkv, D, K, dtype, idx, n)) return rc;
+    if (!q || !k || !v || !out || !lse) return fail(DSA_ERR_ARG, "null tensor pointer");
+    hipError_t e = dsa_launch_attn_fwd(q, k, v, idx, n, cu, N, T, Hq, Hkv, D, K, softmax_scale, out, lse, (hipStream_t)stream);
+    return e == hipSuccess ? DSA_OK : hip_fail(e, "attention forward launch");
+}
+
+static inline int bitmap_ldw(int max_seqlen) { return (max_seqlen + 31) / 32; }
+
+extern "C" size_t dsa_attn_bwd_workspace_bytes(int T, int Hq, int max_seqlen, int has_idx) {
+    if (T <= 0) return 0;
+    size_t b = align_up((size_t)T * Hq * 4, 256);
+    if (has_idx) b += align_up((size_t)T * bitmap_ldw(max_seqlen) * 4, 256);
+    return b;
+}
+
+extern "C" int dsa_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                            const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu, int T, int N,
+                            int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen, void *dq,
+                            void *dk, void *dv, void *ws, size_t ws_bytes, void *stream) {
+    if (int rc = check_attn(T, N, cu, Hq, Hkv, D, K, dtype, idx, n)) return rc;
+    if (!dout || !q || !k || !v || !out || !lse || !dq || !dk || !dv) return fail(DSA_ERR_ARG, "null tensor pointer");
+    if (max_seqlen < 1 || max_seqlen > (T > 0 ? T : 1)) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
+    if (T == 0) return DSA_OK;
+    const size_t need = dsa_attn_bwd_workspace_bytes(T, Hq, max_seqlen, idx != nullptr);
+    if (!ws || ws_bytes < need) return fail(DSA_ERR_WORKSPACE, "backward workspace: have %zu bytes, need %zu", ws_bytes, need);
+    const int ldw = bitmap_ldw(max_seqlen);
+    if (idx && (size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);
+    float *delta = (float *)ws;
+    uint32_t *bitmap = idx ? (uint32_t *)((char *)ws + align_up((size_t)T * Hq * 4, 256)) : nullptr;
+    hipError_t e = dsa_launch_attn_bwd(dout, q, k, v, out, lse, idx, n, cu, N, T, Hq, Hkv, D, K, softmax_scale, max_seqlen,
+                                       dq, dk, dv, delta, bitmap, ldw, (hipStream_t)stream);
+    return e == hipSuccess ? DSA_OK : hip_fail(e, "attention backward launch");
+}

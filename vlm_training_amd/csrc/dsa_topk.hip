@@ -1,0 +1,138 @@
+// Stage D2: per-query top-k over one row of fp32 scores, total order (score descending, column
+// ascending).  One 256-thread workgroup per query row.
+//
+//   1. rows with pos+1 <= K are the whole causal window: write the range, done;
+//   2. MSB-first radix select (4 passes x 8 bits) over order-preserving uint32 keys finds the K-th
+//      largest key tau and how many keys equal to tau are still wanted (need_eq);
+//   3. an index-ordered compaction keeps key > tau, plus the first need_eq keys == tau.  The row is
+//      split into four contiguous quarters (one per wave); per-quarter counts give every wave its
+//      output offset, so the result comes out ascending and deterministic without sorting.
+//
+// Rows up to TOPK_LDS_CAP keys are read from HBM once and kept in LDS as keys.
+#include "dsa_common.h"
+
+#define TOPK_THREADS 256
+#define TOPK_LDS_CAP 8192
+
+__device__ __forceinline__ uint32_t score_key(float x) {
+    uint32_t u = __float_as_uint(x);
+    if (u == 0x80000000u) u = 0u;                       // -0.0 ties with +0.0
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);  // larger float <=> larger key
+}
+
+template <bool CACHED>
+__global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
+    const float *__restrict__ scores, int64_t ld, int row_begin, const int32_t *__restrict__ cu, int N, int K,
+    int32_t *__restrict__ idx_out, int32_t *__restrict__ n_out) {
+    __shared__ uint32_t hist[256];
+    __shared__ uint32_t wave_tot[4];
+    __shared__ uint32_t sel_digit, sel_remaining;
+    __shared__ uint32_t cnt_gt[4], cnt_eq[4];
+    __shared__ uint32_t keys_lds[CACHED ? TOPK_LDS_CAP : 1];
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int t = row_begin + blockIdx.x;
+    const int seg = find_segment(cu, N, t);
+    const int s0 = cu[seg];
+    const int nvalid = t - s0 + 1;
+    int32_t *orow = idx_out + (int64_t)t * K;
+
+    if (nvalid <= K) {
+        for (int i = tid; i < K; i += TOPK_THREADS) orow[i] = (i < nvalid) ? (s0 + i) : -1;
+        if (tid == 0) n_out[t] = nvalid;
+        return;
+    }
+    const float *row = scores + (int64_t)(t - row_begin) * ld;
+    if (CACHED) {
+        for (int i = tid; i < nvalid; i += TOPK_THREADS) keys_lds[i] = score_key(row[i]);
+    }
+    auto key_at = [&](int i) -> uint32_t { return CACHED ? keys_lds[i] : score_key(row[i]); };
+
+    uint32_t prefix = 0u, pmask = 0u, remaining = (uint32_t)K;
+    for (int pass = 0; pass < 4; ++pass) {
+        const int shift = 24 - 8 * pass;
+        hist[tid] = 0u;
+        __syncthreads();
+        for (int i = tid; i < nvalid; i += TOPK_THREADS) {
+            uint32_t key = key_at(i);
+            if ((key & pmask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+        }
+        __syncthreads();
+        // inclusive suffix sum over the 256 digits (digit 255 first)
+        uint32_t h = hist[tid], v = h;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            uint32_t u = __shfl_down(v, off, 64);
+            if (lane + off < 64) v += u;
+        }
+        if (lane == 0) wave_tot[wv] = v;
+        __syncthreads();
+        for (int w2 = wv + 1; w2 < 4; ++w2) v += wave_tot[w2];
+        const uint32_t excl = v - h;                    // keys with a larger digit
+        if (excl < remaining && remaining <= v) {       // exactly one digit satisfies this
+            sel_digit = (uint32_t)tid;
+            sel_remaining = remaining - excl;
+        }
+        __syncthreads();
+        prefix |= sel_digit << shift;
+        pmask |= 255u << shift;
+        remaining = sel_remaining;
+        __syncthreads();
+    }
+    const uint32_t tau = prefix, need_eq = remaining;
+
+    // contiguous quarter of the row per wave, multiple of 64 columns
+    const int per = (((nvalid + 3) >> 2) + 63) & ~63;
+    const int c_begin = min(wv * per, nvalid), c_end = min(c_begin + per, nvalid);
+    uint32_t g = 0, e = 0;
+    for (int i = c_begin + lane; i < c_end; i += 64) {
+        uint32_t key = key_at(i);
+        g += key > tau;
+        e += key == tau;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        g += __shfl_xor(g, off, 64);
+        e += __shfl_xor(e, off, 64);
+    }
+    if (lane == 0) { cnt_gt[wv] = g; cnt_eq[wv] = e; }
+    __syncthreads();
+    uint32_t eq_seen = 0, out_pos = 0;
+    for (int w2 = 0; w2 < wv; ++w2) {
+        uint32_t eq_take = need_eq > eq_seen ? min(need_eq - eq_seen, cnt_eq[w2]) : 0u;
+        out_pos += cnt_gt[w2] + eq_take;
+        eq_seen += cnt_eq[w2];
+    }
+    const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    for (int i0 = c_begin; i0 < c_end; i0 += 64) {
+        const int i = i0 + lane;
+        bool is_gt = false, is_eq = false;
+        if (i < c_end) {
+            uint32_t key = key_at(i);
+            is_gt = key > tau;
+            is_eq = key == tau;
+        }
+        const uint64_t b_eq = __ballot(is_eq);
+        const uint32_t eq_rank = eq_seen + (uint32_t)__popcll(b_eq & lt_mask);
+        const bool take = is_gt || (is_eq && eq_rank < need_eq);
+        const uint64_t b_take = __ballot(take);
+        if (take) orow[out_pos + (uint32_t)__popcll(b_take & lt_mask)] = s0 + i;
+        out_pos += (uint32_t)__popcll(b_take);
+        eq_seen += (uint32_t)__popcll(b_eq);
+    }
+    if (tid == 0) n_out[t] = K;
+}
+
+extern "C" hipError_t dsa_launch_topk(const float *scores, int64_t ld, int row_begin, int row_end,
+                                      const int32_t *cu, int N, int K, int max_row, int32_t *idx, int32_t *n,
+                                      hipStream_t stream) {
+    const int rows = row_end - row_begin;
+    if (rows <= 0) return hipSuccess;
+    if (max_row <= TOPK_LDS_CAP)
+        hipLaunchKernelGGL(dsa_topk_rows_kernel<true>, dim3(rows), dim3(TOPK_THREADS), 0, stream, scores, ld,
+                           row_begin, cu, N, K, idx, n);
+    else
+        hipLaunchKernelGGL(dsa_topk_rows_kernel<false>, dim3(rows), dim3(TOPK_THREADS), 0, stream, scores, ld,
+                           row_begin, cu, N, K, idx, n);
+    return hipGetLastError();
+}

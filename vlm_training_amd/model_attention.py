@@ -1,0 +1,78 @@
+"""Drop-in entry points with the reference's own names and signatures.
+
+* ``varlen_attention_forward(query, key, value, attention_mask)`` - train/model_attention.py:97-143
+  (HF layout ``(1,H,T,D)``; ``attention_mask`` carries the 1-D ``cu_seqlens``; returns
+  ``((1,T,Hq,D), None)``).
+* ``dispatch_varlen_attention(q, k, v, cu_seqlens, max_seqlen, causal=True)`` -
+  models/qwen3_vl/model.py:25-46 (``(T,H,D)`` in and out).
+* ``varlen_attn(q, k, v, cu_seq_q, cu_seq_k, max_q, max_k, ...)`` - the torch routine both call
+  (torch 2.11 ``window_size=(-1, 0)`` form used by the reference, torch 2.10 ``is_causal=`` form).
+* ``run_varlen_attn`` - models/qwen3_5/model.py:90-98 (``SelfAttention._run_varlen_attn``).
+
+All of them take the DSA extension as keyword-only arguments (default off = reference behaviour).
+"""
+from __future__ import annotations
+
+import torch
+
+from .ops import dsa_varlen_attn
+
+_DSA_KEYS = ("indexer_q", "indexer_k", "indexer_w", "top_k", "index_scale", "return_indices")
+
+
+def varlen_attn(query, key, value, cu_seq_q, cu_seq_k, max_q, max_k, is_causal=None, return_aux=None,
+                scale=None, window_size=None, **dsa):
+    unknown = set(dsa) - set(_DSA_KEYS)
+    if unknown:
+        raise TypeError(f"unexpected arguments {sorted(unknown)}")
+    if cu_seq_q is not cu_seq_k and not torch.equal(cu_seq_q, cu_seq_k):
+        raise ValueError("self-attention only: cu_seq_q and cu_seq_k must agree")
+    if max_q != max_k:
+        raise ValueError("self-attention only: max_q and max_k must agree")
+    if window_size is not None:
+        left, right = window_size
+        if left != -1 or right not in (0, -1):
+            raise NotImplementedError("sliding windows are not part of this operator")
+        causal = right == 0
+    else:
+        causal = True if is_causal is None else bool(is_causal)
+    if not causal:
+        raise NotImplementedError("non-causal (vision tower) packed attention is not built yet")
+    if return_aux is not None:
+        raise NotImplementedError("return_aux is not supported")
+    return dsa_varlen_attn(query, key, value, cu_seq_q, int(max_q), softmax_scale=scale, **dsa)
+
+
+def dispatch_varlen_attention(q, k, v, cu_seqlens, max_seqlen, causal: bool = True, **dsa):
+    return varlen_attn(q, k, v, cu_seq_q=cu_seqlens, cu_seq_k=cu_seqlens, max_q=max_seqlen, max_k=max_seqlen,
+                       window_size=(-1, 0) if causal else (-1, -1), **dsa)  # (total, num_heads, head_dim)
+
+
+@torch.compiler.disable
+def run_varlen_attn(q, k, v, cu_seqlens, max_seqlen, **dsa):
+    return varlen_attn(q, k, v, cu_seq_q=cu_seqlens, cu_seq_k=cu_seqlens, max_q=max_seqlen, max_k=max_seqlen,
+                       window_size=(-1, 0), **dsa)
+
+
+def _hf_indexer_to_packed(x):
+    # accepts packed (T,...) tensors as they are, or HF-style tensors with a leading batch dim of 1
+    return x if x is None or x.dim() < 3 or x.shape[0] != 1 else x.squeeze(0)
+
+
+def varlen_attention_forward(query, key, value, attention_mask, **dsa):
+    """(1,Hq,T,D),(1,Hkv,T,D),(1,Hkv,T,D), cu_seqlens -> ((1,T,Hq,D), None)."""
+    # batch, head, seq_len, dim -> batch, seq_len, head, dim -> (T, head, dim)
+    query = query.transpose(1, 2).contiguous()
+    key = key.transpose(1, 2).contiguous()
+    value = value.transpose(1, 2).contiguous()
+    query = query.view(-1, query.size(-2), query.size(-1))
+    key = key.view(-1, key.size(-2), key.size(-1))
+    value = value.view(-1, value.size(-2), value.size(-1))
+    cu_seqlens = attention_mask.squeeze()
+    with torch.no_grad():
+        max_seqlen = torch.diff(cu_seqlens).max().item()
+    attn_output = varlen_attn(query, key, value, cu_seq_q=cu_seqlens, cu_seq_k=cu_seqlens, max_q=max_seqlen,
+                              max_k=max_seqlen, window_size=(-1, 0), **dsa)
+    if isinstance(attn_output, tuple):
+        return (attn_output[0].unsqueeze(0), None) + tuple(attn_output[1:])
+    return attn_output.unsqueeze(0), None

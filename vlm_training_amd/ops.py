@@ -1,0 +1,203 @@
+"""Host side of the DSA packed-attention operator: torch tensors in, HIP kernels through the C ABI.
+
+``dsa_varlen_attn`` is the operator (a ``torch.autograd.Function`` underneath).  With no indexer
+inputs it is dense causal varlen attention, i.e. what the reference gets from
+``varlen_attn(q, k, v, cu_seq_q=cu, cu_seq_k=cu, max_q=m, max_k=m, window_size=(-1, 0))``
+(train/model_attention.py:123-132, models/qwen3_vl/model.py:41-46, models/qwen3_5/model.py:93-98).
+torch is used for device memory and streams only; all arithmetic runs in the HIP library.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("dsa attention runs on the GPU only (tensor on %s); there is no CPU path" % t.device)
+
+
+def _as_bf16(t: torch.Tensor) -> torch.Tensor:
+    # fp32/fp16 inputs are rounded to bf16 once; the kernels compute in bf16 MFMA with fp32 accumulation
+    return (t if t.dtype == torch.bfloat16 else t.to(torch.bfloat16)).contiguous()
+
+
+def _check_cu(cu_seqlens: torch.Tensor, T: int):
+    if cu_seqlens.dim() != 1 or cu_seqlens.numel() < 2:
+        raise ValueError("cu_seqlens must be 1-D with at least two entries")
+    if cu_seqlens.dtype != torch.int32:
+        cu_seqlens = cu_seqlens.to(torch.int32)
+    return cu_seqlens.contiguous()
+
+
+def _check_qkv(q, k, v):
+    if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
+        raise ValueError("q, k, v must be (T, H, D)")
+    T, Hq, D = q.shape
+    if k.shape != v.shape or k.shape[0] != T or k.shape[2] != D:
+        raise ValueError(f"q/k/v shapes disagree: {tuple(q.shape)} {tuple(k.shape)} {tuple(v.shape)}")
+    Hkv = k.shape[1]
+    if Hq % Hkv:
+        raise ValueError(f"Hq={Hq} must be a multiple of Hkv={Hkv}")
+    if q.dtype != k.dtype or q.dtype != v.dtype:
+        raise ValueError("q, k, v must share a dtype")
+    return T, Hq, Hkv, D
+
+
+# ------------------------------------------------------------------------------------------------
+# stage wrappers (also used by the tests to look at each stage on its own)
+# ------------------------------------------------------------------------------------------------
+def indexer_scores(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen: int, index_scale: Optional[float] = None,
+                   skip_dense_k: int = 0) -> torch.Tensor:
+    """Stage D1 for every row: (T, ld) fp32, row t valid on columns [0, pos(t)] (key = seg_start + column)."""
+    _require_cuda(q_idx, k_idx, w_idx, cu_seqlens)
+    T, Hi, Di = q_idx.shape
+    cu = _check_cu(cu_seqlens, T)
+    scale = index_scale if index_scale is not None else (Di ** -0.5) * (Hi ** -0.5)
+    ld = (max_seqlen + 31) // 32 * 32
+    scores = torch.full((T, ld), float("-inf"), dtype=torch.float32, device=q_idx.device)
+    lib = _lib.load()
+    rc = lib.dsa_indexer_scores(_ptr(_as_bf16(q_idx)), _ptr(_as_bf16(k_idx)), _ptr(_as_bf16(w_idx)), _ptr(cu), T,
+                                cu.numel() - 1, Hi, Di, scale, _lib.DSA_DTYPE_BF16, 0, T, skip_dense_k, _ptr(scores), ld,
+                                _stream(q_idx.device))
+    _lib.check(rc, "dsa_indexer_scores")
+    return scores
+
+
+def topk_from_scores(scores: torch.Tensor, cu_seqlens, top_k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Stage D2 on materialised scores (T, ld): returns (idx (T,K) int32, n (T,) int32)."""
+    _require_cuda(scores, cu_seqlens)
+    if scores.dtype != torch.float32 or scores.dim() != 2 or not scores.is_contiguous():
+        raise ValueError("scores must be a contiguous (T, ld) fp32 tensor")
+    T, ld = scores.shape
+    cu = _check_cu(cu_seqlens, T)
+    idx = torch.empty((T, top_k), dtype=torch.int32, device=scores.device)
+    n = torch.empty((T,), dtype=torch.int32, device=scores.device)
+    lib = _lib.load()
+    rc = lib.dsa_topk_from_scores(_ptr(scores), ld, 0, T, _ptr(cu), T, cu.numel() - 1, top_k, _ptr(idx), _ptr(n),
+                                  _stream(scores.device))
+    _lib.check(rc, "dsa_topk_from_scores")
+    return idx, n
+
+
+def index_topk(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen: int, top_k: int,
+               index_scale: Optional[float] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Stages D1+D2: selected key rows per query, (idx (T,K) int32 ascending/-1 padded, n (T,) int32)."""
+    _require_cuda(q_idx, k_idx, w_idx, cu_seqlens)
+    if q_idx.dim() != 3 or k_idx.dim() != 2 or w_idx.dim() != 2:
+        raise ValueError("indexer tensors must be q_idx (T,Hi,Di), k_idx (T,Di), w_idx (T,Hi)")
+    T, Hi, Di = q_idx.shape
+    if k_idx.shape != (T, Di) or w_idx.shape != (T, Hi):
+        raise ValueError("indexer tensor shapes disagree")
+    if top_k < 1:
+        raise ValueError("top_k must be >= 1")
+    cu = _check_cu(cu_seqlens, T)
+    scale = index_scale if index_scale is not None else (Di ** -0.5) * (Hi ** -0.5)
+    lib = _lib.load()
+    idx = torch.empty((T, top_k), dtype=torch.int32, device=q_idx.device)
+    n = torch.empty((T,), dtype=torch.int32, device=q_idx.device)
+    ws_bytes = lib.dsa_index_topk_workspace_bytes(T, max_seqlen, top_k) if max_seqlen > top_k else 0
+    ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q_idx.device)
+    rc = lib.dsa_index_topk(_ptr(_as_bf16(q_idx)), _ptr(_as_bf16(k_idx)), _ptr(_as_bf16(w_idx)), _ptr(cu), T,
+                            cu.numel() - 1, Hi, Di, top_k, scale, _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(idx), _ptr(n),
+                            _ptr(ws), ws_bytes, _stream(q_idx.device))
+    _lib.check(rc, "dsa_index_topk")
+    return idx, n
+
+
+def attn_fwd(q, k, v, idx, n, cu_seqlens, softmax_scale: float):
+    T, Hq, Hkv, D = _check_qkv(q, k, v)
+    cu = _check_cu(cu_seqlens, T)
+    out = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=q.device)
+    lse = torch.empty((Hq, T), dtype=torch.float32, device=q.device)
+    K = idx.shape[1] if idx is not None else 0
+    lib = _lib.load()
+    rc = lib.dsa_attn_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(idx), _ptr(n), _ptr(cu), T, cu.numel() - 1, Hq, Hkv, D, K,
+                          softmax_scale, _lib.DSA_DTYPE_BF16, _ptr(out), _ptr(lse), _stream(q.device))
+    _lib.check(rc, "dsa_attn_fwd")
+    return out, lse
+
+
+def attn_bwd(dout, q, k, v, out, lse, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float):
+    T, Hq, Hkv, D = _check_qkv(q, k, v)
+    cu = _check_cu(cu_seqlens, T)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    K = idx.shape[1] if idx is not None else 0
+    lib = _lib.load()
+    ws_bytes = lib.dsa_attn_bwd_workspace_bytes(T, Hq, max_seqlen, 1 if idx is not None else 0)
+    ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q.device)
+    rc = lib.dsa_attn_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(idx), _ptr(n), _ptr(cu), T,
+                          cu.numel() - 1, Hq, Hkv, D, K, softmax_scale, _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(dq),
+                          _ptr(dk), _ptr(dv), _ptr(ws), ws_bytes, _stream(q.device))
+    _lib.check(rc, "dsa_attn_bwd")
+    return dq, dk, dv
+
+
+# ------------------------------------------------------------------------------------------------
+# the operator
+# ------------------------------------------------------------------------------------------------
+class _DsaVarlenAttn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, cu_seqlens, max_seqlen, idx, n, softmax_scale):
+        in_dtype = q.dtype
+        qb, kb, vb = _as_bf16(q), _as_bf16(k), _as_bf16(v)
+        out, lse = attn_fwd(qb, kb, vb, idx, n, cu_seqlens, softmax_scale)
+        ctx.save_for_backward(qb, kb, vb, out, lse, cu_seqlens, *(() if idx is None else (idx, n)))
+        ctx.has_idx = idx is not None
+        ctx.max_seqlen = int(max_seqlen)
+        ctx.softmax_scale = softmax_scale
+        ctx.in_dtype = in_dtype
+        return out if in_dtype == torch.bfloat16 else out.to(in_dtype)
+
+    @staticmethod
+    def backward(ctx, dout):
+        saved = ctx.saved_tensors
+        qb, kb, vb, out, lse, cu = saved[:6]
+        idx, n = (saved[6], saved[7]) if ctx.has_idx else (None, None)
+        dq, dk, dv = attn_bwd(_as_bf16(dout), qb, kb, vb, out, lse, idx, n, cu, ctx.max_seqlen, ctx.softmax_scale)
+        if ctx.in_dtype != torch.bfloat16:
+            dq, dk, dv = dq.to(ctx.in_dtype), dk.to(ctx.in_dtype), dv.to(ctx.in_dtype)
+        return dq, dk, dv, None, None, None, None, None
+
+
+def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: int, *, indexer_q=None, indexer_k=None, indexer_w=None,
+                    top_k: Optional[int] = None, index_scale: Optional[float] = None,
+                    softmax_scale: Optional[float] = None, return_indices: bool = False):
+    """Packed causal attention over ``cu_seqlens`` segments, optionally sparsified by the DSA indexer.
+
+    q (T,Hq,D), k/v (T,Hkv,D) contiguous, cu_seqlens (N+1,) int32 on the device, max_seqlen host int
+    (the reference's callers already hold it: models/qwen3_vl/model.py:765).  Without indexer inputs
+    every causal key of the token's own segment is attended (the reference's behaviour).  With
+    ``indexer_q (T,Hi,Di)``, ``indexer_k (T,Di)``, ``indexer_w (T,Hi)`` and ``top_k`` each query keeps
+    the top_k keys of its causal window under (indexer score descending, key index ascending).
+    Gradients flow to q, k, v only.
+    """
+    _require_cuda(q, k, v, cu_seqlens)
+    T, Hq, Hkv, D = _check_qkv(q, k, v)
+    cu = _check_cu(cu_seqlens, T)
+    scale = float(softmax_scale) if softmax_scale is not None else D ** -0.5
+    sparse = indexer_q is not None or indexer_k is not None or indexer_w is not None
+    idx = n = None
+    if sparse:
+        if indexer_q is None or indexer_k is None or indexer_w is None or top_k is None:
+            raise ValueError("DSA needs indexer_q, indexer_k, indexer_w and top_k together")
+        if indexer_q.shape[0] != T:
+            raise ValueError("indexer tensors must cover the same T packed tokens as q")
+        with torch.no_grad():
+            idx, n = index_topk(indexer_q, indexer_k, indexer_w, cu, int(max_seqlen), int(top_k), index_scale)
+    elif return_indices:
+        raise ValueError("return_indices needs the indexer inputs")
+    out = _DsaVarlenAttn.apply(q.contiguous(), k.contiguous(), v.contiguous(), cu, int(max_seqlen), idx, n, scale)
+    return (out, idx, n) if return_indices else out

@@ -1,0 +1,126 @@
+"""Synthetic packed batches for the five measurement configurations.
+
+Everything is produced from ``torch.Generator(device='cpu').manual_seed(seed)`` in fp32 and then
+cast, so the same call yields the same batch on any machine.  Segment lengths are literals.
+The packing convention is the reference's: int32 ``cu_seqlens`` prefix sums with the pad tail as
+one more segment (data/energon_dataloader.py:431-464, models/qwen3_vl/model.py:757-765).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class Workload:
+    name: str
+    dtype: torch.dtype
+    seg_lens: Tuple[int, ...]
+    Hq: int
+    Hkv: int
+    D: int
+    Hi: int
+    Di: int
+    top_k: int
+    sigma: float
+    seed: int
+    image_runs: bool = False
+
+    @property
+    def T(self) -> int:
+        return sum(self.seg_lens)
+
+    @property
+    def cu(self) -> List[int]:
+        out = [0]
+        for L in self.seg_lens:
+            out.append(out[-1] + L)
+        return out
+
+    @property
+    def max_seqlen(self) -> int:
+        return max(self.seg_lens)
+
+    def pair_counts(self) -> Tuple[int, int]:
+        """(P, S): causal pairs and selected pairs."""
+        P = S = 0
+        for L in self.seg_lens:
+            P += L * (L + 1) // 2
+            d = min(L, self.top_k)
+            S += d * (d + 1) // 2 + max(0, L - self.top_k) * self.top_k
+        return P, S
+
+    def work(self) -> Dict[str, float]:
+        """Algorithmic flop / byte counts per fwd+bwd pass (bf16 element = 2 bytes)."""
+        P, S = self.pair_counts()
+        e = 2 if self.dtype == torch.bfloat16 else 4
+        T, Hq, Hkv, D, Hi, Di, K = self.T, self.Hq, self.Hkv, self.D, self.Hi, self.Di, self.top_k
+        F1 = P * (2 * Hi * Di + 2 * Hi)
+        B2 = 4 * T * K
+        F3 = 4 * Hq * D * S
+        B3g = S * Hkv * 2 * D * e
+        B3 = B3g + T * 2 * Hq * D * e
+        F4 = 10 * Hq * D * S
+        B4 = 2 * B3g + T * (3 * Hq + 2 * Hkv) * D * e + 8 * S
+        return dict(P=P, S=S, F1=F1, B2=B2, F3=F3, B3_gather=B3g, B3=B3, F4=F4, B4=B4)
+
+
+C1 = Workload("C1-toy", torch.float32, (256, 512, 384, 896), 8, 2, 64, 4, 32, 128, 1.0, 1)
+C2 = Workload("C2-qwen3vl-2b", torch.bfloat16, (1799, 914, 680, 970, 1148, 1763, 918),
+              16, 8, 128, 32, 64, 1024, 0.5, 2)
+C3 = Workload("C3-qwen3vl-8b-32k", torch.bfloat16, (6144, 2048, 5120, 3072, 4096, 7168, 1024, 4096),
+              32, 8, 128, 64, 128, 2048, 0.5, 3, image_runs=True)
+C4 = Workload("C4-long-131k", torch.bfloat16, (131072,), 32, 8, 128, 64, 128, 2048, 0.5, 4)
+C5 = Workload("C5-qwen3.5-short-segments", torch.bfloat16,
+              (716, 65, 73, 107, 133, 129, 75, 135, 512, 1379, 214, 227, 270, 675, 972, 1669, 234, 740,
+               208, 1112, 141, 1309, 367, 789, 407, 190, 354, 76, 74, 400, 333, 1147, 1152),
+              16, 2, 256, 32, 128, 512, 0.5, 5)
+
+WORKLOADS = {w.name.split("-")[0]: w for w in (C1, C2, C3, C4, C5)}
+
+
+def scaled(w: Workload, seg_lens, top_k=None, name=None) -> Workload:
+    """Same head geometry on other segment lengths (parity tests at sizes the CPU finishes)."""
+    return Workload(name or (w.name + "-scaled"), w.dtype, tuple(seg_lens), w.Hq, w.Hkv, w.D, w.Hi, w.Di,
+                    top_k if top_k is not None else w.top_k, w.sigma, w.seed, w.image_runs)
+
+
+def make_inputs(w: Workload, device="cpu", with_dout: bool = True):
+    """Returns dict(q,k,v,q_idx,k_idx,w_idx,dout,cu_seqlens,max_seqlen) on ``device``."""
+    g = torch.Generator(device="cpu").manual_seed(w.seed)
+    T = w.T
+
+    def normal(*shape, sigma):
+        return torch.randn(*shape, generator=g, dtype=torch.float32) * sigma
+
+    t = dict(
+        q=normal(T, w.Hq, w.D, sigma=w.sigma),
+        k=normal(T, w.Hkv, w.D, sigma=w.sigma),
+        v=normal(T, w.Hkv, w.D, sigma=w.sigma),
+        q_idx=normal(T, w.Hi, w.Di, sigma=w.sigma),
+        k_idx=normal(T, w.Di, sigma=w.sigma),
+        w_idx=normal(T, w.Hi, sigma=w.sigma),
+    )
+    if w.image_runs:
+        # image-patch runs: rows share one mean vector per run -> clustered top-k
+        a = 0
+        for L in w.seg_lens:
+            runs = []
+            if L >= 2048:
+                runs.append((16, 16 + 1024))
+            if L >= 4096:
+                runs.append((2048, 3072))
+            for r0, r1 in runs:
+                for name in ("q", "k", "v", "q_idx", "k_idx", "w_idx"):
+                    x = t[name]
+                    m = torch.randn(*x.shape[1:], generator=g, dtype=torch.float32)
+                    x[a + r0:a + r1] = x[a + r0:a + r1] + 0.5 * m
+            a += L
+    if with_dout:
+        t["dout"] = normal(T, w.Hq, w.D, sigma=1.0)
+    out = {name: x.to(w.dtype).to(device) for name, x in t.items()}
+    out["cu_seqlens"] = torch.tensor(w.cu, dtype=torch.int32, device=device)
+    out["max_seqlen"] = w.max_seqlen
+    return out
