@@ -1,0 +1,164 @@
+#!/usr/bin/env python3
+"""Benchmark of the DSA packed-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--no-cpu-baseline]
+
+A step is one forward + backward pass of the whole operator (indexer scores -> top-k -> sparse
+attention forward -> sparse attention backward) over one synthetic packed batch that is already
+resident in HBM.  Prints ONE JSON line: whole-operator tokens/s, the roofline figures of the
+dominant kernel measured live with events on the launch stream, the per-stage times, and the CPU
+oracle timed on a bounded sample of the same workload on this box's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
+PEAK_MFMA_BF16_TFLOPS = 2500.0
+
+
+def timed(fn, iters, warmup=1):
+    """Average milliseconds of fn() measured with events on torch's current stream (the launch stream)."""
+    for _ in range(warmup):
+        fn()
+    beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    beg.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return beg.elapsed_time(end) / iters
+
+
+def cpu_baseline(w, threads):
+    """Oracle (fp32 torch, CPU) fwd+bwd on one segment of the workload, scaled by causal pairs."""
+    from oracle import dsa_ref as R
+    from vlm_training_amd import workloads as W
+    # sample: the shortest segment that is longer than top_k (has both dense and sparse rows)
+    cands = [L for L in w.seg_lens if L > w.top_k] or [max(w.seg_lens)]
+    L = min(min(cands), 3072)
+    sw = W.scaled(w, (L,), name=w.name + "-cpu-sample")
+    t = W.make_inputs(sw, device="cpu")
+    torch.set_num_threads(threads)
+    t0 = time.perf_counter()
+    idx, n = R.dsa_select(t["q_idx"], t["k_idx"], t["w_idx"], sw.cu, sw.top_k)
+    R.sparse_attention_grads(t["q"], t["k"], t["v"], idx, n, sw.cu, t["dout"])
+    dt = time.perf_counter() - t0
+    P_s, _ = sw.pair_counts()
+    P, _ = w.pair_counts()
+    est_total = dt * P / P_s            # the oracle's cost is proportional to causal pairs
+    return {
+        "value": w.T / est_total, "unit": "tokens/s", "cores": threads, "kind": "port",
+        "sample": f"oracle fwd+bwd on one {L}-token segment of {w.name} ({P_s} of {P} causal pairs) took {dt:.2f} s; "
+                  f"scaled by causal pairs to the whole batch",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="C3")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    from vlm_training_amd import ops, workloads as W
+    w = W.WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    t = W.make_inputs(w, device=dev)
+    cu, msl = t["cu_seqlens"], w.max_seqlen
+    q = t["q"].requires_grad_(True)
+    k = t["k"].requires_grad_(True)
+    v = t["v"].requires_grad_(True)
+    scale = w.D ** -0.5
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        out = ops.dsa_varlen_attn(q, k, v, cu, msl, indexer_q=t["q_idx"], indexer_k=t["k_idx"], indexer_w=t["w_idx"],
+                                  top_k=w.top_k)
+        out.backward(t["dout"])
+
+    # ---- the metric: whole-operator fwd+bwd --------------------------------------------------
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    wall0 = time.perf_counter()
+    beg.record()
+    for _ in range(args.steps):
+        step()
+    end.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - wall0) * 1e3 / args.steps
+    ms_per_step = max(beg.elapsed_time(end) / args.steps, wall_ms)
+    tokens_per_s = w.T / (ms_per_step * 1e-3)
+
+    # ---- per-stage times (each kernel alone, same stream) ------------------------------------
+    it = max(2, min(args.steps, 5))
+    with torch.no_grad():
+        qd, kd, vd = q.detach(), k.detach(), v.detach()
+        idx, n = ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k)
+        out, lse = ops.attn_fwd(qd, kd, vd, idx, n, cu, scale)
+        bufs = ops.attn_bwd(t["dout"], qd, kd, vd, out, lse, idx, n, cu, msl, scale, 15,
+                            (torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd),
+                             torch.empty((ops._lib.load().dsa_attn_bwd_workspace_bytes(w.T, w.Hq, msl, 1),),
+                                         dtype=torch.uint8, device=dev)))
+        stage_ms = {
+            "index_topk": timed(lambda: ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k), it),
+            "attn_fwd": timed(lambda: ops.attn_fwd(qd, kd, vd, idx, n, cu, scale), it),
+        }
+        for name, part in (("bwd_delta", 1), ("bwd_bitmap", 2), ("bwd_dq", 4), ("bwd_dkv", 8)):
+            stage_ms[name] = timed(lambda: ops.attn_bwd(t["dout"], qd, kd, vd, out, lse, idx, n, cu, msl, scale, part, bufs), it)
+
+    # ---- roofline ----------------------------------------------------------------------------
+    wk = w.work()
+    e = 2
+    qo_bytes = w.T * 2 * w.Hq * w.D * e
+    kern = {   # algorithmic bytes per launch of the gather kernels (HBM-bound rows of the plan)
+        "attn_fwd": wk["B3_gather"] + qo_bytes,                                     # K,V rows + q in + o out
+        "bwd_dq": wk["B3_gather"] + w.T * 3 * w.Hq * w.D * e,                       # K,V rows + q,dO in + dq out
+    }
+    dom = max(kern, key=lambda name: stage_ms[name])
+    achieved = kern[dom] / (stage_ms[dom] * 1e-3) / 1e9
+    t_roof_ms = {
+        "index_topk": max(wk["F1"] / (PEAK_MFMA_BF16_TFLOPS * 1e12), wk["B2"] / (PEAK_HBM_GBS * 1e9)) * 1e3,
+        "attn_fwd": max(wk["F3"] / (PEAK_MFMA_BF16_TFLOPS * 1e12), wk["B3"] / (PEAK_HBM_GBS * 1e9)) * 1e3,
+        "attn_bwd": max(wk["F4"] / (PEAK_MFMA_BF16_TFLOPS * 1e12), wk["B4"] / (PEAK_HBM_GBS * 1e9)) * 1e3,
+    }
+    roof_total = sum(t_roof_ms.values())
+    result = {
+        "metric": "DSA attn fwd+bwd packed tokens/s on 1 GPU at 32K; % MFMA/HBM roofline",
+        "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{w.name}: T={w.T} packed tokens, segments={list(w.seg_lens)}, Hq/Hkv/D={w.Hq}/{w.Hkv}/{w.D}, "
+                               f"indexer {w.Hi}x{w.Di}, top_k={w.top_k}, fwd+bwd"},
+        "roofline": {"bound": "hbm", "kernel": "dsa_attn_fwd_kernel" if dom == "attn_fwd" else "dsa_bwd_dq_kernel",
+                     "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS,
+                     "traffic": None, "algorithmic_bytes": kern[dom], "avg_ms": stage_ms[dom]},
+        "stage_ms": stage_ms,
+        "roofline_whole_op": {"t_roof_ms": t_roof_ms, "sum_ms": roof_total, "frac": roof_total / ms_per_step,
+                              "compute_only_bound_ms": (wk["F1"] + 3.5 * wk["F3"]) / (PEAK_MFMA_BF16_TFLOPS * 1e12) * 1e3},
+        "device": torch.cuda.get_device_name(0),
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(w, torch.get_num_threads())
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -98,6 +98,22 @@ int dsa_attn_bwd(const void *dout, const void *q, const void *k, const void *v, 
                  int D, int K, float softmax_scale, int dtype, int max_seqlen, void *dq, void *dk, void *dv,
                  void *ws, size_t ws_bytes, void *stream);
 
+/*
+ * Measurement hook: dsa_attn_bwd restricted to the kernels named in `parts`, so that each can be
+ * timed on its own with events on the caller's stream.  Parts must be run in bit order at least once
+ * on the same workspace before a later part is timed alone (the later kernels read what the earlier
+ * ones leave in ws).  No reference counterpart.
+ */
+#define DSA_BWD_DELTA 1  /* delta = rowsum(dO * O) */
+#define DSA_BWD_BITMAP 2 /* inverted selection bitmap (only when idx != NULL) */
+#define DSA_BWD_DQ 4     /* query-side gather pass */
+#define DSA_BWD_DKV 8    /* key-side pass */
+#define DSA_BWD_ALL 15
+int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                       const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu_seqlens, int T, int N,
+                       int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen, void *dq, void *dk,
+                       void *dv, void *ws, size_t ws_bytes, int parts, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

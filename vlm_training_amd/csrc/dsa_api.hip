@@ -18,7 +18,7 @@ hipError_t dsa_launch_attn_fwd(const void *q, const void *k, const void *v, cons
 hipError_t dsa_launch_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
                                const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu, int N, int T,
                                int Hq, int Hkv, int D, int K, float scale, int max_seqlen, void *dq, void *dk,
-                               void *dv, float *delta, uint32_t *bitmap, int ldw, hipStream_t stream);
+                               void *dv, float *delta, uint32_t *bitmap, int ldw, int parts, hipStream_t stream);
 }
 
 static thread_local char g_err[512] = "";
@@ -138,10 +138,10 @@ extern "C" size_t dsa_attn_bwd_workspace_bytes(int T, int Hq, int max_seqlen, in
     return b;
 }
 
-extern "C" int dsa_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
-                            const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu, int T, int N,
-                            int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen, void *dq,
-                            void *dk, void *dv, void *ws, size_t ws_bytes, void *stream) {
+extern "C" int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                                  const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu, int T,
+                                  int N, int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen,
+                                  void *dq, void *dk, void *dv, void *ws, size_t ws_bytes, int parts, void *stream) {
     if (int rc = check_attn(T, N, cu, Hq, Hkv, D, K, dtype, idx, n)) return rc;
     if (!dout || !q || !k || !v || !out || !lse || !dq || !dk || !dv) return fail(DSA_ERR_ARG, "null tensor pointer");
     if (max_seqlen < 1 || max_seqlen > (T > 0 ? T : 1)) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
@@ -153,6 +153,14 @@ extern "C" int dsa_attn_bwd(const void *dout, const void *q, const void *k, cons
     float *delta = (float *)ws;
     uint32_t *bitmap = idx ? (uint32_t *)((char *)ws + align_up((size_t)T * Hq * 4, 256)) : nullptr;
     hipError_t e = dsa_launch_attn_bwd(dout, q, k, v, out, lse, idx, n, cu, N, T, Hq, Hkv, D, K, softmax_scale, max_seqlen,
-                                       dq, dk, dv, delta, bitmap, ldw, (hipStream_t)stream);
+                                       dq, dk, dv, delta, bitmap, ldw, parts, (hipStream_t)stream);
     return e == hipSuccess ? DSA_OK : hip_fail(e, "attention backward launch");
+}
+
+extern "C" int dsa_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                            const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu, int T, int N,
+                            int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen, void *dq,
+                            void *dk, void *dv, void *ws, size_t ws_bytes, void *stream) {
+    return dsa_attn_bwd_parts(dout, q, k, v, out, lse, idx, n, cu, T, N, Hq, Hkv, D, K, softmax_scale, dtype, max_seqlen,
+                              dq, dk, dv, ws, ws_bytes, DSA_BWD_ALL, stream);
 }

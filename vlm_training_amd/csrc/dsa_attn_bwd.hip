@@ -361,10 +361,11 @@ template <int D>
 static hipError_t launch_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
                              const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu, int N, int T,
                              int Hq, int Hkv, int K, float scale, int max_seqlen, void *dq, void *dk, void *dv,
-                             float *delta, uint32_t *bitmap, int ldw, hipStream_t stream) {
+                             float *delta, uint32_t *bitmap, int ldw, int parts, hipStream_t stream) {
     const int64_t rows = (int64_t)T * Hq;
-    hipLaunchKernelGGL(dsa_bwd_delta_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, stream,
-                       (const bf16_t *)dout, (const bf16_t *)out, T, Hq, D, delta);
+    if (parts & 1)
+        hipLaunchKernelGGL(dsa_bwd_delta_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, stream,
+                           (const bf16_t *)dout, (const bf16_t *)out, T, Hq, D, delta);
     const dim3 gq((unsigned)((int64_t)T * Hkv));
     const int G = Hq / Hkv;
     int gshift = 0;
@@ -372,21 +373,26 @@ static hipError_t launch_bwd(const void *dout, const void *q, const void *k, con
     const int Gp = 1 << gshift;
     const dim3 gk((unsigned)(((int64_t)T / 64 + N + 1) * Hkv));
     if (idx) {
-        hipLaunchKernelGGL(dsa_bwd_bitmap_kernel, dim3(T), dim3(256), (size_t)ldw * 4, stream, idx, n, cu, N, K, ldw,
-                           bitmap);
-        hipLaunchKernelGGL((dsa_bwd_dq_kernel<D, true>), gq, dim3(64), 0, stream, (const bf16_t *)dout,
-                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, idx, n, cu, N, T, Hq,
-                           Hkv, K, scale, (bf16_t *)dq);
-        hipLaunchKernelGGL((dsa_bwd_dkv_kernel<D, true>), gk, dim3(256), 0, stream, (const bf16_t *)dout,
-                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T,
-                           Hq, Hkv, Gp, gshift, scale, (bf16_t *)dk, (bf16_t *)dv);
+        if (parts & 2)
+            hipLaunchKernelGGL(dsa_bwd_bitmap_kernel, dim3(T), dim3(256), (size_t)ldw * 4, stream, idx, n, cu, N, K,
+                               ldw, bitmap);
+        if (parts & 4)
+            hipLaunchKernelGGL((dsa_bwd_dq_kernel<D, true>), gq, dim3(64), 0, stream, (const bf16_t *)dout,
+                               (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, idx, n, cu, N, T,
+                               Hq, Hkv, K, scale, (bf16_t *)dq);
+        if (parts & 8)
+            hipLaunchKernelGGL((dsa_bwd_dkv_kernel<D, true>), gk, dim3(256), 0, stream, (const bf16_t *)dout,
+                               (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N,
+                               T, Hq, Hkv, Gp, gshift, scale, (bf16_t *)dk, (bf16_t *)dv);
     } else {
-        hipLaunchKernelGGL((dsa_bwd_dq_kernel<D, false>), gq, dim3(64), 0, stream, (const bf16_t *)dout,
-                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, idx, n, cu, N, T, Hq,
-                           Hkv, K, scale, (bf16_t *)dq);
-        hipLaunchKernelGGL((dsa_bwd_dkv_kernel<D, false>), gk, dim3(256), 0, stream, (const bf16_t *)dout,
-                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T,
-                           Hq, Hkv, Gp, gshift, scale, (bf16_t *)dk, (bf16_t *)dv);
+        if (parts & 4)
+            hipLaunchKernelGGL((dsa_bwd_dq_kernel<D, false>), gq, dim3(64), 0, stream, (const bf16_t *)dout,
+                               (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, idx, n, cu, N, T,
+                               Hq, Hkv, K, scale, (bf16_t *)dq);
+        if (parts & 8)
+            hipLaunchKernelGGL((dsa_bwd_dkv_kernel<D, false>), gk, dim3(256), 0, stream, (const bf16_t *)dout,
+                               (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N,
+                               T, Hq, Hkv, Gp, gshift, scale, (bf16_t *)dk, (bf16_t *)dv);
     }
     return hipGetLastError();
 }
@@ -395,12 +401,12 @@ extern "C" hipError_t dsa_launch_attn_bwd(const void *dout, const void *q, const
                                           const void *out, const float *lse, const int32_t *idx, const int32_t *n,
                                           const int32_t *cu, int N, int T, int Hq, int Hkv, int D, int K, float scale,
                                           int max_seqlen, void *dq, void *dk, void *dv, float *delta,
-                                          uint32_t *bitmap, int ldw, hipStream_t stream) {
+                                          uint32_t *bitmap, int ldw, int parts, hipStream_t stream) {
     if (T == 0) return hipSuccess;
     switch (D) {
-        case 64: return launch_bwd<64>(dout, q, k, v, out, lse, idx, n, cu, N, T, Hq, Hkv, K, scale, max_seqlen, dq, dk, dv, delta, bitmap, ldw, stream);
-        case 128: return launch_bwd<128>(dout, q, k, v, out, lse, idx, n, cu, N, T, Hq, Hkv, K, scale, max_seqlen, dq, dk, dv, delta, bitmap, ldw, stream);
-        case 256: return launch_bwd<256>(dout, q, k, v, out, lse, idx, n, cu, N, T, Hq, Hkv, K, scale, max_seqlen, dq, dk, dv, delta, bitmap, ldw, stream);
+        case 64: return launch_bwd<64>(dout, q, k, v, out, lse, idx, n, cu, N, T, Hq, Hkv, K, scale, max_seqlen, dq, dk, dv, delta, bitmap, ldw, parts, stream);
+        case 128: return launch_bwd<128>(dout, q, k, v, out, lse, idx, n, cu, N, T, Hq, Hkv, K, scale, max_seqlen, dq, dk, dv, delta, bitmap, ldw, parts, stream);
+        case 256: return launch_bwd<256>(dout, q, k, v, out, lse, idx, n, cu, N, T, Hq, Hkv, K, scale, max_seqlen, dq, dk, dv, delta, bitmap, ldw, parts, stream);
         default: return hipErrorInvalidValue;
     }
 }

@@ -69,7 +69,8 @@ def indexer_scores(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen: int, index_scale
     ld = (max_seqlen + 31) // 32 * 32
     scores = torch.full((T, ld), float("-inf"), dtype=torch.float32, device=q_idx.device)
     lib = _lib.load()
-    rc = lib.dsa_indexer_scores(_ptr(_as_bf16(q_idx)), _ptr(_as_bf16(k_idx)), _ptr(_as_bf16(w_idx)), _ptr(cu), T,
+    qi, ki, wi = _as_bf16(q_idx), _as_bf16(k_idx), _as_bf16(w_idx)     # keep the casts alive over the launch
+    rc = lib.dsa_indexer_scores(_ptr(qi), _ptr(ki), _ptr(wi), _ptr(cu), T,
                                 cu.numel() - 1, Hi, Di, scale, _lib.DSA_DTYPE_BF16, 0, T, skip_dense_k, _ptr(scores), ld,
                                 _stream(q_idx.device))
     _lib.check(rc, "dsa_indexer_scores")
@@ -110,7 +111,8 @@ def index_topk(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen: int, top_k: int,
     n = torch.empty((T,), dtype=torch.int32, device=q_idx.device)
     ws_bytes = lib.dsa_index_topk_workspace_bytes(T, max_seqlen, top_k) if max_seqlen > top_k else 0
     ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q_idx.device)
-    rc = lib.dsa_index_topk(_ptr(_as_bf16(q_idx)), _ptr(_as_bf16(k_idx)), _ptr(_as_bf16(w_idx)), _ptr(cu), T,
+    qi, ki, wi = _as_bf16(q_idx), _as_bf16(k_idx), _as_bf16(w_idx)     # keep the casts alive over the launch
+    rc = lib.dsa_index_topk(_ptr(qi), _ptr(ki), _ptr(wi), _ptr(cu), T,
                             cu.numel() - 1, Hi, Di, top_k, scale, _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(idx), _ptr(n),
                             _ptr(ws), ws_bytes, _stream(q_idx.device))
     _lib.check(rc, "dsa_index_topk")
@@ -130,19 +132,25 @@ def attn_fwd(q, k, v, idx, n, cu_seqlens, softmax_scale: float):
     return out, lse
 
 
-def attn_bwd(dout, q, k, v, out, lse, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float):
+def attn_bwd(dout, q, k, v, out, lse, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float,
+             parts: int = 15, buffers=None):
+    """Stage D4.  ``parts``/``buffers`` exist for per-kernel timing: ``buffers=(dq, dk, dv, ws)`` reuses
+    the outputs and workspace of an earlier full call."""
     T, Hq, Hkv, D = _check_qkv(q, k, v)
     cu = _check_cu(cu_seqlens, T)
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     K = idx.shape[1] if idx is not None else 0
     lib = _lib.load()
     ws_bytes = lib.dsa_attn_bwd_workspace_bytes(T, Hq, max_seqlen, 1 if idx is not None else 0)
-    ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q.device)
-    rc = lib.dsa_attn_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(idx), _ptr(n), _ptr(cu), T,
-                          cu.numel() - 1, Hq, Hkv, D, K, softmax_scale, _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(dq),
-                          _ptr(dk), _ptr(dv), _ptr(ws), ws_bytes, _stream(q.device))
+    if buffers is None:
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q.device)
+    else:
+        dq, dk, dv, ws = buffers
+    rc = lib.dsa_attn_bwd_parts(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(idx), _ptr(n),
+                                _ptr(cu), T, cu.numel() - 1, Hq, Hkv, D, K, softmax_scale, _lib.DSA_DTYPE_BF16,
+                                max_seqlen, _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), ws_bytes, parts, _stream(q.device))
     _lib.check(rc, "dsa_attn_bwd")
-    return dq, dk, dv
+    return (dq, dk, dv) if buffers is None else (dq, dk, dv, ws)
 
 
 # ------------------------------------------------------------------------------------------------
