@@ -69,6 +69,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="C3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 1 GiB device copy (a known-size kernel to scale rocprof's FETCH_SIZE/WRITE_SIZE by)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1",
@@ -85,6 +87,13 @@ def main():
     k = t["k"].requires_grad_(True)
     v = t["v"].requires_grad_(True)
     scale = w.D ** -0.5
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)          # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     def step():
         q.grad = k.grad = v.grad = None
@@ -140,6 +149,13 @@ def main():
         "attn_bwd": max(wk["F4"] / (PEAK_MFMA_BF16_TFLOPS * 1e12), wk["B4"] / (PEAK_HBM_GBS * 1e9)) * 1e3,
     }
     roof_total = sum(t_roof_ms.values())
+    dom_kernel = "dsa_attn_fwd_kernel" if dom == "attn_fwd" else "dsa_bwd_dq_kernel"
+    traffic = None      # HBM bytes per launch as last measured with rocprofv3 --pmc (separate runs)
+    try:
+        with open(os.path.join(ROOT, "profiles", f"hbm_traffic_{args.workload}.json")) as fh:
+            traffic = json.load(fh).get(dom_kernel)
+    except OSError:
+        pass
     result = {
         "metric": "DSA attn fwd+bwd packed tokens/s on 1 GPU at 32K; % MFMA/HBM roofline",
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -147,9 +163,9 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{w.name}: T={w.T} packed tokens, segments={list(w.seg_lens)}, Hq/Hkv/D={w.Hq}/{w.Hkv}/{w.D}, "
                                f"indexer {w.Hi}x{w.Di}, top_k={w.top_k}, fwd+bwd"},
-        "roofline": {"bound": "hbm", "kernel": "dsa_attn_fwd_kernel" if dom == "attn_fwd" else "dsa_bwd_dq_kernel",
+        "roofline": {"bound": "hbm", "kernel": dom_kernel,
                      "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS,
-                     "traffic": None, "algorithmic_bytes": kern[dom], "avg_ms": stage_ms[dom]},
+                     "traffic": traffic, "algorithmic_bytes": kern[dom], "avg_ms": stage_ms[dom]},
         "stage_ms": stage_ms,
         "roofline_whole_op": {"t_roof_ms": t_roof_ms, "sum_ms": roof_total, "frac": roof_total / ms_per_step,
                               "compute_only_bound_ms": (wk["F1"] + 3.5 * wk["F3"]) / (PEAK_MFMA_BF16_TFLOPS * 1e12) * 1e3},

@@ -156,17 +156,47 @@ def attn_bwd(dout, q, k, v, out, lse, idx, n, cu_seqlens, max_seqlen: int, softm
 # ------------------------------------------------------------------------------------------------
 # the operator
 # ------------------------------------------------------------------------------------------------
+def _split_bf16(x: torch.Tensor):
+    hi = x.to(torch.bfloat16)
+    lo = (x.float() - hi.float()).to(torch.bfloat16)
+    return hi, lo
+
+
+def _stack(parts, D):
+    """Concatenate bf16 parts along head_dim and zero-pad to 4*D (a head_dim the kernels cover)."""
+    z = torch.zeros_like(parts[0])
+    return torch.cat(list(parts) + [z] * (4 - len(parts)), dim=-1).contiguous()
+
+
 class _DsaVarlenAttn(torch.autograd.Function):
+    """bf16 inputs go to the kernels as they are.  fp32 inputs with 4*D <= 256 are carried as split-bf16
+    operands (x = hi + lo) stacked along head_dim, which keeps near-fp32 logits on the bf16 MFMA path:
+        Q' = [q_hi, q_lo, q_hi, 0]   K' = [k_hi, k_hi, k_lo, 0]   ->  Q'.K' = q.k - q_lo.k_lo
+        V' = [v_hi, v_lo, v_hi, 0]   ->  out = out'[0:D] + out'[D:2D]
+        dO' = [g_hi, g_hi, g_lo, 0]  ->  dO'.V' = g.v - g_lo.v_lo ;  dq = dq'[0:D] + dq'[2D:3D],
+                                         dk = dk'[0:D] + dk'[D:2D], dv = dv'[0:D] + dv'[2D:3D]
+    Other dtypes / larger head_dim are rounded to bf16 once."""
+
     @staticmethod
     def forward(ctx, q, k, v, cu_seqlens, max_seqlen, idx, n, softmax_scale):
         in_dtype = q.dtype
-        qb, kb, vb = _as_bf16(q), _as_bf16(k), _as_bf16(v)
+        D = q.shape[-1]
+        split = in_dtype == torch.float32 and 4 * D <= 256
+        if split:
+            (qh, ql), (kh, kl), (vh, vl) = _split_bf16(q), _split_bf16(k), _split_bf16(v)
+            qb, kb, vb = _stack((qh, ql, qh), D), _stack((kh, kh, kl), D), _stack((vh, vl, vh), D)
+        else:
+            qb, kb, vb = _as_bf16(q), _as_bf16(k), _as_bf16(v)
         out, lse = attn_fwd(qb, kb, vb, idx, n, cu_seqlens, softmax_scale)
         ctx.save_for_backward(qb, kb, vb, out, lse, cu_seqlens, *(() if idx is None else (idx, n)))
         ctx.has_idx = idx is not None
         ctx.max_seqlen = int(max_seqlen)
         ctx.softmax_scale = softmax_scale
         ctx.in_dtype = in_dtype
+        ctx.split = split
+        ctx.D = D
+        if split:
+            return out[..., :D].float() + out[..., D:2 * D].float()
         return out if in_dtype == torch.bfloat16 else out.to(in_dtype)
 
     @staticmethod
@@ -174,8 +204,18 @@ class _DsaVarlenAttn(torch.autograd.Function):
         saved = ctx.saved_tensors
         qb, kb, vb, out, lse, cu = saved[:6]
         idx, n = (saved[6], saved[7]) if ctx.has_idx else (None, None)
-        dq, dk, dv = attn_bwd(_as_bf16(dout), qb, kb, vb, out, lse, idx, n, cu, ctx.max_seqlen, ctx.softmax_scale)
-        if ctx.in_dtype != torch.bfloat16:
+        D = ctx.D
+        if ctx.split:
+            gh, gl = _split_bf16(dout)
+            db = _stack((gh, gh, gl), D)
+        else:
+            db = _as_bf16(dout)
+        dq, dk, dv = attn_bwd(db, qb, kb, vb, out, lse, idx, n, cu, ctx.max_seqlen, ctx.softmax_scale)
+        if ctx.split:
+            dq = dq[..., :D].float() + dq[..., 2 * D:3 * D].float()
+            dk = dk[..., :D].float() + dk[..., D:2 * D].float()
+            dv = dv[..., :D].float() + dv[..., 2 * D:3 * D].float()
+        elif ctx.in_dtype != torch.bfloat16:
             dq, dk, dv = dq.to(ctx.in_dtype), dk.to(ctx.in_dtype), dv.to(ctx.in_dtype)
         return dq, dk, dv, None, None, None, None, None
 
