@@ -121,14 +121,14 @@ def main():
     with torch.no_grad():
         qd, kd, vd = q.detach(), k.detach(), v.detach()
         idx, n = ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k)
-        out, lse = ops.attn_fwd(qd, kd, vd, idx, n, cu, scale)
+        out, lse = ops.attn_fwd(qd, kd, vd, idx, n, cu, msl, scale)
         bufs = ops.attn_bwd(t["dout"], qd, kd, vd, out, lse, idx, n, cu, msl, scale, 15,
                             (torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd),
                              torch.empty((ops._lib.load().dsa_attn_bwd_workspace_bytes(w.T, w.Hq, msl, 1),),
                                          dtype=torch.uint8, device=dev)))
         stage_ms = {
             "index_topk": timed(lambda: ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k), it),
-            "attn_fwd": timed(lambda: ops.attn_fwd(qd, kd, vd, idx, n, cu, scale), it),
+            "attn_fwd": timed(lambda: ops.attn_fwd(qd, kd, vd, idx, n, cu, msl, scale), it),
         }
         for name, part in (("bwd_delta", 1), ("bwd_bitmap", 2), ("bwd_dq", 4), ("bwd_dkv", 8)):
             stage_ms[name] = timed(lambda: ops.attn_bwd(t["dout"], qd, kd, vd, out, lse, idx, n, cu, msl, scale, part, bufs), it)

@@ -84,7 +84,19 @@ int dsa_index_topk(const void *q_idx, const void *k_idx, const void *w_idx, cons
  */
 int dsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
                  const int32_t *cu_seqlens, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
-                 int dtype, void *out, float *lse, void *stream);
+                 int dtype, int max_seqlen, void *out, float *lse, void *ws, size_t ws_bytes, void *stream);
+
+/* Bytes of workspace dsa_attn_fwd needs (the inverted selection bitmap; 0 without idx). */
+size_t dsa_attn_fwd_workspace_bytes(int T, int max_seqlen, int has_idx);
+
+/*
+ * Tuning knob (process-wide, no reference counterpart): query rows whose position in their segment is
+ * below top_k * crossover run on the dense MFMA tile kernels with the selection as a bitmap mask, the
+ * rest on the gather kernels.  Default 16; 0 = gather only; INT_MAX/top_k or more = tiles only.
+ * idx == NULL (dense causal attention) always uses the tile kernels.
+ */
+int dsa_set_tile_crossover(int crossover);
+int dsa_get_tile_crossover(void);
 
 /* Bytes of workspace dsa_attn_bwd needs (softmax row terms + the inverted selection bitmap). */
 size_t dsa_attn_bwd_workspace_bytes(int T, int Hq, int max_seqlen, int has_idx);
@@ -106,7 +118,7 @@ int dsa_attn_bwd(const void *dout, const void *q, const void *k, const void *v, 
  */
 #define DSA_BWD_DELTA 1  /* delta = rowsum(dO * O) */
 #define DSA_BWD_BITMAP 2 /* inverted selection bitmap (only when idx != NULL) */
-#define DSA_BWD_DQ 4     /* query-side gather pass */
+#define DSA_BWD_DQ 4     /* query-side pass (tile and/or gather kernel) */
 #define DSA_BWD_DKV 8    /* key-side pass */
 #define DSA_BWD_ALL 15
 int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k, const void *v, const void *out,

@@ -36,11 +36,16 @@ def test_workspace_sizes_without_a_gpu():
     up = lambda x: (x + 255) // 256 * 256                  # both parts are 256-byte aligned
     assert lib.dsa_attn_bwd_workspace_bytes(1000, 8, 640, 0) == up(1000 * 8 * 4)
     assert lib.dsa_attn_bwd_workspace_bytes(1000, 8, 640, 1) == up(1000 * 8 * 4) + up(1000 * 20 * 4)
+    assert lib.dsa_attn_fwd_workspace_bytes(1000, 640, 1) == up(1000 * 20 * 4)
+    assert lib.dsa_attn_fwd_workspace_bytes(1000, 640, 0) == 0
+    old = lib.dsa_get_tile_crossover()
+    assert old == 16 and lib.dsa_set_tile_crossover(-1) == -1 and lib.dsa_set_tile_crossover(3) == 0
+    assert lib.dsa_get_tile_crossover() == 3 and lib.dsa_set_tile_crossover(old) == 0
 
 
 def test_argument_errors_are_reported_not_thrown():
     lib = _lib.load()
-    rc = lib.dsa_attn_fwd(None, None, None, None, None, None, 8, 1, 4, 3, 64, 0, 1.0, 0, None, None, None)
+    rc = lib.dsa_attn_fwd(None, None, None, None, None, None, 8, 1, 4, 3, 64, 0, 1.0, 0, 8, None, None, None, 0, None)
     assert rc == -1 and b"cu_seqlens" in lib.dsa_last_error()
     with pytest.raises(ValueError):
         _lib.check(rc, "dsa_attn_fwd")

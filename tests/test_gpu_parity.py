@@ -93,6 +93,15 @@ def test_indexer_scores_match_oracle(Hi, Di):
 
 
 # ------------------------------------------------------------------------------------------ whole operator
+@pytest.fixture
+def crossover():
+    """Lets a test drive the tile kernels, the gather kernels, or a mix; restores the default afterwards."""
+    old = ops.set_tile_crossover(16)
+    ops.set_tile_crossover(old)
+    yield ops.set_tile_crossover
+    ops.set_tile_crossover(old)
+
+
 def _run_case(w, check_bwd=True):
     t = W.make_inputs(w, device="cpu")
     cu = t["cu_seqlens"]
@@ -134,6 +143,28 @@ def test_c1_toy_fp32_full():
 def test_scaled_configs(name, segs, K):
     _log(f"scaled {name}")
     _run_case(W.scaled(W.WORKLOADS[name], segs, top_k=K, name=name + "-scaled"))
+
+
+@pytest.mark.parametrize("name,segs,K", [
+    ("C3", (900, 70, 333), 64),
+    ("C5", (420, 65, 300), 32),
+    ("C1", (300, 200), 16),
+])
+def test_tile_and_gather_paths_agree_with_the_oracle(crossover, name, segs, K):
+    """crossover 0 = gather kernels only, 1<<20 = tile kernels only, 2 = rows split at pos 2K (rounded to 128)."""
+    _log(f"paths {name}")
+    w = W.scaled(W.WORKLOADS[name], segs, top_k=K, name=name + "-paths")
+    outs = {}
+    for c in (0, 1 << 20, 2):
+        crossover(c)
+        outs[c] = _run_case(w).detach().float()
+    assert (outs[0] - outs[1 << 20]).abs().max().item() < 2e-2
+    split = (2 * K + 127) // 128 * 128            # mixed run: tile rows before the split, gather rows after
+    a = 0
+    for L in segs:
+        assert torch.equal(outs[2][a:a + min(L, split)], outs[1 << 20][a:a + min(L, split)])
+        assert torch.equal(outs[2][a + min(L, split):a + L], outs[0][a + min(L, split):a + L])
+        a += L
 
 
 def test_dense_path_equals_reference_semantics():

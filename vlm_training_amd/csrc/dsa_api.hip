@@ -13,12 +13,24 @@ hipError_t dsa_launch_indexer(const void *q_idx, const void *k_idx, const void *
                               int T, int Hi, int Di, float scale, int row_begin, int row_end, int skip_dense_k,
                               float *scores, int64_t ld, hipStream_t stream);
 hipError_t dsa_launch_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
-                               const int32_t *cu, int N, int T, int Hq, int Hkv, int D, int K, float scale, void *out,
-                               float *lse, hipStream_t stream);
-hipError_t dsa_launch_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
-                               const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu, int N, int T,
-                               int Hq, int Hkv, int D, int K, float scale, int max_seqlen, void *dq, void *dk,
-                               void *dv, float *delta, uint32_t *bitmap, int ldw, int parts, hipStream_t stream);
+                               const int32_t *cu, int N, int T, int Hq, int Hkv, int D, int K, float scale, int pos_min,
+                               void *out, float *lse, hipStream_t stream);
+hipError_t dsa_launch_delta(const void *dout, const void *out, int T, int Hq, int D, float *delta, hipStream_t stream);
+hipError_t dsa_launch_bitmap(const int32_t *idx, const int32_t *n, const int32_t *cu, int N, int T, int K, int ldw,
+                             uint32_t *bitmap, hipStream_t stream);
+hipError_t dsa_launch_gather_dq(const void *dout, const void *q, const void *k, const void *v, const float *lse,
+                                const float *delta, const int32_t *idx, const int32_t *n, const int32_t *cu, int N,
+                                int T, int Hq, int Hkv, int D, int K, float scale, int pos_min, void *dq,
+                                hipStream_t stream);
+hipError_t dsa_launch_tile_fwd(const void *q, const void *k, const void *v, const uint32_t *bitmap, int ldw,
+                               const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale, int pos_split,
+                               void *out, float *lse, hipStream_t stream);
+hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const void *k, const void *v, const float *lse,
+                              const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T,
+                              int Hq, int Hkv, int D, float scale, int pos_split, void *dq, hipStream_t stream);
+hipError_t dsa_launch_tile_dkv(const void *dout, const void *q, const void *k, const void *v, const float *lse,
+                               const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T,
+                               int Hq, int Hkv, int D, float scale, void *dk, void *dv, hipStream_t stream);
 }
 
 static thread_local char g_err[512] = "";
@@ -120,16 +132,62 @@ static int check_attn(int T, int N, const int32_t *cu, int Hq, int Hkv, int D, i
     return DSA_OK;
 }
 
-extern "C" int dsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
-                            const int32_t *cu, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
-                            int dtype, void *out, float *lse, void *stream) {
-    if (int rc = check_attn(T, N, cu, Hq, Hkv, D, K, dtype, idx, n)) return rc;
-    if (!q || !k || !v || !out || !lse) return fail(DSA_ERR_ARG, "null tensor pointer");
-    hipError_t e = dsa_launch_attn_fwd(q, k, v, idx, n, cu, N, T, Hq, Hkv, D, K, softmax_scale, out, lse, (hipStream_t)stream);
-    return e == hipSuccess ? DSA_OK : hip_fail(e, "attention forward launch");
+static inline int bitmap_ldw(int max_seqlen) { return (max_seqlen + 31) / 32; }
+
+// Query rows whose position in their segment is below top_k * crossover are handled by the tile
+// kernels (their selection covers more than 1/crossover of the causal window), the rest by the
+// gather kernels.  Process-wide tuning knob; 0 = gather only, a huge value = tile only.
+static int g_tile_crossover = 16;
+extern "C" int dsa_set_tile_crossover(int crossover) {
+    if (crossover < 0) return fail(DSA_ERR_ARG, "crossover=%d must be >= 0", crossover);
+    g_tile_crossover = crossover;
+    return DSA_OK;
+}
+extern "C" int dsa_get_tile_crossover(void) { return g_tile_crossover; }
+
+// first query position handled by the gather kernels (multiple of 128, the coarsest tile block)
+static int pos_split_for(const int32_t *idx, int K) {
+    if (!idx) return INT32_MAX;                       // dense causal: tiles everywhere
+    const int64_t p = (int64_t)K * g_tile_crossover;
+    if (p >= INT32_MAX - 256) return INT32_MAX;
+    return (int)((p + 127) / 128 * 128);
 }
 
-static inline int bitmap_ldw(int max_seqlen) { return (max_seqlen + 31) / 32; }
+extern "C" size_t dsa_attn_fwd_workspace_bytes(int T, int max_seqlen, int has_idx) {
+    if (T <= 0 || !has_idx) return 0;
+    return align_up((size_t)T * bitmap_ldw(max_seqlen) * 4, 256);
+}
+
+extern "C" int dsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
+                            const int32_t *cu, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
+                            int dtype, int max_seqlen, void *out, float *lse, void *ws, size_t ws_bytes, void *stream) {
+    if (int rc = check_attn(T, N, cu, Hq, Hkv, D, K, dtype, idx, n)) return rc;
+    if (!q || !k || !v || !out || !lse) return fail(DSA_ERR_ARG, "null tensor pointer");
+    if (max_seqlen < 1 || max_seqlen > (T > 0 ? T : 1)) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
+    if (T == 0) return DSA_OK;
+    const int split = pos_split_for(idx, K);
+    const int ldw = bitmap_ldw(max_seqlen);
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e = hipSuccess;
+    if (split > 0) {
+        uint32_t *bitmap = nullptr;
+        if (idx) {
+            const size_t need = dsa_attn_fwd_workspace_bytes(T, max_seqlen, 1);
+            if (!ws || ws_bytes < need) return fail(DSA_ERR_WORKSPACE, "forward workspace: have %zu bytes, need %zu", ws_bytes, need);
+            if ((size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);
+            bitmap = (uint32_t *)ws;
+            e = dsa_launch_bitmap(idx, n, cu, N, T, K, ldw, bitmap, st);
+            if (e != hipSuccess) return hip_fail(e, "bitmap launch");
+        }
+        e = dsa_launch_tile_fwd(q, k, v, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, split, out, lse, st);
+        if (e != hipSuccess) return hip_fail(e, "tile forward launch");
+    }
+    if (max_seqlen > split) {
+        e = dsa_launch_attn_fwd(q, k, v, idx, n, cu, N, T, Hq, Hkv, D, K, softmax_scale, split, out, lse, st);
+        if (e != hipSuccess) return hip_fail(e, "gather forward launch");
+    }
+    return DSA_OK;
+}
 
 extern "C" size_t dsa_attn_bwd_workspace_bytes(int T, int Hq, int max_seqlen, int has_idx) {
     if (T <= 0) return 0;
@@ -152,9 +210,32 @@ extern "C" int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k
     if (idx && (size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);
     float *delta = (float *)ws;
     uint32_t *bitmap = idx ? (uint32_t *)((char *)ws + align_up((size_t)T * Hq * 4, 256)) : nullptr;
-    hipError_t e = dsa_launch_attn_bwd(dout, q, k, v, out, lse, idx, n, cu, N, T, Hq, Hkv, D, K, softmax_scale, max_seqlen,
-                                       dq, dk, dv, delta, bitmap, ldw, parts, (hipStream_t)stream);
-    return e == hipSuccess ? DSA_OK : hip_fail(e, "attention backward launch");
+    const int split = pos_split_for(idx, K);
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e = hipSuccess;
+    if (parts & DSA_BWD_DELTA) {
+        e = dsa_launch_delta(dout, out, T, Hq, D, delta, st);
+        if (e != hipSuccess) return hip_fail(e, "delta launch");
+    }
+    if ((parts & DSA_BWD_BITMAP) && idx) {
+        e = dsa_launch_bitmap(idx, n, cu, N, T, K, ldw, bitmap, st);
+        if (e != hipSuccess) return hip_fail(e, "bitmap launch");
+    }
+    if (parts & DSA_BWD_DQ) {
+        if (split > 0) {
+            e = dsa_launch_tile_dq(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, split, dq, st);
+            if (e != hipSuccess) return hip_fail(e, "tile dq launch");
+        }
+        if (max_seqlen > split) {
+            e = dsa_launch_gather_dq(dout, q, k, v, lse, delta, idx, n, cu, N, T, Hq, Hkv, D, K, softmax_scale, split, dq, st);
+            if (e != hipSuccess) return hip_fail(e, "gather dq launch");
+        }
+    }
+    if (parts & DSA_BWD_DKV) {
+        e = dsa_launch_tile_dkv(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, dk, dv, st);
+        if (e != hipSuccess) return hip_fail(e, "tile dkv launch");
+    }
+    return DSA_OK;
 }
 
 extern "C" int dsa_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,

@@ -21,7 +21,7 @@ template <int D, bool HAS_IDX>
 __global__ __launch_bounds__(64) void dsa_attn_fwd_kernel(
     const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
     const int32_t *__restrict__ idx, const int32_t *__restrict__ nsel, const int32_t *__restrict__ cu, int N, int T,
-    int Hq, int Hkv, int K, float scale_log2, bf16_t *__restrict__ out, float *__restrict__ lse) {
+    int Hq, int Hkv, int K, float scale_log2, int pos_min, bf16_t *__restrict__ out, float *__restrict__ lse) {
     constexpr int KS = D / 32;            // MFMA k-steps of the QK^T contraction
     constexpr int DT = D / 16;            // 16-row tiles of O^T
     constexpr int ROW_B = D * 2 + 8;      // padded LDS row: conflict-free transposed reads
@@ -33,6 +33,7 @@ __global__ __launch_bounds__(64) void dsa_attn_fwd_kernel(
     const int kvh = blockIdx.x % Hkv, t = blockIdx.x / Hkv;
     const int G = Hq / Hkv;
     const int s0 = cu[find_segment(cu, N, t)];
+    if (t - s0 < pos_min) return;                             // rows before the split belong to the tile kernel
     const int nt = HAS_IDX ? nsel[t] : (t - s0 + 1);
     const int32_t *irow = HAS_IDX ? idx + (int64_t)t * K : nullptr;
     auto key_of = [&](int j) -> int {
@@ -152,27 +153,27 @@ __global__ __launch_bounds__(64) void dsa_attn_fwd_kernel(
 
 template <int D>
 static hipError_t launch_fwd(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
-                             const int32_t *cu, int N, int T, int Hq, int Hkv, int K, float scale, void *out,
-                             float *lse, hipStream_t stream) {
+                             const int32_t *cu, int N, int T, int Hq, int Hkv, int K, float scale, int pos_min,
+                             void *out, float *lse, hipStream_t stream) {
     const dim3 grid((unsigned)((int64_t)T * Hkv)), block(64);
     const float sl2 = scale * LOG2E_F;
     if (idx)
         hipLaunchKernelGGL((dsa_attn_fwd_kernel<D, true>), grid, block, 0, stream, (const bf16_t *)q, (const bf16_t *)k,
-                           (const bf16_t *)v, idx, n, cu, N, T, Hq, Hkv, K, sl2, (bf16_t *)out, lse);
+                           (const bf16_t *)v, idx, n, cu, N, T, Hq, Hkv, K, sl2, pos_min, (bf16_t *)out, lse);
     else
         hipLaunchKernelGGL((dsa_attn_fwd_kernel<D, false>), grid, block, 0, stream, (const bf16_t *)q,
-                           (const bf16_t *)k, (const bf16_t *)v, idx, n, cu, N, T, Hq, Hkv, K, sl2, (bf16_t *)out, lse);
+                           (const bf16_t *)k, (const bf16_t *)v, idx, n, cu, N, T, Hq, Hkv, K, sl2, pos_min, (bf16_t *)out, lse);
     return hipGetLastError();
 }
 
 extern "C" hipError_t dsa_launch_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx,
                                           const int32_t *n, const int32_t *cu, int N, int T, int Hq, int Hkv, int D,
-                                          int K, float scale, void *out, float *lse, hipStream_t stream) {
+                                          int K, float scale, int pos_min, void *out, float *lse, hipStream_t stream) {
     if (T == 0) return hipSuccess;
     switch (D) {
-        case 64: return launch_fwd<64>(q, k, v, idx, n, cu, N, T, Hq, Hkv, K, scale, out, lse, stream);
-        case 128: return launch_fwd<128>(q, k, v, idx, n, cu, N, T, Hq, Hkv, K, scale, out, lse, stream);
-        case 256: return launch_fwd<256>(q, k, v, idx, n, cu, N, T, Hq, Hkv, K, scale, out, lse, stream);
+        case 64: return launch_fwd<64>(q, k, v, idx, n, cu, N, T, Hq, Hkv, K, scale, pos_min, out, lse, stream);
+        case 128: return launch_fwd<128>(q, k, v, idx, n, cu, N, T, Hq, Hkv, K, scale, pos_min, out, lse, stream);
+        case 256: return launch_fwd<256>(q, k, v, idx, n, cu, N, T, Hq, Hkv, K, scale, pos_min, out, lse, stream);
         default: return hipErrorInvalidValue;
     }
 }

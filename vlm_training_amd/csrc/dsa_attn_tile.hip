@@ -1,0 +1,537 @@
+// Tile kernels: attention forward / dQ / dK,dV over 32x32 MFMA tiles with the selection applied as a
+// bitmap mask.  They do the same arithmetic as the gather kernels but visit every (query block, key
+// tile) pair of the causal triangle, so they win wherever the selection is dense: one selected pair
+// costs the gather kernels 2*D*e bytes of L2 traffic per kv head, a causal pair costs these kernels
+// 4*G*D flop on the matrix cores - on MI355X the tile walk is cheaper down to a few percent density.
+//
+// Common scheme (wave64, v_mfma_f32_32x32x16_bf16):
+//   rows of the problem are (query, head-in-group) pairs, `Gp` (power of two >= G) rows per query;
+//   the mask depends on the query only.  Operands that move (K,V tiles for the query-stationary
+//   kernels, q,dO blocks for the key-stationary one) are staged once per workgroup in LDS, row-major
+//   with an XOR swizzle of the 16-byte chunks, and read either row-wise (16-byte reads, contraction
+//   over D) or transposed with ds_read_b64_tr_b16 (contraction over rows/keys) - both conflict-free.
+//   The second GEMM of each chain takes its B operand straight from the C layout of the first
+//   (the contraction order over the 32 keys/rows of a tile is permuted identically on both operands).
+#include "dsa_common.h"
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }   // v_exp_f32; exp2(-inf) = 0
+
+// ---- swizzled LDS tile: rows of D bf16 (D*2 bytes, no padding); chunk = 16 bytes -----------------
+__device__ __forceinline__ int tile_sw(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
+template <int D>
+__device__ __forceinline__ int tile_off(int row, int chunk) { return row * (D * 2) + ((chunk ^ tile_sw(row)) << 4); }
+
+// A operand of mfma32 read row-wise: lane (i = row, h) takes elements [16*ks + 8h, +8) of row i
+template <int D>
+__device__ __forceinline__ bf16x8 tile_rowop(const unsigned char *tile, int row, int ks, int h) {
+    return *reinterpret_cast<const bf16x8 *>(tile + tile_off<D>(row, 2 * ks + h));
+}
+// A operand of mfma32 read transposed: lane l takes column c = m0 + (l & 15) and the 8 rows
+// {R0..R0+3, R0+8..R0+11}.  ds_read_b64_tr_b16: within 16 lanes, lane s supplies the address of 4
+// consecutive elements of row R0 + s/4 at column m0 + 4*(s%4); lane s receives rows R0..R0+3 of column m0+s.
+template <int D>
+__device__ __forceinline__ bf16x8 tile_trop(const unsigned char *tile, int R0, int m0, int lane) {
+    const int s = lane & 15;
+    const int row = R0 + (s >> 2), col = m0 + ((s & 3) << 2);
+    const int sub = ((col >> 2) & 1) << 3;
+    const unsigned char *p0 = tile + tile_off<D>(row, col >> 3) + sub;
+    const unsigned char *p1 = tile + tile_off<D>(row + 8, col >> 3) + sub;
+    const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p0);
+    const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p1);
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    const s16x8 r = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+    return __builtin_bit_cast(bf16x8, r);
+}
+__device__ __forceinline__ bf16x8 pack8(const float *x) {
+    const u32x4 w = {pack2bf(x[0], x[1]), pack2bf(x[2], x[3]), pack2bf(x[4], x[5]), pack2bf(x[6], x[7])};
+    return __builtin_bit_cast(bf16x8, w);
+}
+__device__ __forceinline__ f32x16 zero16() {
+    f32x16 z;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) z[v] = 0.f;
+    return z;
+}
+// key / row index inside a 32-tile held by accumulator element v of lane half h (C layout of mfma32)
+__device__ __forceinline__ int c_row(int v, int h) { return 8 * (v >> 2) + 4 * h + (v & 3); }
+
+// slot -> (segment, block) for blocks of `blk` columns handed out segment by segment; within a segment
+// the blocks are numbered from the end when `reverse` (heaviest causal blocks first).  Returns false
+// for spare slots.
+__device__ __forceinline__ bool locate_block(const int32_t *cu, int N, int slot, int blk, bool reverse, int &s0, int &L,
+                                             int &b) {
+    for (int seg = 0; seg < N; ++seg) {
+        s0 = cu[seg];
+        L = cu[seg + 1] - s0;
+        const int nb = (L + blk - 1) / blk;
+        if (slot < nb) {
+            b = reverse ? nb - 1 - slot : slot;
+            return true;
+        }
+        slot -= nb;
+    }
+    return false;
+}
+
+// ==================================================================================================
+// forward: query-stationary.  Workgroup = 4 waves x 32 rows = 128 rows = 128/Gp queries of one
+// segment and one kv head; loops over 32-key tiles of the causal range.
+//   S^T[key,row] = K[key,:].Q[row,:]   (A = K tile row-wise from LDS, B = Q^T in registers)
+//   online softmax on the C layout (lane = row; one cross-lane step per statistic)
+//   O^T[d,row]  += V^T[d,key] P^T[key,row]   (A = V tile transposed from LDS, B = P^T from the C layout)
+// ==================================================================================================
+template <int D, bool HAS_IDX>
+__global__ __launch_bounds__(256) void dsa_tile_fwd_kernel(
+    const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
+    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv, int Gp,
+    int gshift, float scale_log2, int pos_split, bf16_t *__restrict__ out, float *__restrict__ lse) {
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2, LOADS = 32 * CPR / 256;
+    constexpr int NBUF = (D > 128) ? 1 : 2;           // double buffering where 64 KiB of static LDS allow it
+    static_assert(LOADS >= 1, "tile must give every thread a chunk");
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];   // [buffer][K|V]
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
+    const int G = Hq / Hkv, QBW = 128 >> gshift;
+    const int kvh = blockIdx.x % Hkv;
+    int s0, L, blk;
+    if (!locate_block(cu, N, blockIdx.x / Hkv, QBW, true, s0, L, blk)) return;
+    const int qc0 = blk * QBW;
+    if (qc0 >= pos_split) return;                       // rows past the split belong to the gather kernel
+
+    const int r = wv * 32 + j;
+    const int qcol = qc0 + (r >> gshift), head = r & (Gp - 1);
+    const bool row_ok = qcol < L && head < G;
+    const int t = s0 + min(qcol, L - 1), hq = kvh * G + min(head, G - 1);
+    bf16x8 qB[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+        qB[ks] = row_ok ? load_bf16x8(q + ((int64_t)t * Hq + hq) * D + 16 * ks + 8 * h) : zero_bf16x8();
+    const int wq_last = min(qc0 + ((wv * 32 + 31) >> gshift), L - 1);
+    const int ntiles = min(qc0 + QBW - 1, L - 1) / 32 + 1;
+
+    u32x4 kst[LOADS], vst[LOADS];
+    auto load_tile = [&](int kc0) {
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const int c = i * 256 + tid;
+            const int row = c / CPR, ch = c % CPR;
+            const int64_t off = ((int64_t)(s0 + min(kc0 + row, L - 1)) * Hkv + kvh) * D + ch * 8;
+            kst[i] = *reinterpret_cast<const u32x4 *>(k + off);
+            vst[i] = *reinterpret_cast<const u32x4 *>(v + off);
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const int c = i * 256 + tid;
+            const int row = c / CPR, ch = c % CPR;
+            *reinterpret_cast<u32x4 *>(&lds[buf][0][tile_off<D>(row, ch)]) = kst[i];
+            *reinterpret_cast<u32x4 *>(&lds[buf][1][tile_off<D>(row, ch)]) = vst[i];
+        }
+    };
+
+    f32x16 oacc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) oacc[dt] = zero16();
+    float mrun = -INFINITY, lsum = 0.f;
+
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+    for (int it = 0; it < ntiles; ++it) {
+        const int kc0 = it * 32;
+        if (it + 1 < ntiles) load_tile(kc0 + 32);
+        uint32_t word = 0u;
+        if (HAS_IDX && row_ok) word = bitmap[(int64_t)t * ldw + it];
+        if (kc0 <= wq_last) {                            // wave-uniform: tile not entirely above the diagonal
+            const unsigned char *kt = lds[it & (NBUF - 1)][0], *vt = lds[it & (NBUF - 1)][1];
+            f32x16 sacc = zero16();
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) sacc = mfma32(tile_rowop<D>(kt, j, ks, h), qB[ks], sacc);
+            float s2[16], mloc = -INFINITY;
+#pragma unroll
+            for (int vi = 0; vi < 16; ++vi) {
+                const int kk = c_row(vi, h);
+                const bool on = HAS_IDX ? ((word >> kk) & 1u) : (row_ok && kc0 + kk <= qcol);
+                s2[vi] = on ? sacc[vi] * scale_log2 : -INFINITY;
+                mloc = fmaxf(mloc, s2[vi]);
+            }
+            mloc = fmaxf(mloc, wave_xor_f(mloc, 32));
+            const float mnew = fmaxf(mrun, mloc);
+            const float mref = (mnew == -INFINITY) ? 0.f : mnew;     // rows with nothing selected so far
+            const float alpha = fast_exp2(mrun - mref);
+            float psum = 0.f;
+#pragma unroll
+            for (int vi = 0; vi < 16; ++vi) { s2[vi] = fast_exp2(s2[vi] - mref); psum += s2[vi]; }
+            lsum = lsum * alpha + psum;
+            mrun = mnew;
+            const bf16x8 pB0 = pack8(s2), pB1 = pack8(s2 + 8);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                oacc[dt] *= alpha;
+                const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;
+                oacc[dt] = mfma32(tile_trop<D>(vt, 4 * h, m0, lane), pB0, oacc[dt]);
+                oacc[dt] = mfma32(tile_trop<D>(vt, 16 + 4 * h, m0, lane), pB1, oacc[dt]);
+            }
+        }
+        if (NBUF == 1) __syncthreads();                   // single buffer: everyone is done reading it
+        if (it + 1 < ntiles) store_tile((it + 1) & (NBUF - 1));
+        __syncthreads();
+    }
+    float l = lsum + wave_xor_f(lsum, 32);
+    if (row_ok) {
+        const float inv = 1.f / l;
+        bf16_t *op = out + ((int64_t)t * Hq + hq) * D + 4 * h;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const u32x2 w2 = {pack2bf(oacc[dt][4 * g4] * inv, oacc[dt][4 * g4 + 1] * inv),
+                                  pack2bf(oacc[dt][4 * g4 + 2] * inv, oacc[dt][4 * g4 + 3] * inv)};
+                *reinterpret_cast<u32x2 *>(op + dt * 32 + 8 * g4) = w2;
+            }
+        if (h == 0) lse[(int64_t)hq * T + t] = (mrun + log2f(l)) * LN2_F;
+    }
+}
+
+// ==================================================================================================
+// dQ: query-stationary, same walk as the forward.
+//   S^T = K Q^T, dP^T = V dO^T  (A = K / V tiles row-wise, B = Q^T / dO^T in registers)
+//   dS^T = P^T * (dP^T - delta)  on the C layout
+//   dQ^T[d,row] += K^T[d,key] dS^T[key,row]   (A = K tile transposed, B = dS^T from the C layout)
+// ==================================================================================================
+template <int D, bool HAS_IDX>
+__global__ __launch_bounds__(256) void dsa_tile_dq_kernel(
+    const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
+    const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
+    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv, int Gp,
+    int gshift, float scale, int pos_split, bf16_t *__restrict__ dq) {
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2, LOADS = 32 * CPR / 256;
+    constexpr int NBUF = (D > 128) ? 1 : 2;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
+    const int G = Hq / Hkv, QBW = 128 >> gshift;
+    const int kvh = blockIdx.x % Hkv;
+    int s0, L, blk;
+    if (!locate_block(cu, N, blockIdx.x / Hkv, QBW, true, s0, L, blk)) return;
+    const int qc0 = blk * QBW;
+    if (qc0 >= pos_split) return;
+
+    const int r = wv * 32 + j;
+    const int qcol = qc0 + (r >> gshift), head = r & (Gp - 1);
+    const bool row_ok = qcol < L && head < G;
+    const int t = s0 + min(qcol, L - 1), hq = kvh * G + min(head, G - 1);
+    const float scale_log2 = scale * LOG2E_F;
+    bf16x8 qB[KS], doB[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const int64_t off = ((int64_t)t * Hq + hq) * D + 16 * ks + 8 * h;
+        qB[ks] = row_ok ? load_bf16x8(q + off) : zero_bf16x8();
+        doB[ks] = row_ok ? load_bf16x8(dout + off) : zero_bf16x8();
+    }
+    const float lse2 = lse[(int64_t)hq * T + t] * LOG2E_F;
+    const float dlt = delta[(int64_t)hq * T + t];
+    const int wq_last = min(qc0 + ((wv * 32 + 31) >> gshift), L - 1);
+    const int ntiles = min(qc0 + QBW - 1, L - 1) / 32 + 1;
+
+    u32x4 kst[LOADS], vst[LOADS];
+    auto load_tile = [&](int kc0) {
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const int c = i * 256 + tid;
+            const int row = c / CPR, ch = c % CPR;
+            const int64_t off = ((int64_t)(s0 + min(kc0 + row, L - 1)) * Hkv + kvh) * D + ch * 8;
+            kst[i] = *reinterpret_cast<const u32x4 *>(k + off);
+            vst[i] = *reinterpret_cast<const u32x4 *>(v + off);
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const int c = i * 256 + tid;
+            const int row = c / CPR, ch = c % CPR;
+            *reinterpret_cast<u32x4 *>(&lds[buf][0][tile_off<D>(row, ch)]) = kst[i];
+            *reinterpret_cast<u32x4 *>(&lds[buf][1][tile_off<D>(row, ch)]) = vst[i];
+        }
+    };
+    f32x16 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
+
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+    for (int it = 0; it < ntiles; ++it) {
+        const int kc0 = it * 32;
+        if (it + 1 < ntiles) load_tile(kc0 + 32);
+        uint32_t word = 0u;
+        if (HAS_IDX && row_ok) word = bitmap[(int64_t)t * ldw + it];
+        if (kc0 <= wq_last) {
+            const unsigned char *kt = lds[it & (NBUF - 1)][0], *vt = lds[it & (NBUF - 1)][1];
+            f32x16 sacc = zero16(), pacc = zero16();
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                sacc = mfma32(tile_rowop<D>(kt, j, ks, h), qB[ks], sacc);
+                pacc = mfma32(tile_rowop<D>(vt, j, ks, h), doB[ks], pacc);
+            }
+            float ds[16];
+#pragma unroll
+            for (int vi = 0; vi < 16; ++vi) {
+                const int kk = c_row(vi, h);
+                const bool on = HAS_IDX ? ((word >> kk) & 1u) : (row_ok && kc0 + kk <= qcol);
+                const float p = on ? fast_exp2(sacc[vi] * scale_log2 - lse2) : 0.f;
+                ds[vi] = p * (pacc[vi] - dlt);
+            }
+            const bf16x8 dB0 = pack8(ds), dB1 = pack8(ds + 8);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;
+                acc[dt] = mfma32(tile_trop<D>(kt, 4 * h, m0, lane), dB0, acc[dt]);
+                acc[dt] = mfma32(tile_trop<D>(kt, 16 + 4 * h, m0, lane), dB1, acc[dt]);
+            }
+        }
+        if (NBUF == 1) __syncthreads();                   // single buffer: everyone is done reading it
+        if (it + 1 < ntiles) store_tile((it + 1) & (NBUF - 1));
+        __syncthreads();
+    }
+    if (row_ok) {
+        bf16_t *op = dq + ((int64_t)t * Hq + hq) * D + 4 * h;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const u32x2 w2 = {pack2bf(acc[dt][4 * g4] * scale, acc[dt][4 * g4 + 1] * scale),
+                                  pack2bf(acc[dt][4 * g4 + 2] * scale, acc[dt][4 * g4 + 3] * scale)};
+                *reinterpret_cast<u32x2 *>(op + dt * 32 + 8 * g4) = w2;
+            }
+    }
+}
+
+// ==================================================================================================
+// dK, dV: key-stationary ("scatter by key": every key row is reduced by exactly one wave, in query
+// order, so the result needs no atomics and is bit-reproducible).  Workgroup = 4 waves x 32 keys = one
+// 128-key tile of a segment and one kv head; walks the queries from the tile's first column to the end
+// of the segment in blocks of 32 (query, head) rows staged in LDS.
+//   S[row,key] = Q K^T, dP = dO V^T     (A = q / dO block row-wise, B = K^T / V^T in registers)
+//   dV^T[d,key] += dO^T[d,row] P[row,key]   dK^T[d,key] += Q^T[d,row] dS[row,key]
+//                                           (A = dO / q block transposed, B = P / dS from the C layout)
+// ==================================================================================================
+template <int D, bool HAS_IDX>
+__global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
+    const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
+    const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
+    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv, int Gp,
+    int gshift, float scale, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2, LOADS = 32 * CPR / 256;
+    constexpr int NBUF = (D > 128) ? 1 : 2;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];   // [buffer][q|dO]
+    __shared__ float lse_s[NBUF][32], dlt_s[NBUF][32];
+    __shared__ uint32_t mask_s[NBUF][32][4];                                     // [buffer][query in block][wave]
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
+    const int G = Hq / Hkv, QB = 32 >> gshift;
+    const int kvh = blockIdx.x % Hkv;
+    int s0, L, blk;
+    if (!locate_block(cu, N, blockIdx.x / Hkv, 128, false, s0, L, blk)) return;
+    const int c0 = blk * 128, kc = c0 + wv * 32;
+    const int mykey = kc + j;
+    const bool key_ok = mykey < L;
+    const int64_t krow = (int64_t)(s0 + min(mykey, L - 1)) * Hkv + kvh;
+    bf16x8 kB[KS], vB[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        kB[ks] = load_bf16x8(k + krow * D + 16 * ks + 8 * h);
+        vB[ks] = load_bf16x8(v + krow * D + 16 * ks + 8 * h);
+    }
+    f32x16 dkacc[DT], dvacc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) { dkacc[dt] = zero16(); dvacc[dt] = zero16(); }
+    const float scale_log2 = scale * LOG2E_F;
+
+    u32x4 qst[LOADS], dost[LOADS];
+    float lse_st = 0.f, dlt_st = 0.f;
+    uint32_t mask_st = 0u;
+    auto load_block = [&](int qc0) {
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const int c = i * 256 + tid;
+            const int row = c / CPR, ch = c % CPR;
+            const int qc = min(qc0 + (row >> gshift), L - 1);
+            const int hd = min(row & (Gp - 1), G - 1);
+            const int64_t off = ((int64_t)(s0 + qc) * Hq + kvh * G + hd) * D + ch * 8;
+            qst[i] = *reinterpret_cast<const u32x4 *>(q + off);
+            dost[i] = *reinterpret_cast<const u32x4 *>(dout + off);
+        }
+        if (tid < 32) {
+            const int qc = min(qc0 + (tid >> gshift), L - 1);
+            const int hd = min(tid & (Gp - 1), G - 1);
+            lse_st = lse[(int64_t)(kvh * G + hd) * T + s0 + qc] * LOG2E_F;
+            dlt_st = delta[(int64_t)(kvh * G + hd) * T + s0 + qc];
+        } else if (HAS_IDX && tid >= 64 && tid < 64 + 4 * QB) {
+            const int qi = (tid - 64) >> 2, w = (tid - 64) & 3;
+            const int qc = qc0 + qi;
+            mask_st = (qc < L && (c0 >> 5) + w < ldw) ? bitmap[(int64_t)(s0 + qc) * ldw + (c0 >> 5) + w] : 0u;
+        }
+    };
+    auto store_block = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const int c = i * 256 + tid;
+            const int row = c / CPR, ch = c % CPR;
+            *reinterpret_cast<u32x4 *>(&lds[buf][0][tile_off<D>(row, ch)]) = qst[i];
+            *reinterpret_cast<u32x4 *>(&lds[buf][1][tile_off<D>(row, ch)]) = dost[i];
+        }
+        if (tid < 32) { lse_s[buf][tid] = lse_st; dlt_s[buf][tid] = dlt_st; }
+        else if (HAS_IDX && tid >= 64 && tid < 64 + 4 * QB) mask_s[buf][(tid - 64) >> 2][(tid - 64) & 3] = mask_st;
+    };
+
+    const int nblocks = (L - c0 + QB - 1) / QB;          // queries c0 .. L-1
+    load_block(c0);
+    store_block(0);
+    __syncthreads();
+    for (int b = 0; b < nblocks; ++b) {
+        const int qc0 = c0 + b * QB, buf = b & (NBUF - 1);
+        if (b + 1 < nblocks) load_block(qc0 + QB);
+        if (qc0 + QB - 1 >= kc) {                          // wave-uniform: some query of the block sees this wave's keys
+            const unsigned char *qt = lds[buf][0], *dot = lds[buf][1];
+            f32x16 sacc = zero16(), pacc = zero16();
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                sacc = mfma32(tile_rowop<D>(qt, j, ks, h), kB[ks], sacc);
+                pacc = mfma32(tile_rowop<D>(dot, j, ks, h), vB[ks], pacc);
+            }
+            float pv[16], dsv[16];
+#pragma unroll
+            for (int vi = 0; vi < 16; ++vi) {
+                const int row = c_row(vi, h);
+                const int qi = row >> gshift, hd = row & (Gp - 1);
+                const int qc = qc0 + qi;
+                bool on = key_ok && qc < L && hd < G && mykey <= qc;
+                if (HAS_IDX) on = on && ((mask_s[buf][qi][wv] >> j) & 1u);
+                const float p = on ? fast_exp2(sacc[vi] * scale_log2 - lse_s[buf][row]) : 0.f;
+                pv[vi] = p;
+                dsv[vi] = p * (pacc[vi] - dlt_s[buf][row]);
+            }
+            const bf16x8 pB0 = pack8(pv), pB1 = pack8(pv + 8), dB0 = pack8(dsv), dB1 = pack8(dsv + 8);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;
+                dvacc[dt] = mfma32(tile_trop<D>(dot, 4 * h, m0, lane), pB0, dvacc[dt]);
+                dvacc[dt] = mfma32(tile_trop<D>(dot, 16 + 4 * h, m0, lane), pB1, dvacc[dt]);
+                dkacc[dt] = mfma32(tile_trop<D>(qt, 4 * h, m0, lane), dB0, dkacc[dt]);
+                dkacc[dt] = mfma32(tile_trop<D>(qt, 16 + 4 * h, m0, lane), dB1, dkacc[dt]);
+            }
+        }
+        if (NBUF == 1) __syncthreads();
+        if (b + 1 < nblocks) store_block((b + 1) & (NBUF - 1));
+        __syncthreads();
+    }
+    if (key_ok) {
+        bf16_t *pk = dk + krow * D + 4 * h, *pv_ = dv + krow * D + 4 * h;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const u32x2 wk = {pack2bf(dkacc[dt][4 * g4] * scale, dkacc[dt][4 * g4 + 1] * scale),
+                                  pack2bf(dkacc[dt][4 * g4 + 2] * scale, dkacc[dt][4 * g4 + 3] * scale)};
+                const u32x2 wvv = {pack2bf(dvacc[dt][4 * g4], dvacc[dt][4 * g4 + 1]),
+                                   pack2bf(dvacc[dt][4 * g4 + 2], dvacc[dt][4 * g4 + 3])};
+                *reinterpret_cast<u32x2 *>(pk + dt * 32 + 8 * g4) = wk;
+                *reinterpret_cast<u32x2 *>(pv_ + dt * 32 + 8 * g4) = wvv;
+            }
+    }
+}
+
+// ==================================================================================================
+// launchers
+// ==================================================================================================
+static inline void group_shape(int Hq, int Hkv, int &Gp, int &gshift) {
+    const int G = Hq / Hkv;
+    gshift = 0;
+    while ((1 << gshift) < G) ++gshift;
+    Gp = 1 << gshift;
+}
+
+template <int D>
+static hipError_t launch_tile_fwd(const void *q, const void *k, const void *v, const uint32_t *bitmap, int ldw,
+                                  const int32_t *cu, int N, int T, int Hq, int Hkv, float scale, int pos_split,
+                                  void *out, float *lse, hipStream_t stream) {
+    int Gp, gshift;
+    group_shape(Hq, Hkv, Gp, gshift);
+    const int QBW = 128 >> gshift;
+    const dim3 grid((unsigned)(((int64_t)T / QBW + N + 1) * Hkv));
+    if (bitmap)
+        hipLaunchKernelGGL((dsa_tile_fwd_kernel<D, true>), grid, dim3(256), 0, stream, (const bf16_t *)q,
+                           (const bf16_t *)k, (const bf16_t *)v, bitmap, ldw, cu, N, T, Hq, Hkv, Gp, gshift,
+                           scale * LOG2E_F, pos_split, (bf16_t *)out, lse);
+    else
+        hipLaunchKernelGGL((dsa_tile_fwd_kernel<D, false>), grid, dim3(256), 0, stream, (const bf16_t *)q,
+                           (const bf16_t *)k, (const bf16_t *)v, bitmap, ldw, cu, N, T, Hq, Hkv, Gp, gshift,
+                           scale * LOG2E_F, pos_split, (bf16_t *)out, lse);
+    return hipGetLastError();
+}
+
+template <int D>
+static hipError_t launch_tile_dq(const void *dout, const void *q, const void *k, const void *v, const float *lse,
+                                 const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T,
+                                 int Hq, int Hkv, float scale, int pos_split, void *dq, hipStream_t stream) {
+    int Gp, gshift;
+    group_shape(Hq, Hkv, Gp, gshift);
+    const int QBW = 128 >> gshift;
+    const dim3 grid((unsigned)(((int64_t)T / QBW + N + 1) * Hkv));
+    if (bitmap)
+        hipLaunchKernelGGL((dsa_tile_dq_kernel<D, true>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
+                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T,
+                           Hq, Hkv, Gp, gshift, scale, pos_split, (bf16_t *)dq);
+    else
+        hipLaunchKernelGGL((dsa_tile_dq_kernel<D, false>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
+                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T,
+                           Hq, Hkv, Gp, gshift, scale, pos_split, (bf16_t *)dq);
+    return hipGetLastError();
+}
+
+template <int D>
+static hipError_t launch_tile_dkv(const void *dout, const void *q, const void *k, const void *v, const float *lse,
+                                  const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T,
+                                  int Hq, int Hkv, float scale, void *dk, void *dv, hipStream_t stream) {
+    int Gp, gshift;
+    group_shape(Hq, Hkv, Gp, gshift);
+    const dim3 grid((unsigned)(((int64_t)T / 128 + N + 1) * Hkv));
+    if (bitmap)
+        hipLaunchKernelGGL((dsa_tile_dkv_kernel<D, true>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
+                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T,
+                           Hq, Hkv, Gp, gshift, scale, (bf16_t *)dk, (bf16_t *)dv);
+    else
+        hipLaunchKernelGGL((dsa_tile_dkv_kernel<D, false>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
+                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T,
+                           Hq, Hkv, Gp, gshift, scale, (bf16_t *)dk, (bf16_t *)dv);
+    return hipGetLastError();
+}
+
+#define TILE_DISPATCH(fn, ...)                    \
+    switch (D) {                                  \
+        case 64: return fn<64>(__VA_ARGS__);      \
+        case 128: return fn<128>(__VA_ARGS__);    \
+        case 256: return fn<256>(__VA_ARGS__);    \
+        default: return hipErrorInvalidValue;     \
+    }
+
+extern "C" hipError_t dsa_launch_tile_fwd(const void *q, const void *k, const void *v, const uint32_t *bitmap, int ldw,
+                                          const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale,
+                                          int pos_split, void *out, float *lse, hipStream_t stream) {
+    TILE_DISPATCH(launch_tile_fwd, q, k, v, bitmap, ldw, cu, N, T, Hq, Hkv, scale, pos_split, out, lse, stream)
+}
+extern "C" hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const void *k, const void *v,
+                                         const float *lse, const float *delta, const uint32_t *bitmap, int ldw,
+                                         const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale,
+                                         int pos_split, void *dq, hipStream_t stream) {
+    TILE_DISPATCH(launch_tile_dq, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, pos_split, dq, stream)
+}
+extern "C" hipError_t dsa_launch_tile_dkv(const void *dout, const void *q, const void *k, const void *v,
+                                          const float *lse, const float *delta, const uint32_t *bitmap, int ldw,
+                                          const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale, void *dk,
+                                          void *dv, hipStream_t stream) {
+    TILE_DISPATCH(launch_tile_dkv, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, dk, dv, stream)
+}

@@ -119,15 +119,27 @@ def index_topk(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen: int, top_k: int,
     return idx, n
 
 
-def attn_fwd(q, k, v, idx, n, cu_seqlens, softmax_scale: float):
+def set_tile_crossover(crossover: int) -> int:
+    """Rows with pos < top_k * crossover use the MFMA tile kernels, later rows the gather kernels.
+    Returns the previous value (tests use it to drive each path on its own)."""
+    lib = _lib.load()
+    old = lib.dsa_get_tile_crossover()
+    _lib.check(lib.dsa_set_tile_crossover(int(crossover)), "dsa_set_tile_crossover")
+    return old
+
+
+def attn_fwd(q, k, v, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float):
     T, Hq, Hkv, D = _check_qkv(q, k, v)
     cu = _check_cu(cu_seqlens, T)
     out = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=q.device)
     lse = torch.empty((Hq, T), dtype=torch.float32, device=q.device)
     K = idx.shape[1] if idx is not None else 0
     lib = _lib.load()
+    ws_bytes = lib.dsa_attn_fwd_workspace_bytes(T, max_seqlen, 1 if idx is not None else 0)
+    ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q.device)
     rc = lib.dsa_attn_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(idx), _ptr(n), _ptr(cu), T, cu.numel() - 1, Hq, Hkv, D, K,
-                          softmax_scale, _lib.DSA_DTYPE_BF16, _ptr(out), _ptr(lse), _stream(q.device))
+                          softmax_scale, _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
+                          _stream(q.device))
     _lib.check(rc, "dsa_attn_fwd")
     return out, lse
 
@@ -187,7 +199,7 @@ class _DsaVarlenAttn(torch.autograd.Function):
             qb, kb, vb = _stack((qh, ql, qh), D), _stack((kh, kh, kl), D), _stack((vh, vl, vh), D)
         else:
             qb, kb, vb = _as_bf16(q), _as_bf16(k), _as_bf16(v)
-        out, lse = attn_fwd(qb, kb, vb, idx, n, cu_seqlens, softmax_scale)
+        out, lse = attn_fwd(qb, kb, vb, idx, n, cu_seqlens, int(max_seqlen), softmax_scale)
         ctx.save_for_backward(qb, kb, vb, out, lse, cu_seqlens, *(() if idx is None else (idx, n)))
         ctx.has_idx = idx is not None
         ctx.max_seqlen = int(max_seqlen)
