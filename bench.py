@@ -135,21 +135,22 @@ def main():
 
     # ---- roofline ----------------------------------------------------------------------------
     wk = w.work()
-    e = 2
-    qo_bytes = w.T * 2 * w.Hq * w.D * e
-    kern = {   # algorithmic bytes per launch of the gather kernels (HBM-bound rows of the plan)
-        "attn_fwd": wk["B3_gather"] + qo_bytes,                                     # K,V rows + q in + o out
-        "bwd_dq": wk["B3_gather"] + w.T * 3 * w.Hq * w.D * e,                       # K,V rows + q,dO in + dq out
+    S = wk["S"]
+    unit = w.Hq * w.D * S                 # one flop-unit: a multiply-add pass over every selected (query, key, head, d)
+    kern = {   # algorithmic flop per launch of the three attention kernels (selected pairs only)
+        "attn_fwd": ("dsa_tile_fwd_kernel", 4 * unit),          # QK^T + PV
+        "bwd_dq": ("dsa_tile_dq_kernel", 6 * unit),             # QK^T + dO V^T + dS K
+        "bwd_dkv": ("dsa_tile_dkv_kernel", 8 * unit),           # QK^T + dO V^T + P^T dO + dS^T Q
     }
     dom = max(kern, key=lambda name: stage_ms[name])
-    achieved = kern[dom] / (stage_ms[dom] * 1e-3) / 1e9
+    dom_kernel, dom_flop = kern[dom]
+    achieved = dom_flop / (stage_ms[dom] * 1e-3) / 1e12
     t_roof_ms = {
         "index_topk": max(wk["F1"] / (PEAK_MFMA_BF16_TFLOPS * 1e12), wk["B2"] / (PEAK_HBM_GBS * 1e9)) * 1e3,
         "attn_fwd": max(wk["F3"] / (PEAK_MFMA_BF16_TFLOPS * 1e12), wk["B3"] / (PEAK_HBM_GBS * 1e9)) * 1e3,
         "attn_bwd": max(wk["F4"] / (PEAK_MFMA_BF16_TFLOPS * 1e12), wk["B4"] / (PEAK_HBM_GBS * 1e9)) * 1e3,
     }
     roof_total = sum(t_roof_ms.values())
-    dom_kernel = "dsa_attn_fwd_kernel" if dom == "attn_fwd" else "dsa_bwd_dq_kernel"
     traffic = None      # HBM bytes per launch as last measured with rocprofv3 --pmc (separate runs)
     try:
         with open(os.path.join(ROOT, "profiles", f"hbm_traffic_{args.workload}.json")) as fh:
@@ -163,9 +164,9 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{w.name}: T={w.T} packed tokens, segments={list(w.seg_lens)}, Hq/Hkv/D={w.Hq}/{w.Hkv}/{w.D}, "
                                f"indexer {w.Hi}x{w.Di}, top_k={w.top_k}, fwd+bwd"},
-        "roofline": {"bound": "hbm", "kernel": dom_kernel,
-                     "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS,
-                     "traffic": traffic, "algorithmic_bytes": kern[dom], "avg_ms": stage_ms[dom]},
+        "roofline": {"bound": "mfma", "kernel": dom_kernel, "achieved": achieved, "peak": PEAK_MFMA_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_BF16_TFLOPS, "traffic": traffic,
+                     "algorithmic_flop": dom_flop, "avg_ms": stage_ms[dom]},
         "stage_ms": stage_ms,
         "roofline_whole_op": {"t_roof_ms": t_roof_ms, "sum_ms": roof_total, "frac": roof_total / ms_per_step,
                               "compute_only_bound_ms": (wk["F1"] + 3.5 * wk["F3"]) / (PEAK_MFMA_BF16_TFLOPS * 1e12) * 1e3},

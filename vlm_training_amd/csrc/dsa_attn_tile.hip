@@ -43,6 +43,8 @@ __device__ __forceinline__ bf16x8 tile_trop(const unsigned char *tile, int R0, i
     const s16x8 r = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
     return __builtin_bit_cast(bf16x8, r);
 }
+// accumulate in place (kept as a function so that the accumulation sites read alike)
+__device__ __forceinline__ void mfma32_acc(f32x16 &c, bf16x8 a, bf16x8 b) { c = mfma32(a, b, c); }
 __device__ __forceinline__ bf16x8 pack8(const float *x) {
     const u32x4 w = {pack2bf(x[0], x[1]), pack2bf(x[2], x[3]), pack2bf(x[4], x[5]), pack2bf(x[6], x[7])};
     return __builtin_bit_cast(bf16x8, w);
@@ -80,19 +82,46 @@ __device__ __forceinline__ bool locate_block(const int32_t *cu, int N, int slot,
 //   S^T[key,row] = K[key,:].Q[row,:]   (A = K tile row-wise from LDS, B = Q^T in registers)
 //   online softmax on the C layout (lane = row; one cross-lane step per statistic)
 //   O^T[d,row]  += V^T[d,key] P^T[key,row]   (A = V tile transposed from LDS, B = P^T from the C layout)
+// K/V tiles are fetched two tiles ahead into registers and one tile ahead into LDS (double buffer),
+// so a global load has two tile-times to land; one barrier per tile.
 // ==================================================================================================
-template <int D, bool HAS_IDX>
+#define TILE_PIPELINE(NT, LOAD, STORE, COMPUTE)                                                     \
+    {                                                                                              \
+        LOAD(0, 0);                                                                                \
+        STORE(0, 0);                                                                               \
+        if ((NT) > 1) LOAD(0, 1);                                                                  \
+        if ((NT) > 2) LOAD(1, 2);                                                                  \
+        __syncthreads();                                                                           \
+        for (int it = 0; it < (NT); it += 2) {                                                     \
+            /* even tile: LDS buffer 0 holds tile it, register set 0 tile it+1, set 1 tile it+2 */   \
+            COMPUTE(it, 0);                                                                        \
+            if (NBUF == 1) __syncthreads();                                                        \
+            if (it + 1 < (NT)) STORE(0, NBUF - 1);                                                 \
+            if (it + 3 < (NT)) LOAD(0, it + 3);                                                    \
+            __syncthreads();                                                                       \
+            if (it + 1 < (NT)) {                                                                   \
+                COMPUTE(it + 1, NBUF - 1);                                                         \
+                if (NBUF == 1) __syncthreads();                                                    \
+                if (it + 2 < (NT)) STORE(1, 0);                                                    \
+                if (it + 4 < (NT)) LOAD(1, it + 4);                                                \
+                __syncthreads();                                                                   \
+            }                                                                                      \
+        }                                                                                          \
+    }
+
+template <int D, bool HAS_IDX, int GSHIFT>
 __global__ __launch_bounds__(256) void dsa_tile_fwd_kernel(
     const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
-    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv, int Gp,
-    int gshift, float scale_log2, int pos_split, bf16_t *__restrict__ out, float *__restrict__ lse) {
+    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
+    float scale_log2, int pos_split, bf16_t *__restrict__ out, float *__restrict__ lse) {
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2, LOADS = 32 * CPR / 256;
     constexpr int NBUF = (D > 128) ? 1 : 2;           // double buffering where 64 KiB of static LDS allow it
+    constexpr int Gp = 1 << GSHIFT, QBW = 128 >> GSHIFT;
     static_assert(LOADS >= 1, "tile must give every thread a chunk");
     __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];   // [buffer][K|V]
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
-    const int G = Hq / Hkv, QBW = 128 >> gshift;
+    const int G = Hq / Hkv;
     const int kvh = blockIdx.x % Hkv;
     int s0, L, blk;
     if (!locate_block(cu, N, blockIdx.x / Hkv, QBW, true, s0, L, blk)) return;
@@ -100,85 +129,80 @@ __global__ __launch_bounds__(256) void dsa_tile_fwd_kernel(
     if (qc0 >= pos_split) return;                       // rows past the split belong to the gather kernel
 
     const int r = wv * 32 + j;
-    const int qcol = qc0 + (r >> gshift), head = r & (Gp - 1);
+    const int qcol = qc0 + (r >> GSHIFT), head = r & (Gp - 1);
     const bool row_ok = qcol < L && head < G;
     const int t = s0 + min(qcol, L - 1), hq = kvh * G + min(head, G - 1);
     bf16x8 qB[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
         qB[ks] = row_ok ? load_bf16x8(q + ((int64_t)t * Hq + hq) * D + 16 * ks + 8 * h) : zero_bf16x8();
-    const int wq_last = min(qc0 + ((wv * 32 + 31) >> gshift), L - 1);
     const int ntiles = min(qc0 + QBW - 1, L - 1) / 32 + 1;
+    const uint32_t *wrow = bitmap + (int64_t)t * ldw;
 
-    u32x4 kst[LOADS], vst[LOADS];
-    auto load_tile = [&](int kc0) {
-#pragma unroll
-        for (int i = 0; i < LOADS; ++i) {
-            const int c = i * 256 + tid;
-            const int row = c / CPR, ch = c % CPR;
-            const int64_t off = ((int64_t)(s0 + min(kc0 + row, L - 1)) * Hkv + kvh) * D + ch * 8;
-            kst[i] = *reinterpret_cast<const u32x4 *>(k + off);
-            vst[i] = *reinterpret_cast<const u32x4 *>(v + off);
-        }
-    };
-    auto store_tile = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < LOADS; ++i) {
-            const int c = i * 256 + tid;
-            const int row = c / CPR, ch = c % CPR;
-            *reinterpret_cast<u32x4 *>(&lds[buf][0][tile_off<D>(row, ch)]) = kst[i];
-            *reinterpret_cast<u32x4 *>(&lds[buf][1][tile_off<D>(row, ch)]) = vst[i];
-        }
-    };
-
+    u32x4 kst[2][LOADS], vst[2][LOADS];
     f32x16 oacc[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) oacc[dt] = zero16();
     float mrun = -INFINITY, lsum = 0.f;
+    uint32_t word_next = (HAS_IDX && row_ok) ? wrow[0] : 0u;
 
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
-    for (int it = 0; it < ntiles; ++it) {
-        const int kc0 = it * 32;
-        if (it + 1 < ntiles) load_tile(kc0 + 32);
-        uint32_t word = 0u;
-        if (HAS_IDX && row_ok) word = bitmap[(int64_t)t * ldw + it];
-        if (kc0 <= wq_last) {                            // wave-uniform: tile not entirely above the diagonal
-            const unsigned char *kt = lds[it & (NBUF - 1)][0], *vt = lds[it & (NBUF - 1)][1];
-            f32x16 sacc = zero16();
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) sacc = mfma32(tile_rowop<D>(kt, j, ks, h), qB[ks], sacc);
-            float s2[16], mloc = -INFINITY;
-#pragma unroll
-            for (int vi = 0; vi < 16; ++vi) {
-                const int kk = c_row(vi, h);
-                const bool on = HAS_IDX ? ((word >> kk) & 1u) : (row_ok && kc0 + kk <= qcol);
-                s2[vi] = on ? sacc[vi] * scale_log2 : -INFINITY;
-                mloc = fmaxf(mloc, s2[vi]);
-            }
-            mloc = fmaxf(mloc, wave_xor_f(mloc, 32));
-            const float mnew = fmaxf(mrun, mloc);
-            const float mref = (mnew == -INFINITY) ? 0.f : mnew;     // rows with nothing selected so far
-            const float alpha = fast_exp2(mrun - mref);
-            float psum = 0.f;
-#pragma unroll
-            for (int vi = 0; vi < 16; ++vi) { s2[vi] = fast_exp2(s2[vi] - mref); psum += s2[vi]; }
-            lsum = lsum * alpha + psum;
-            mrun = mnew;
-            const bf16x8 pB0 = pack8(s2), pB1 = pack8(s2 + 8);
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                oacc[dt] *= alpha;
-                const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;
-                oacc[dt] = mfma32(tile_trop<D>(vt, 4 * h, m0, lane), pB0, oacc[dt]);
-                oacc[dt] = mfma32(tile_trop<D>(vt, 16 + 4 * h, m0, lane), pB1, oacc[dt]);
-            }
-        }
-        if (NBUF == 1) __syncthreads();                   // single buffer: everyone is done reading it
-        if (it + 1 < ntiles) store_tile((it + 1) & (NBUF - 1));
-        __syncthreads();
+#define FWD_LOAD(SET, TILE)                                                                         \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+        const int c = i * 256 + tid;                                                               \
+        const int row = c / CPR, ch = c % CPR;                                                     \
+        const int64_t off = ((int64_t)(s0 + min((TILE) * 32 + row, L - 1)) * Hkv + kvh) * D + ch * 8; \
+        kst[SET][i] = *reinterpret_cast<const u32x4 *>(k + off);                                   \
+        vst[SET][i] = *reinterpret_cast<const u32x4 *>(v + off);                                   \
     }
+#define FWD_STORE(SET, BUF)                                                                         \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+        const int c = i * 256 + tid;                                                               \
+        const int row = c / CPR, ch = c % CPR;                                                     \
+        *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(row, ch)]) = kst[SET][i];              \
+        *reinterpret_cast<u32x4 *>(&lds[BUF][1][tile_off<D>(row, ch)]) = vst[SET][i];              \
+    }
+#define FWD_COMPUTE(TILE, BUF)                                                                      \
+    {                                                                                              \
+        const int kc0 = (TILE) * 32;                                                               \
+        const unsigned char *kt = lds[BUF][0], *vt = lds[BUF][1];                                  \
+        const uint32_t word = word_next;                                                           \
+        if (HAS_IDX && row_ok && (TILE) + 1 < ntiles) word_next = wrow[(TILE) + 1];                \
+        f32x16 sacc = zero16();                                                                    \
+        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                          \
+            sacc = mfma32(tile_rowop<D>(kt, j, ks, h), qB[ks], sacc);                              \
+        float s2[16], mloc = -INFINITY;                                                            \
+        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
+            const int kk = c_row(vi, h);                                                           \
+            const bool on = HAS_IDX ? ((word >> kk) & 1u) : (row_ok && kc0 + kk <= qcol);          \
+            s2[vi] = on ? sacc[vi] * scale_log2 : -INFINITY;                                       \
+            mloc = fmaxf(mloc, s2[vi]);                                                            \
+        }                                                                                          \
+        mloc = fmaxf(mloc, wave_xor_f(mloc, 32));                                                  \
+        const float mnew = fmaxf(mrun, mloc);                                                      \
+        const float mref = (mnew == -INFINITY) ? 0.f : mnew; /* rows with nothing selected so far */ \
+        const float alpha = fast_exp2(mrun - mref);                                                \
+        float psum = 0.f;                                                                          \
+        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
+            s2[vi] = fast_exp2(s2[vi] - mref);                                                     \
+            psum += s2[vi];                                                                        \
+        }                                                                                          \
+        lsum = lsum * alpha + psum;                                                                \
+        if (__builtin_amdgcn_ballot_w64(mnew != mrun)) { /* some row's maximum moved: rescale */     \
+            _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) oacc[dt] *= alpha;                   \
+        }                                                                                          \
+        mrun = mnew;                                                                               \
+        const bf16x8 pB0 = pack8(s2), pB1 = pack8(s2 + 8);                                         \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
+            const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;                                       \
+            mfma32_acc(oacc[dt], tile_trop<D>(vt, 4 * h, m0, lane), pB0);                          \
+            mfma32_acc(oacc[dt], tile_trop<D>(vt, 16 + 4 * h, m0, lane), pB1);                     \
+        }                                                                                          \
+    }
+    TILE_PIPELINE(ntiles, FWD_LOAD, FWD_STORE, FWD_COMPUTE)
+#undef FWD_LOAD
+#undef FWD_STORE
+#undef FWD_COMPUTE
+
     float l = lsum + wave_xor_f(lsum, 32);
     if (row_ok) {
         const float inv = 1.f / l;
@@ -201,18 +225,19 @@ __global__ __launch_bounds__(256) void dsa_tile_fwd_kernel(
 //   dS^T = P^T * (dP^T - delta)  on the C layout
 //   dQ^T[d,row] += K^T[d,key] dS^T[key,row]   (A = K tile transposed, B = dS^T from the C layout)
 // ==================================================================================================
-template <int D, bool HAS_IDX>
+template <int D, bool HAS_IDX, int GSHIFT>
 __global__ __launch_bounds__(256) void dsa_tile_dq_kernel(
     const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
-    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv, int Gp,
-    int gshift, float scale, int pos_split, bf16_t *__restrict__ dq) {
+    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
+    float scale, int pos_split, bf16_t *__restrict__ dq) {
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2, LOADS = 32 * CPR / 256;
     constexpr int NBUF = (D > 128) ? 1 : 2;
+    constexpr int Gp = 1 << GSHIFT, QBW = 128 >> GSHIFT;
     __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
-    const int G = Hq / Hkv, QBW = 128 >> gshift;
+    const int G = Hq / Hkv;
     const int kvh = blockIdx.x % Hkv;
     int s0, L, blk;
     if (!locate_block(cu, N, blockIdx.x / Hkv, QBW, true, s0, L, blk)) return;
@@ -220,7 +245,7 @@ __global__ __launch_bounds__(256) void dsa_tile_dq_kernel(
     if (qc0 >= pos_split) return;
 
     const int r = wv * 32 + j;
-    const int qcol = qc0 + (r >> gshift), head = r & (Gp - 1);
+    const int qcol = qc0 + (r >> GSHIFT), head = r & (Gp - 1);
     const bool row_ok = qcol < L && head < G;
     const int t = s0 + min(qcol, L - 1), hq = kvh * G + min(head, G - 1);
     const float scale_log2 = scale * LOG2E_F;
@@ -233,69 +258,60 @@ __global__ __launch_bounds__(256) void dsa_tile_dq_kernel(
     }
     const float lse2 = lse[(int64_t)hq * T + t] * LOG2E_F;
     const float dlt = delta[(int64_t)hq * T + t];
-    const int wq_last = min(qc0 + ((wv * 32 + 31) >> gshift), L - 1);
     const int ntiles = min(qc0 + QBW - 1, L - 1) / 32 + 1;
+    const uint32_t *wrow = bitmap + (int64_t)t * ldw;
 
-    u32x4 kst[LOADS], vst[LOADS];
-    auto load_tile = [&](int kc0) {
-#pragma unroll
-        for (int i = 0; i < LOADS; ++i) {
-            const int c = i * 256 + tid;
-            const int row = c / CPR, ch = c % CPR;
-            const int64_t off = ((int64_t)(s0 + min(kc0 + row, L - 1)) * Hkv + kvh) * D + ch * 8;
-            kst[i] = *reinterpret_cast<const u32x4 *>(k + off);
-            vst[i] = *reinterpret_cast<const u32x4 *>(v + off);
-        }
-    };
-    auto store_tile = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < LOADS; ++i) {
-            const int c = i * 256 + tid;
-            const int row = c / CPR, ch = c % CPR;
-            *reinterpret_cast<u32x4 *>(&lds[buf][0][tile_off<D>(row, ch)]) = kst[i];
-            *reinterpret_cast<u32x4 *>(&lds[buf][1][tile_off<D>(row, ch)]) = vst[i];
-        }
-    };
+    u32x4 kst[2][LOADS], vst[2][LOADS];
     f32x16 acc[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
+    uint32_t word_next = (HAS_IDX && row_ok) ? wrow[0] : 0u;
 
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
-    for (int it = 0; it < ntiles; ++it) {
-        const int kc0 = it * 32;
-        if (it + 1 < ntiles) load_tile(kc0 + 32);
-        uint32_t word = 0u;
-        if (HAS_IDX && row_ok) word = bitmap[(int64_t)t * ldw + it];
-        if (kc0 <= wq_last) {
-            const unsigned char *kt = lds[it & (NBUF - 1)][0], *vt = lds[it & (NBUF - 1)][1];
-            f32x16 sacc = zero16(), pacc = zero16();
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                sacc = mfma32(tile_rowop<D>(kt, j, ks, h), qB[ks], sacc);
-                pacc = mfma32(tile_rowop<D>(vt, j, ks, h), doB[ks], pacc);
-            }
-            float ds[16];
-#pragma unroll
-            for (int vi = 0; vi < 16; ++vi) {
-                const int kk = c_row(vi, h);
-                const bool on = HAS_IDX ? ((word >> kk) & 1u) : (row_ok && kc0 + kk <= qcol);
-                const float p = on ? fast_exp2(sacc[vi] * scale_log2 - lse2) : 0.f;
-                ds[vi] = p * (pacc[vi] - dlt);
-            }
-            const bf16x8 dB0 = pack8(ds), dB1 = pack8(ds + 8);
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;
-                acc[dt] = mfma32(tile_trop<D>(kt, 4 * h, m0, lane), dB0, acc[dt]);
-                acc[dt] = mfma32(tile_trop<D>(kt, 16 + 4 * h, m0, lane), dB1, acc[dt]);
-            }
-        }
-        if (NBUF == 1) __syncthreads();                   // single buffer: everyone is done reading it
-        if (it + 1 < ntiles) store_tile((it + 1) & (NBUF - 1));
-        __syncthreads();
+#define DQ_LOAD(SET, TILE)                                                                          \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+        const int c = i * 256 + tid;                                                               \
+        const int row = c / CPR, ch = c % CPR;                                                     \
+        const int64_t off = ((int64_t)(s0 + min((TILE) * 32 + row, L - 1)) * Hkv + kvh) * D + ch * 8; \
+        kst[SET][i] = *reinterpret_cast<const u32x4 *>(k + off);                                   \
+        vst[SET][i] = *reinterpret_cast<const u32x4 *>(v + off);                                   \
     }
+#define DQ_STORE(SET, BUF)                                                                          \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+        const int c = i * 256 + tid;                                                               \
+        const int row = c / CPR, ch = c % CPR;                                                     \
+        *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(row, ch)]) = kst[SET][i];              \
+        *reinterpret_cast<u32x4 *>(&lds[BUF][1][tile_off<D>(row, ch)]) = vst[SET][i];              \
+    }
+#define DQ_COMPUTE(TILE, BUF)                                                                       \
+    {                                                                                              \
+        const int kc0 = (TILE) * 32;                                                               \
+        const unsigned char *kt = lds[BUF][0], *vt = lds[BUF][1];                                  \
+        const uint32_t word = word_next;                                                           \
+        if (HAS_IDX && row_ok && (TILE) + 1 < ntiles) word_next = wrow[(TILE) + 1];                \
+        f32x16 sacc = zero16(), pacc = zero16();                                                   \
+        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
+            sacc = mfma32(tile_rowop<D>(kt, j, ks, h), qB[ks], sacc);                              \
+            pacc = mfma32(tile_rowop<D>(vt, j, ks, h), doB[ks], pacc);                             \
+        }                                                                                          \
+        float ds[16];                                                                              \
+        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
+            const int kk = c_row(vi, h);                                                           \
+            const bool on = HAS_IDX ? ((word >> kk) & 1u) : (row_ok && kc0 + kk <= qcol);          \
+            const float p = on ? fast_exp2(sacc[vi] * scale_log2 - lse2) : 0.f;                    \
+            ds[vi] = p * (pacc[vi] - dlt);                                                         \
+        }                                                                                          \
+        const bf16x8 dB0 = pack8(ds), dB1 = pack8(ds + 8);                                         \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
+            const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;                                       \
+            mfma32_acc(acc[dt], tile_trop<D>(kt, 4 * h, m0, lane), dB0);                           \
+            mfma32_acc(acc[dt], tile_trop<D>(kt, 16 + 4 * h, m0, lane), dB1);                      \
+        }                                                                                          \
+    }
+    TILE_PIPELINE(ntiles, DQ_LOAD, DQ_STORE, DQ_COMPUTE)
+#undef DQ_LOAD
+#undef DQ_STORE
+#undef DQ_COMPUTE
+
     if (row_ok) {
         bf16_t *op = dq + ((int64_t)t * Hq + hq) * D + 4 * h;
 #pragma unroll
@@ -313,25 +329,26 @@ __global__ __launch_bounds__(256) void dsa_tile_dq_kernel(
 // dK, dV: key-stationary ("scatter by key": every key row is reduced by exactly one wave, in query
 // order, so the result needs no atomics and is bit-reproducible).  Workgroup = 4 waves x 32 keys = one
 // 128-key tile of a segment and one kv head; walks the queries from the tile's first column to the end
-// of the segment in blocks of 32 (query, head) rows staged in LDS.
+// of the segment in blocks of 32 (query, head) rows staged in LDS (same two-ahead pipeline).
 //   S[row,key] = Q K^T, dP = dO V^T     (A = q / dO block row-wise, B = K^T / V^T in registers)
 //   dV^T[d,key] += dO^T[d,row] P[row,key]   dK^T[d,key] += Q^T[d,row] dS[row,key]
 //                                           (A = dO / q block transposed, B = P / dS from the C layout)
 // ==================================================================================================
-template <int D, bool HAS_IDX>
+template <int D, bool HAS_IDX, int GSHIFT>
 __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
     const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
-    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv, int Gp,
-    int gshift, float scale, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
+    float scale, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2, LOADS = 32 * CPR / 256;
     constexpr int NBUF = (D > 128) ? 1 : 2;
+    constexpr int Gp = 1 << GSHIFT, QB = 32 >> GSHIFT;                           // queries per block
     __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];   // [buffer][q|dO]
-    __shared__ float lse_s[NBUF][32], dlt_s[NBUF][32];
-    __shared__ uint32_t mask_s[NBUF][32][4];                                     // [buffer][query in block][wave]
+    __shared__ __attribute__((aligned(16))) float lse_s[NBUF][32], dlt_s[NBUF][32];
+    __shared__ uint32_t mask_s[NBUF][4][32];                                      // [buffer][wave][query in block]
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
-    const int G = Hq / Hkv, QB = 32 >> gshift;
+    const int G = Hq / Hkv;
     const int kvh = blockIdx.x % Hkv;
     int s0, L, blk;
     if (!locate_block(cu, N, blockIdx.x / Hkv, 128, false, s0, L, blk)) return;
@@ -349,85 +366,87 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) { dkacc[dt] = zero16(); dvacc[dt] = zero16(); }
     const float scale_log2 = scale * LOG2E_F;
-
-    u32x4 qst[LOADS], dost[LOADS];
-    float lse_st = 0.f, dlt_st = 0.f;
-    uint32_t mask_st = 0u;
-    auto load_block = [&](int qc0) {
-#pragma unroll
-        for (int i = 0; i < LOADS; ++i) {
-            const int c = i * 256 + tid;
-            const int row = c / CPR, ch = c % CPR;
-            const int qc = min(qc0 + (row >> gshift), L - 1);
-            const int hd = min(row & (Gp - 1), G - 1);
-            const int64_t off = ((int64_t)(s0 + qc) * Hq + kvh * G + hd) * D + ch * 8;
-            qst[i] = *reinterpret_cast<const u32x4 *>(q + off);
-            dost[i] = *reinterpret_cast<const u32x4 *>(dout + off);
-        }
-        if (tid < 32) {
-            const int qc = min(qc0 + (tid >> gshift), L - 1);
-            const int hd = min(tid & (Gp - 1), G - 1);
-            lse_st = lse[(int64_t)(kvh * G + hd) * T + s0 + qc] * LOG2E_F;
-            dlt_st = delta[(int64_t)(kvh * G + hd) * T + s0 + qc];
-        } else if (HAS_IDX && tid >= 64 && tid < 64 + 4 * QB) {
-            const int qi = (tid - 64) >> 2, w = (tid - 64) & 3;
-            const int qc = qc0 + qi;
-            mask_st = (qc < L && (c0 >> 5) + w < ldw) ? bitmap[(int64_t)(s0 + qc) * ldw + (c0 >> 5) + w] : 0u;
-        }
-    };
-    auto store_block = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < LOADS; ++i) {
-            const int c = i * 256 + tid;
-            const int row = c / CPR, ch = c % CPR;
-            *reinterpret_cast<u32x4 *>(&lds[buf][0][tile_off<D>(row, ch)]) = qst[i];
-            *reinterpret_cast<u32x4 *>(&lds[buf][1][tile_off<D>(row, ch)]) = dost[i];
-        }
-        if (tid < 32) { lse_s[buf][tid] = lse_st; dlt_s[buf][tid] = dlt_st; }
-        else if (HAS_IDX && tid >= 64 && tid < 64 + 4 * QB) mask_s[buf][(tid - 64) >> 2][(tid - 64) & 3] = mask_st;
-    };
-
     const int nblocks = (L - c0 + QB - 1) / QB;          // queries c0 .. L-1
-    load_block(c0);
-    store_block(0);
-    __syncthreads();
-    for (int b = 0; b < nblocks; ++b) {
-        const int qc0 = c0 + b * QB, buf = b & (NBUF - 1);
-        if (b + 1 < nblocks) load_block(qc0 + QB);
-        if (qc0 + QB - 1 >= kc) {                          // wave-uniform: some query of the block sees this wave's keys
-            const unsigned char *qt = lds[buf][0], *dot = lds[buf][1];
-            f32x16 sacc = zero16(), pacc = zero16();
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                sacc = mfma32(tile_rowop<D>(qt, j, ks, h), kB[ks], sacc);
-                pacc = mfma32(tile_rowop<D>(dot, j, ks, h), vB[ks], pacc);
-            }
-            float pv[16], dsv[16];
-#pragma unroll
-            for (int vi = 0; vi < 16; ++vi) {
-                const int row = c_row(vi, h);
-                const int qi = row >> gshift, hd = row & (Gp - 1);
-                const int qc = qc0 + qi;
-                bool on = key_ok && qc < L && hd < G && mykey <= qc;
-                if (HAS_IDX) on = on && ((mask_s[buf][qi][wv] >> j) & 1u);
-                const float p = on ? fast_exp2(sacc[vi] * scale_log2 - lse_s[buf][row]) : 0.f;
-                pv[vi] = p;
-                dsv[vi] = p * (pacc[vi] - dlt_s[buf][row]);
-            }
-            const bf16x8 pB0 = pack8(pv), pB1 = pack8(pv + 8), dB0 = pack8(dsv), dB1 = pack8(dsv + 8);
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;
-                dvacc[dt] = mfma32(tile_trop<D>(dot, 4 * h, m0, lane), pB0, dvacc[dt]);
-                dvacc[dt] = mfma32(tile_trop<D>(dot, 16 + 4 * h, m0, lane), pB1, dvacc[dt]);
-                dkacc[dt] = mfma32(tile_trop<D>(qt, 4 * h, m0, lane), dB0, dkacc[dt]);
-                dkacc[dt] = mfma32(tile_trop<D>(qt, 16 + 4 * h, m0, lane), dB1, dkacc[dt]);
-            }
-        }
-        if (NBUF == 1) __syncthreads();
-        if (b + 1 < nblocks) store_block((b + 1) & (NBUF - 1));
-        __syncthreads();
+
+    u32x4 qst[2][LOADS], dost[2][LOADS];
+    float aux_st[2] = {0.f, 0.f};                        // lse / delta / mask word of the staging threads
+    // threads 0..31: lse of row tid; 32..63: delta of row tid-32; 64..64+4*QB-1: mask word (wave w, query qi)
+#define DKV_LOAD(SET, BLK)                                                                          \
+    {                                                                                              \
+        const int qcb = c0 + (BLK) * QB;                                                           \
+        _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                        \
+            const int c = i * 256 + tid;                                                           \
+            const int row = c / CPR, ch = c % CPR;                                                 \
+            const int qc = min(qcb + (row >> GSHIFT), L - 1);                                      \
+            const int hd = min(row & (Gp - 1), G - 1);                                             \
+            const int64_t off = ((int64_t)(s0 + qc) * Hq + kvh * G + hd) * D + ch * 8;             \
+            qst[SET][i] = *reinterpret_cast<const u32x4 *>(q + off);                               \
+            dost[SET][i] = *reinterpret_cast<const u32x4 *>(dout + off);                           \
+        }                                                                                          \
+        if (tid < 64) {                                                                            \
+            const int row = tid & 31;                                                              \
+            const int qc = min(qcb + (row >> GSHIFT), L - 1);                                      \
+            const int hd = min(row & (Gp - 1), G - 1);                                             \
+            const int64_t o = (int64_t)(kvh * G + hd) * T + s0 + qc;                               \
+            aux_st[SET] = (tid < 32) ? lse[o] * LOG2E_F : delta[o];                                \
+        } else if (HAS_IDX && tid < 64 + 4 * QB) {                                                 \
+            const int w = (tid - 64) / QB, qi = (tid - 64) % QB;                                   \
+            const int qc = qcb + qi;                                                               \
+            const uint32_t m = (qc < L && (c0 >> 5) + w < ldw) ? bitmap[(int64_t)(s0 + qc) * ldw + (c0 >> 5) + w] : 0u; \
+            aux_st[SET] = __uint_as_float(m);                                                      \
+        }                                                                                          \
     }
+#define DKV_STORE(SET, BUF)                                                                         \
+    {                                                                                              \
+        _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                        \
+            const int c = i * 256 + tid;                                                           \
+            const int row = c / CPR, ch = c % CPR;                                                 \
+            *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(row, ch)]) = qst[SET][i];          \
+            *reinterpret_cast<u32x4 *>(&lds[BUF][1][tile_off<D>(row, ch)]) = dost[SET][i];         \
+        }                                                                                          \
+        if (tid < 32) lse_s[BUF][tid] = aux_st[SET];                                               \
+        else if (tid < 64) dlt_s[BUF][tid - 32] = aux_st[SET];                                     \
+        else if (HAS_IDX && tid < 64 + 4 * QB) mask_s[BUF][(tid - 64) / QB][(tid - 64) % QB] = __float_as_uint(aux_st[SET]); \
+    }
+#define DKV_COMPUTE(BLK, BUF)                                                                       \
+    {                                                                                              \
+        const int qcb = c0 + (BLK) * QB;                                                           \
+        const unsigned char *qt = lds[BUF][0], *dot = lds[BUF][1];                                 \
+        f32x16 sacc = zero16(), pacc = zero16();                                                   \
+        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
+            sacc = mfma32(tile_rowop<D>(qt, j, ks, h), kB[ks], sacc);                              \
+            pacc = mfma32(tile_rowop<D>(dot, j, ks, h), vB[ks], pacc);                             \
+        }                                                                                          \
+        float pv[16], dsv[16];                                                                     \
+        _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {                                         \
+            const f32x4 l4 = *reinterpret_cast<const f32x4 *>(&lse_s[BUF][8 * g4 + 4 * h]);        \
+            const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&dlt_s[BUF][8 * g4 + 4 * h]);        \
+            _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                        \
+                const int vi = 4 * g4 + e, row = 8 * g4 + 4 * h + e;                               \
+                const int qi = row >> GSHIFT, hd = row & (Gp - 1);                                 \
+                const int qc = qcb + qi;                                                           \
+                const uint32_t mw = HAS_IDX ? mask_s[BUF][wv][qi] : 0xffffffffu;                   \
+                const int on = (int)key_ok & (int)(qc < L) & (int)(hd < G) & (int)(mykey <= qc) &  \
+                               (int)((mw >> j) & 1u);                 /* branch-free */             \
+                const float p = fast_exp2(on ? sacc[vi] * scale_log2 - l4[e] : -INFINITY);         \
+                pv[vi] = p;                                                                        \
+                dsv[vi] = p * (pacc[vi] - d4[e]);                                                  \
+            }                                                                                      \
+        }                                                                                          \
+        const bf16x8 pB0 = pack8(pv), pB1 = pack8(pv + 8), dB0 = pack8(dsv), dB1 = pack8(dsv + 8); \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
+            const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;                                       \
+            mfma32_acc(dvacc[dt], tile_trop<D>(dot, 4 * h, m0, lane), pB0);                        \
+            mfma32_acc(dvacc[dt], tile_trop<D>(dot, 16 + 4 * h, m0, lane), pB1);                   \
+            mfma32_acc(dkacc[dt], tile_trop<D>(qt, 4 * h, m0, lane), dB0);                         \
+            mfma32_acc(dkacc[dt], tile_trop<D>(qt, 16 + 4 * h, m0, lane), dB1);                    \
+        }                                                                                          \
+    }
+    TILE_PIPELINE(nblocks, DKV_LOAD, DKV_STORE, DKV_COMPUTE)
+#undef DKV_LOAD
+#undef DKV_STORE
+#undef DKV_COMPUTE
+
     if (key_ok) {
         bf16_t *pk = dk + krow * D + 4 * h, *pv_ = dv + krow * D + 4 * h;
 #pragma unroll
@@ -445,93 +464,78 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
 }
 
 // ==================================================================================================
-// launchers
+// launchers: instantiate per head_dim, mask kind and (power-of-two padded) group size
 // ==================================================================================================
-static inline void group_shape(int Hq, int Hkv, int &Gp, int &gshift) {
+static inline int group_shift(int Hq, int Hkv) {
     const int G = Hq / Hkv;
-    gshift = 0;
+    int gshift = 0;
     while ((1 << gshift) < G) ++gshift;
-    Gp = 1 << gshift;
+    return gshift;
 }
 
-template <int D>
-static hipError_t launch_tile_fwd(const void *q, const void *k, const void *v, const uint32_t *bitmap, int ldw,
-                                  const int32_t *cu, int N, int T, int Hq, int Hkv, float scale, int pos_split,
-                                  void *out, float *lse, hipStream_t stream) {
-    int Gp, gshift;
-    group_shape(Hq, Hkv, Gp, gshift);
-    const int QBW = 128 >> gshift;
-    const dim3 grid((unsigned)(((int64_t)T / QBW + N + 1) * Hkv));
-    if (bitmap)
-        hipLaunchKernelGGL((dsa_tile_fwd_kernel<D, true>), grid, dim3(256), 0, stream, (const bf16_t *)q,
-                           (const bf16_t *)k, (const bf16_t *)v, bitmap, ldw, cu, N, T, Hq, Hkv, Gp, gshift,
-                           scale * LOG2E_F, pos_split, (bf16_t *)out, lse);
-    else
-        hipLaunchKernelGGL((dsa_tile_fwd_kernel<D, false>), grid, dim3(256), 0, stream, (const bf16_t *)q,
-                           (const bf16_t *)k, (const bf16_t *)v, bitmap, ldw, cu, N, T, Hq, Hkv, Gp, gshift,
-                           scale * LOG2E_F, pos_split, (bf16_t *)out, lse);
-    return hipGetLastError();
+template <int D, bool HAS_IDX, int GS>
+static void launch_fwd_i(dim3 grid, hipStream_t stream, const void *q, const void *k, const void *v,
+                         const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T, int Hq, int Hkv, float sl2,
+                         int pos_split, void *out, float *lse) {
+    hipLaunchKernelGGL((dsa_tile_fwd_kernel<D, HAS_IDX, GS>), grid, dim3(256), 0, stream, (const bf16_t *)q,
+                       (const bf16_t *)k, (const bf16_t *)v, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, pos_split, (bf16_t *)out, lse);
+}
+template <int D, bool HAS_IDX, int GS>
+static void launch_dq_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
+                        const float *lse, const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N,
+                        int T, int Hq, int Hkv, float scale, int pos_split, void *dq) {
+    hipLaunchKernelGGL((dsa_tile_dq_kernel<D, HAS_IDX, GS>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
+                       (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv,
+                       scale, pos_split, (bf16_t *)dq);
+}
+template <int D, bool HAS_IDX, int GS>
+static void launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
+                         const float *lse, const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N,
+                         int T, int Hq, int Hkv, float scale, void *dk, void *dv) {
+    hipLaunchKernelGGL((dsa_tile_dkv_kernel<D, HAS_IDX, GS>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
+                       (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv,
+                       scale, (bf16_t *)dk, (bf16_t *)dv);
 }
 
-template <int D>
-static hipError_t launch_tile_dq(const void *dout, const void *q, const void *k, const void *v, const float *lse,
-                                 const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T,
-                                 int Hq, int Hkv, float scale, int pos_split, void *dq, hipStream_t stream) {
-    int Gp, gshift;
-    group_shape(Hq, Hkv, Gp, gshift);
-    const int QBW = 128 >> gshift;
-    const dim3 grid((unsigned)(((int64_t)T / QBW + N + 1) * Hkv));
-    if (bitmap)
-        hipLaunchKernelGGL((dsa_tile_dq_kernel<D, true>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
-                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T,
-                           Hq, Hkv, Gp, gshift, scale, pos_split, (bf16_t *)dq);
-    else
-        hipLaunchKernelGGL((dsa_tile_dq_kernel<D, false>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
-                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T,
-                           Hq, Hkv, Gp, gshift, scale, pos_split, (bf16_t *)dq);
-    return hipGetLastError();
-}
-
-template <int D>
-static hipError_t launch_tile_dkv(const void *dout, const void *q, const void *k, const void *v, const float *lse,
-                                  const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T,
-                                  int Hq, int Hkv, float scale, void *dk, void *dv, hipStream_t stream) {
-    int Gp, gshift;
-    group_shape(Hq, Hkv, Gp, gshift);
-    const dim3 grid((unsigned)(((int64_t)T / 128 + N + 1) * Hkv));
-    if (bitmap)
-        hipLaunchKernelGGL((dsa_tile_dkv_kernel<D, true>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
-                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T,
-                           Hq, Hkv, Gp, gshift, scale, (bf16_t *)dk, (bf16_t *)dv);
-    else
-        hipLaunchKernelGGL((dsa_tile_dkv_kernel<D, false>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
-                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T,
-                           Hq, Hkv, Gp, gshift, scale, (bf16_t *)dk, (bf16_t *)dv);
-    return hipGetLastError();
-}
-
-#define TILE_DISPATCH(fn, ...)                    \
-    switch (D) {                                  \
-        case 64: return fn<64>(__VA_ARGS__);      \
-        case 128: return fn<128>(__VA_ARGS__);    \
-        case 256: return fn<256>(__VA_ARGS__);    \
-        default: return hipErrorInvalidValue;     \
+#define GS_SWITCH(FN, DD, HI, ...)                                    \
+    switch (gs) {                                                     \
+        case 0: FN<DD, HI, 0>(__VA_ARGS__); break;                    \
+        case 1: FN<DD, HI, 1>(__VA_ARGS__); break;                    \
+        case 2: FN<DD, HI, 2>(__VA_ARGS__); break;                    \
+        case 3: FN<DD, HI, 3>(__VA_ARGS__); break;                    \
+        default: FN<DD, HI, 4>(__VA_ARGS__); break;                   \
+    }
+#define TILE_SWITCH(FN, ...)                                                              \
+    switch (D) {                                                                          \
+        case 64: if (bitmap) { GS_SWITCH(FN, 64, true, __VA_ARGS__) } else { GS_SWITCH(FN, 64, false, __VA_ARGS__) } break;    \
+        case 128: if (bitmap) { GS_SWITCH(FN, 128, true, __VA_ARGS__) } else { GS_SWITCH(FN, 128, false, __VA_ARGS__) } break; \
+        case 256: if (bitmap) { GS_SWITCH(FN, 256, true, __VA_ARGS__) } else { GS_SWITCH(FN, 256, false, __VA_ARGS__) } break; \
+        default: return hipErrorInvalidValue;                                             \
     }
 
 extern "C" hipError_t dsa_launch_tile_fwd(const void *q, const void *k, const void *v, const uint32_t *bitmap, int ldw,
                                           const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale,
                                           int pos_split, void *out, float *lse, hipStream_t stream) {
-    TILE_DISPATCH(launch_tile_fwd, q, k, v, bitmap, ldw, cu, N, T, Hq, Hkv, scale, pos_split, out, lse, stream)
+    const int gs = group_shift(Hq, Hkv);
+    const dim3 grid((unsigned)(((int64_t)T / (128 >> gs) + N + 1) * Hkv));
+    TILE_SWITCH(launch_fwd_i, grid, stream, q, k, v, bitmap, ldw, cu, N, T, Hq, Hkv, scale * LOG2E_F, pos_split, out, lse)
+    return hipGetLastError();
 }
 extern "C" hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const void *k, const void *v,
                                          const float *lse, const float *delta, const uint32_t *bitmap, int ldw,
                                          const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale,
                                          int pos_split, void *dq, hipStream_t stream) {
-    TILE_DISPATCH(launch_tile_dq, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, pos_split, dq, stream)
+    const int gs = group_shift(Hq, Hkv);
+    const dim3 grid((unsigned)(((int64_t)T / (128 >> gs) + N + 1) * Hkv));
+    TILE_SWITCH(launch_dq_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, pos_split, dq)
+    return hipGetLastError();
 }
 extern "C" hipError_t dsa_launch_tile_dkv(const void *dout, const void *q, const void *k, const void *v,
                                           const float *lse, const float *delta, const uint32_t *bitmap, int ldw,
                                           const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale, void *dk,
                                           void *dv, hipStream_t stream) {
-    TILE_DISPATCH(launch_tile_dkv, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, dk, dv, stream)
+    const int gs = group_shift(Hq, Hkv);
+    const dim3 grid((unsigned)(((int64_t)T / 128 + N + 1) * Hkv));
+    TILE_SWITCH(launch_dkv_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, dk, dv)
+    return hipGetLastError();
 }

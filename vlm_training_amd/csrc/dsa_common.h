@@ -35,15 +35,13 @@ __device__ __forceinline__ bf16x8 load_bf16x8(const bf16_t *p) {   // 16-byte al
     return *reinterpret_cast<const bf16x8 *>(p);
 }
 
-// round-to-nearest-even fp32 -> bf16 bits (finite inputs; NaN stays NaN)
-__device__ __forceinline__ uint32_t f2bf_bits(float x) {
-    uint32_t u = __float_as_uint(x);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return u >> 16;
+// two fp32 -> packed bf16 pair, round-to-nearest-even (one v_cvt_pk_bf16_f32 on gfx950)
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack2bf(float lo, float hi) {
+    const f32x2 f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
 }
-__device__ __forceinline__ uint32_t pack2bf(float lo, float hi) { return f2bf_bits(lo) | (f2bf_bits(hi) << 16); }
-__device__ __forceinline__ float bf_bits2f(uint32_t b) { return __uint_as_float(b << 16); }
 
 // segment lookup: index i with cu[i] <= t < cu[i+1] (zero-length segments are stepped over)
 __device__ __forceinline__ int find_segment(const int32_t *__restrict__ cu, int N, int t) {
