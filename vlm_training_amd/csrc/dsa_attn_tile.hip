@@ -110,7 +110,7 @@ __device__ __forceinline__ bool locate_block(const int32_t *cu, int N, int slot,
     }
 
 template <int D, bool HAS_IDX, int GSHIFT>
-__global__ __launch_bounds__(256) void dsa_tile_fwd_kernel(
+__global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
     const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
     float scale_log2, int pos_split, bf16_t *__restrict__ out, float *__restrict__ lse) {
@@ -226,7 +226,7 @@ __global__ __launch_bounds__(256) void dsa_tile_fwd_kernel(
 //   dQ^T[d,row] += K^T[d,key] dS^T[key,row]   (A = K tile transposed, B = dS^T from the C layout)
 // ==================================================================================================
 template <int D, bool HAS_IDX, int GSHIFT>
-__global__ __launch_bounds__(256) void dsa_tile_dq_kernel(
+__global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
     const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
@@ -464,6 +464,143 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
 }
 
 // ==================================================================================================
+// dK, dV for head_dim <= 128: the same key-stationary walk with 8 waves per workgroup.  Waves 0-3
+// accumulate dV^T for the four 32-key groups of the tile, waves 4-7 accumulate dK^T for the same
+// groups, so one wave holds a single D x 32 fp32 accumulator, everything fits the 256 registers that
+// two waves per SIMD allow, and the softmax arithmetic of one wave overlaps the MFMAs of the other.
+// (S is computed by both roles: 40 MFMAs per 32x32 block pair instead of 32.)
+// ==================================================================================================
+template <int D, bool HAS_IDX, int GSHIFT>
+__global__ __launch_bounds__(512, 1) void dsa_tile_dkv8_kernel(
+    const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
+    const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
+    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
+    float scale, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2;
+    constexpr int NCHUNK = 32 * CPR;                     // 16-byte chunks per staged operand (<= 512 threads)
+    constexpr int NBUF = 2;
+    constexpr int Gp = 1 << GSHIFT, QB = 32 >> GSHIFT;
+    static_assert(NCHUNK <= 512, "one chunk per thread");
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];   // [buffer][q|dO]
+    __shared__ __attribute__((aligned(16))) float lse_s[NBUF][32], dlt_s[NBUF][32];
+    __shared__ uint32_t mask_s[NBUF][4][32];                                      // [buffer][key group][query in block]
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
+    const int kg = wv & 3, role = wv >> 2;               // role 0: dV, role 1: dK
+    const int G = Hq / Hkv;
+    const int kvh = blockIdx.x % Hkv;
+    int s0, L, blk;
+    if (!locate_block(cu, N, blockIdx.x / Hkv, 128, false, s0, L, blk)) return;
+    const int c0 = blk * 128, kc = c0 + kg * 32;
+    const int mykey = kc + j;
+    const bool key_ok = mykey < L;
+    const int64_t krow = (int64_t)(s0 + min(mykey, L - 1)) * Hkv + kvh;
+    bf16x8 kB[KS], vB[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        kB[ks] = load_bf16x8(k + krow * D + 16 * ks + 8 * h);
+        vB[ks] = load_bf16x8(v + krow * D + 16 * ks + 8 * h);
+    }
+    f32x16 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
+    const float scale_log2 = scale * LOG2E_F;
+    const float gamma = role ? 1.f : 0.f;                // B = p * (gamma * dP - delta'), delta' = -1 for the dV role
+    const int nblocks = (L - c0 + QB - 1) / QB;          // queries c0 .. L-1
+    const bool stager = tid < NCHUNK;
+    const int srow = tid / CPR, sch = tid % CPR;
+
+    u32x4 qst[2], dost[2];
+    float aux_st[2] = {0.f, 0.f};
+    // aux staging threads: 0..31 lse of row tid; 32..63 delta of row tid-32; 64..64+4*QB-1 mask words
+#define DKV8_LOAD(SET, BLK)                                                                         \
+    {                                                                                              \
+        const int qcb = c0 + (BLK) * QB;                                                           \
+        if (stager) {                                                                              \
+            const int qc = min(qcb + (srow >> GSHIFT), L - 1);                                     \
+            const int hd = min(srow & (Gp - 1), G - 1);                                            \
+            const int64_t off = ((int64_t)(s0 + qc) * Hq + kvh * G + hd) * D + sch * 8;            \
+            qst[SET] = *reinterpret_cast<const u32x4 *>(q + off);                                  \
+            dost[SET] = *reinterpret_cast<const u32x4 *>(dout + off);                              \
+        }                                                                                          \
+        if (tid < 64) {                                                                            \
+            const int row = tid & 31;                                                              \
+            const int qc = min(qcb + (row >> GSHIFT), L - 1);                                      \
+            const int hd = min(row & (Gp - 1), G - 1);                                             \
+            const int64_t o = (int64_t)(kvh * G + hd) * T + s0 + qc;                               \
+            aux_st[SET] = (tid < 32) ? lse[o] * LOG2E_F : delta[o];                                \
+        } else if (HAS_IDX && tid < 64 + 4 * QB) {                                                 \
+            const int w = (tid - 64) / QB, qi = (tid - 64) % QB;                                   \
+            const int qc = qcb + qi;                                                               \
+            const uint32_t m = (qc < L && (c0 >> 5) + w < ldw) ? bitmap[(int64_t)(s0 + qc) * ldw + (c0 >> 5) + w] : 0u; \
+            aux_st[SET] = __uint_as_float(m);                                                      \
+        }                                                                                          \
+    }
+#define DKV8_STORE(SET, BUF)                                                                        \
+    {                                                                                              \
+        if (stager) {                                                                              \
+            *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(srow, sch)]) = qst[SET];           \
+            *reinterpret_cast<u32x4 *>(&lds[BUF][1][tile_off<D>(srow, sch)]) = dost[SET];          \
+        }                                                                                          \
+        if (tid < 32) lse_s[BUF][tid] = aux_st[SET];                                               \
+        else if (tid < 64) dlt_s[BUF][tid - 32] = aux_st[SET];                                     \
+        else if (HAS_IDX && tid < 64 + 4 * QB) mask_s[BUF][(tid - 64) / QB][(tid - 64) % QB] = __float_as_uint(aux_st[SET]); \
+    }
+#define DKV8_COMPUTE(BLK, BUF)                                                                      \
+    {                                                                                              \
+        const int qcb = c0 + (BLK) * QB;                                                           \
+        const unsigned char *qt = lds[BUF][0], *dot = lds[BUF][1];                                 \
+        const unsigned char *t2 = role ? qt : dot;      /* operand of the second GEMM */            \
+        f32x16 sacc = zero16(), pacc = zero16();                                                   \
+        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                          \
+            sacc = mfma32(tile_rowop<D>(qt, j, ks, h), kB[ks], sacc);                              \
+        if (role) {                                     /* wave-uniform */                          \
+            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                      \
+                pacc = mfma32(tile_rowop<D>(dot, j, ks, h), vB[ks], pacc);                         \
+        }                                                                                          \
+        float bv[16];                                                                              \
+        _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {                                         \
+            const f32x4 l4 = *reinterpret_cast<const f32x4 *>(&lse_s[BUF][8 * g4 + 4 * h]);        \
+            const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&dlt_s[BUF][8 * g4 + 4 * h]);        \
+            _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                        \
+                const int vi = 4 * g4 + e, row = 8 * g4 + 4 * h + e;                               \
+                const int qi = row >> GSHIFT, hd = row & (Gp - 1);                                 \
+                const int qc = qcb + qi;                                                           \
+                const uint32_t mw = HAS_IDX ? mask_s[BUF][kg][qi] : 0xffffffffu;                   \
+                const int on = (int)key_ok & (int)(qc < L) & (int)(hd < G) & (int)(mykey <= qc) &  \
+                               (int)((mw >> j) & 1u);                                              \
+                const float p = fast_exp2(on ? sacc[vi] * scale_log2 - l4[e] : -INFINITY);         \
+                const float dl = role ? d4[e] : -1.f;                                              \
+                bv[vi] = p * (gamma * pacc[vi] - dl);                                              \
+            }                                                                                      \
+        }                                                                                          \
+        const bf16x8 b0 = pack8(bv), b1 = pack8(bv + 8);                                           \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
+            const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;                                       \
+            acc[dt] = mfma32(tile_trop<D>(t2, 4 * h, m0, lane), b0, acc[dt]);                      \
+            acc[dt] = mfma32(tile_trop<D>(t2, 16 + 4 * h, m0, lane), b1, acc[dt]);                 \
+        }                                                                                          \
+    }
+    TILE_PIPELINE(nblocks, DKV8_LOAD, DKV8_STORE, DKV8_COMPUTE)
+#undef DKV8_LOAD
+#undef DKV8_STORE
+#undef DKV8_COMPUTE
+
+    if (key_ok) {
+        bf16_t *po = (role ? dk : dv) + krow * D + 4 * h;
+        const float osc = role ? scale : 1.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const u32x2 w2 = {pack2bf(acc[dt][4 * g4] * osc, acc[dt][4 * g4 + 1] * osc),
+                                  pack2bf(acc[dt][4 * g4 + 2] * osc, acc[dt][4 * g4 + 3] * osc)};
+                *reinterpret_cast<u32x2 *>(po + dt * 32 + 8 * g4) = w2;
+            }
+    }
+}
+
+// ==================================================================================================
 // launchers: instantiate per head_dim, mask kind and (power-of-two padded) group size
 // ==================================================================================================
 static inline int group_shift(int Hq, int Hkv) {
@@ -492,9 +629,14 @@ template <int D, bool HAS_IDX, int GS>
 static void launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
                          const float *lse, const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N,
                          int T, int Hq, int Hkv, float scale, void *dk, void *dv) {
-    hipLaunchKernelGGL((dsa_tile_dkv_kernel<D, HAS_IDX, GS>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
-                       (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv,
-                       scale, (bf16_t *)dk, (bf16_t *)dv);
+    if constexpr (D <= 128)
+        hipLaunchKernelGGL((dsa_tile_dkv8_kernel<D, HAS_IDX, GS>), grid, dim3(512), 0, stream, (const bf16_t *)dout,
+                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T, Hq,
+                           Hkv, scale, (bf16_t *)dk, (bf16_t *)dv);
+    else
+        hipLaunchKernelGGL((dsa_tile_dkv_kernel<D, HAS_IDX, GS>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
+                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T, Hq,
+                           Hkv, scale, (bf16_t *)dk, (bf16_t *)dv);
 }
 
 #define GS_SWITCH(FN, DD, HI, ...)                                    \
