@@ -45,6 +45,16 @@ __device__ __forceinline__ bf16x8 tile_trop(const unsigned char *tile, int R0, i
 }
 // accumulate in place (kept as a function so that the accumulation sites read alike)
 __device__ __forceinline__ void mfma32_acc(f32x16 &c, bf16x8 a, bf16x8 b) { c = mfma32(a, b, c); }
+// all-ones if bit `b` of `word` is set, else 0 (v_bfe_i32 when b is a compile-time constant)
+__device__ __forceinline__ uint32_t bit_mask(uint32_t word, int b) {
+    return (uint32_t)(((int32_t)(word << (31 - b))) >> 31);
+}
+// x where keep is all-ones, -inf where it is 0 (one v_bfi_b32 / v_bitop3_b32)
+__device__ __forceinline__ float keep_or_neginf(float x, uint32_t keep) {
+    return __uint_as_float((keep & __float_as_uint(x)) | (~keep & 0xff800000u));
+}
+// bits j <= d of a 32-key tile (keys at or before the diagonal when d = query column - tile start)
+__device__ __forceinline__ uint32_t causal_bits(int d) { return d >= 31 ? 0xffffffffu : (d < 0 ? 0u : ((2u << d) - 1u)); }
 __device__ __forceinline__ bf16x8 pack8(const float *x) {
     const u32x4 w = {pack2bf(x[0], x[1]), pack2bf(x[2], x[3]), pack2bf(x[4], x[5]), pack2bf(x[6], x[7])};
     return __builtin_bit_cast(bf16x8, w);
@@ -85,28 +95,32 @@ __device__ __forceinline__ bool locate_block(const int32_t *cu, int N, int slot,
 // K/V tiles are fetched two tiles ahead into registers and one tile ahead into LDS (double buffer),
 // so a global load has two tile-times to land; one barrier per tile.
 // ==================================================================================================
+// Every global load of the pipeline is issued unconditionally (indices past the end are clamped to
+// the last tile) and nothing is computed from a loaded value before the matching STORE, so the
+// compiler can wait with exact vmcnt counts and a load has two tile-times to land.
 #define TILE_PIPELINE(NT, LOAD, STORE, COMPUTE)                                                     \
     {                                                                                              \
+        const int nt_last = (NT) - 1;                                                              \
         LOAD(0, 0);                                                                                \
-        STORE(0, 0);                                                                               \
-        if ((NT) > 1) LOAD(0, 1);                                                                  \
-        if ((NT) > 2) LOAD(1, 2);                                                                  \
+        STORE(0, 0, 0);                                                                            \
+        LOAD(0, min(1, nt_last));                                                                  \
+        LOAD(1, min(2, nt_last));                                                                  \
         __syncthreads();                                                                           \
-        for (int it = 0; it < (NT); it += 2) {                                                     \
-            /* even tile: LDS buffer 0 holds tile it, register set 0 tile it+1, set 1 tile it+2 */   \
+        int it = 0;                                                                                \
+        for (; it + 1 < (NT); it += 2) {                                                           \
+            /* LDS buffer 0 holds tile it, register set 0 tile it+1, register set 1 tile it+2 */     \
             COMPUTE(it, 0);                                                                        \
             if (NBUF == 1) __syncthreads();                                                        \
-            if (it + 1 < (NT)) STORE(0, NBUF - 1);                                                 \
-            if (it + 3 < (NT)) LOAD(0, it + 3);                                                    \
+            STORE(0, NBUF - 1, it + 1);                                                            \
+            LOAD(0, min(it + 3, nt_last));                                                         \
             __syncthreads();                                                                       \
-            if (it + 1 < (NT)) {                                                                   \
-                COMPUTE(it + 1, NBUF - 1);                                                         \
-                if (NBUF == 1) __syncthreads();                                                    \
-                if (it + 2 < (NT)) STORE(1, 0);                                                    \
-                if (it + 4 < (NT)) LOAD(1, it + 4);                                                \
-                __syncthreads();                                                                   \
-            }                                                                                      \
+            COMPUTE(it + 1, NBUF - 1);                                                             \
+            if (NBUF == 1) __syncthreads();                                                        \
+            STORE(1, 0, min(it + 2, nt_last));                                                     \
+            LOAD(1, min(it + 4, nt_last));                                                         \
+            __syncthreads();                                                                       \
         }                                                                                          \
+        if (it < (NT)) COMPUTE(it, 0);                                                             \
     }
 
 template <int D, bool HAS_IDX, int GSHIFT>
@@ -144,7 +158,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) oacc[dt] = zero16();
     float mrun = -INFINITY, lsum = 0.f;
-    uint32_t word_next = (HAS_IDX && row_ok) ? wrow[0] : 0u;
+    uint32_t word_next = HAS_IDX ? wrow[0] : 0u;        // unconditional loads; rows that are not live are masked at use
 
 #define FWD_LOAD(SET, TILE)                                                                         \
     _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
@@ -154,7 +168,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
         kst[SET][i] = *reinterpret_cast<const u32x4 *>(k + off);                                   \
         vst[SET][i] = *reinterpret_cast<const u32x4 *>(v + off);                                   \
     }
-#define FWD_STORE(SET, BUF)                                                                         \
+#define FWD_STORE(SET, BUF, TILE)                                                                        \
     _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
         const int c = i * 256 + tid;                                                               \
         const int row = c / CPR, ch = c % CPR;                                                     \
@@ -165,32 +179,36 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
     {                                                                                              \
         const int kc0 = (TILE) * 32;                                                               \
         const unsigned char *kt = lds[BUF][0], *vt = lds[BUF][1];                                  \
-        const uint32_t word = word_next;                                                           \
-        if (HAS_IDX && row_ok && (TILE) + 1 < ntiles) word_next = wrow[(TILE) + 1];                \
+        uint32_t word = row_ok ? word_next : 0u;                                                   \
+        if (HAS_IDX) word_next = wrow[min((TILE) + 1, ntiles - 1)];                                \
+        if (!HAS_IDX) word = row_ok ? causal_bits(qcol - kc0) : 0u;                                \
+        word >>= 4 * h;                                  /* element vi then sits at bit 8*(vi/4) + vi%4 */ \
         f32x16 sacc = zero16();                                                                    \
         _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                          \
             sacc = mfma32(tile_rowop<D>(kt, j, ks, h), qB[ks], sacc);                              \
         float s2[16], mloc = -INFINITY;                                                            \
         _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
-            const int kk = c_row(vi, h);                                                           \
-            const bool on = HAS_IDX ? ((word >> kk) & 1u) : (row_ok && kc0 + kk <= qcol);          \
-            s2[vi] = on ? sacc[vi] * scale_log2 : -INFINITY;                                       \
+            s2[vi] = keep_or_neginf(sacc[vi], bit_mask(word, 8 * (vi >> 2) + (vi & 3)));           \
             mloc = fmaxf(mloc, s2[vi]);                                                            \
         }                                                                                          \
-        mloc = fmaxf(mloc, wave_xor_f(mloc, 32));                                                  \
-        const float mnew = fmaxf(mrun, mloc);                                                      \
-        const float mref = (mnew == -INFINITY) ? 0.f : mnew; /* rows with nothing selected so far */ \
-        const float alpha = fast_exp2(mrun - mref);                                                \
+        mloc = fmaxf(mloc, wave_xor_f(mloc, 32)) * scale_log2;                                     \
+        /* the reference maximum only moves when a row's maximum grows by more than 2^8 (rare      \
+           after the first tiles); until then P stays below 2^8, exact in fp32 and safe in bf16 */ \
+        if (__builtin_amdgcn_ballot_w64(mloc > mrun + 8.f)) {                                      \
+            const float mnew = fmaxf(mrun, mloc);                                                  \
+            float alpha = fast_exp2(mrun - ((mnew == -INFINITY) ? 0.f : mnew));                    \
+            asm volatile("" : "+v"(alpha));              /* keep the rescale inside the branch */   \
+            lsum *= alpha;                                                                         \
+            _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) oacc[dt] *= alpha;                   \
+            mrun = mnew;                                                                           \
+        }                                                                                          \
+        const float mneg = (mrun == -INFINITY) ? 0.f : -mrun; /* rows with nothing selected yet */   \
         float psum = 0.f;                                                                          \
         _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
-            s2[vi] = fast_exp2(s2[vi] - mref);                                                     \
+            s2[vi] = fast_exp2(fmaf(s2[vi], scale_log2, mneg));                                    \
             psum += s2[vi];                                                                        \
         }                                                                                          \
-        lsum = lsum * alpha + psum;                                                                \
-        if (__builtin_amdgcn_ballot_w64(mnew != mrun)) { /* some row's maximum moved: rescale */     \
-            _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) oacc[dt] *= alpha;                   \
-        }                                                                                          \
-        mrun = mnew;                                                                               \
+        lsum += psum;                                                                              \
         const bf16x8 pB0 = pack8(s2), pB1 = pack8(s2 + 8);                                         \
         _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
             const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;                                       \
@@ -265,7 +283,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
     f32x16 acc[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
-    uint32_t word_next = (HAS_IDX && row_ok) ? wrow[0] : 0u;
+    uint32_t word_next = HAS_IDX ? wrow[0] : 0u;        // unconditional loads; rows that are not live are masked at use
 
 #define DQ_LOAD(SET, TILE)                                                                          \
     _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
@@ -275,7 +293,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
         kst[SET][i] = *reinterpret_cast<const u32x4 *>(k + off);                                   \
         vst[SET][i] = *reinterpret_cast<const u32x4 *>(v + off);                                   \
     }
-#define DQ_STORE(SET, BUF)                                                                          \
+#define DQ_STORE(SET, BUF, TILE)                                                                         \
     _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
         const int c = i * 256 + tid;                                                               \
         const int row = c / CPR, ch = c % CPR;                                                     \
@@ -286,8 +304,10 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
     {                                                                                              \
         const int kc0 = (TILE) * 32;                                                               \
         const unsigned char *kt = lds[BUF][0], *vt = lds[BUF][1];                                  \
-        const uint32_t word = word_next;                                                           \
-        if (HAS_IDX && row_ok && (TILE) + 1 < ntiles) word_next = wrow[(TILE) + 1];                \
+        uint32_t word = row_ok ? word_next : 0u;                                                   \
+        if (HAS_IDX) word_next = wrow[min((TILE) + 1, ntiles - 1)];                                \
+        if (!HAS_IDX) word = row_ok ? causal_bits(qcol - kc0) : 0u;                                \
+        word >>= 4 * h;                                                                            \
         f32x16 sacc = zero16(), pacc = zero16();                                                   \
         _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
             sacc = mfma32(tile_rowop<D>(kt, j, ks, h), qB[ks], sacc);                              \
@@ -295,10 +315,9 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
         }                                                                                          \
         float ds[16];                                                                              \
         _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
-            const int kk = c_row(vi, h);                                                           \
-            const bool on = HAS_IDX ? ((word >> kk) & 1u) : (row_ok && kc0 + kk <= qcol);          \
-            const float p = on ? fast_exp2(sacc[vi] * scale_log2 - lse2) : 0.f;                    \
-            ds[vi] = p * (pacc[vi] - dlt);                                                         \
+            const float x = keep_or_neginf(fmaf(sacc[vi], scale_log2, -lse2),                      \
+                                           bit_mask(word, 8 * (vi >> 2) + (vi & 3)));              \
+            ds[vi] = fast_exp2(x) * (pacc[vi] - dlt);                                              \
         }                                                                                          \
         const bf16x8 dB0 = pack8(ds), dB1 = pack8(ds + 8);                                         \
         _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
@@ -369,8 +388,27 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
     const int nblocks = (L - c0 + QB - 1) / QB;          // queries c0 .. L-1
 
     u32x4 qst[2][LOADS], dost[2][LOADS];
-    float aux_st[2] = {0.f, 0.f};                        // lse / delta / mask word of the staging threads
-    // threads 0..31: lse of row tid; 32..63: delta of row tid-32; 64..64+4*QB-1: mask word (wave w, query qi)
+    // Per-block side data, one 32-bit word per staging thread, loaded raw and interpreted at STORE time:
+    //   tid 0..31: lse of row tid;  32..63: delta of row tid-32;  64..64+4*QB-1: selection word of
+    //   (key group w, query qi);  the rest re-read a valid word and drop it.
+    const uint32_t *aux_base;
+    int aux_q = 0, aux_stride = 1;                       // word index = aux_stride * min(block start + aux_q, L-1)
+    bool aux_mask_ok = false;
+    if (tid < 64) {
+        const int row = tid & 31;
+        const int hd = min(row & (Gp - 1), G - 1);
+        aux_q = row >> GSHIFT;
+        aux_base = reinterpret_cast<const uint32_t *>((tid < 32 ? lse : delta) + (int64_t)(kvh * G + hd) * T + s0);
+    } else if (HAS_IDX && tid < 64 + 4 * QB) {
+        const int w = (tid - 64) / QB;
+        aux_q = (tid - 64) % QB;
+        aux_stride = ldw;
+        aux_mask_ok = (c0 >> 5) + w < ldw;
+        aux_base = bitmap + (int64_t)s0 * ldw + (aux_mask_ok ? (c0 >> 5) + w : 0);
+    } else {
+        aux_base = reinterpret_cast<const uint32_t *>(lse);
+    }
+    uint32_t aux_st[2] = {0u, 0u};
 #define DKV_LOAD(SET, BLK)                                                                          \
     {                                                                                              \
         const int qcb = c0 + (BLK) * QB;                                                           \
@@ -383,30 +421,24 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
             qst[SET][i] = *reinterpret_cast<const u32x4 *>(q + off);                               \
             dost[SET][i] = *reinterpret_cast<const u32x4 *>(dout + off);                           \
         }                                                                                          \
-        if (tid < 64) {                                                                            \
-            const int row = tid & 31;                                                              \
-            const int qc = min(qcb + (row >> GSHIFT), L - 1);                                      \
-            const int hd = min(row & (Gp - 1), G - 1);                                             \
-            const int64_t o = (int64_t)(kvh * G + hd) * T + s0 + qc;                               \
-            aux_st[SET] = (tid < 32) ? lse[o] * LOG2E_F : delta[o];                                \
-        } else if (HAS_IDX && tid < 64 + 4 * QB) {                                                 \
-            const int w = (tid - 64) / QB, qi = (tid - 64) % QB;                                   \
-            const int qc = qcb + qi;                                                               \
-            const uint32_t m = (qc < L && (c0 >> 5) + w < ldw) ? bitmap[(int64_t)(s0 + qc) * ldw + (c0 >> 5) + w] : 0u; \
-            aux_st[SET] = __uint_as_float(m);                                                      \
-        }                                                                                          \
+        aux_st[SET] = aux_base[(int64_t)aux_stride * min(qcb + aux_q, L - 1)];                     \
     }
-#define DKV_STORE(SET, BUF)                                                                         \
+#define DKV_STORE(SET, BUF, BLK)                                                                    \
     {                                                                                              \
+        const int qcb = c0 + (BLK) * QB;                                                           \
+        const u32x4 z4 = {0u, 0u, 0u, 0u};                                                         \
         _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                        \
             const int c = i * 256 + tid;                                                           \
             const int row = c / CPR, ch = c % CPR;                                                 \
-            *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(row, ch)]) = qst[SET][i];          \
-            *reinterpret_cast<u32x4 *>(&lds[BUF][1][tile_off<D>(row, ch)]) = dost[SET][i];         \
+            /* rows past the segment and padded heads are zeroed: they add nothing to dK, dV */     \
+            const bool live = qcb + (row >> GSHIFT) < L && (row & (Gp - 1)) < G;                   \
+            *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(row, ch)]) = live ? qst[SET][i] : z4;  \
+            *reinterpret_cast<u32x4 *>(&lds[BUF][1][tile_off<D>(row, ch)]) = live ? dost[SET][i] : z4; \
         }                                                                                          \
-        if (tid < 32) lse_s[BUF][tid] = aux_st[SET];                                               \
-        else if (tid < 64) dlt_s[BUF][tid - 32] = aux_st[SET];                                     \
-        else if (HAS_IDX && tid < 64 + 4 * QB) mask_s[BUF][(tid - 64) / QB][(tid - 64) % QB] = __float_as_uint(aux_st[SET]); \
+        if (tid < 32) lse_s[BUF][tid] = __uint_as_float(aux_st[SET]) * LOG2E_F;                    \
+        else if (tid < 64) dlt_s[BUF][tid - 32] = __uint_as_float(aux_st[SET]);                    \
+        else if (HAS_IDX && tid < 64 + 4 * QB)                                                     \
+            mask_s[BUF][(tid - 64) / QB][(tid - 64) % QB] = (aux_mask_ok && qcb + aux_q < L) ? aux_st[SET] : 0u; \
     }
 #define DKV_COMPUTE(BLK, BUF)                                                                       \
     {                                                                                              \
@@ -418,17 +450,20 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
             pacc = mfma32(tile_rowop<D>(dot, j, ks, h), vB[ks], pacc);                             \
         }                                                                                          \
         float pv[16], dsv[16];                                                                     \
+        const bool diag = qcb < kc + 32;                /* wave-uniform: block touches the diagonal */ \
         _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {                                         \
             const f32x4 l4 = *reinterpret_cast<const f32x4 *>(&lse_s[BUF][8 * g4 + 4 * h]);        \
             const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&dlt_s[BUF][8 * g4 + 4 * h]);        \
+            uint32_t keep = 0u;                                                                    \
             _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                        \
                 const int vi = 4 * g4 + e, row = 8 * g4 + 4 * h + e;                               \
-                const int qi = row >> GSHIFT, hd = row & (Gp - 1);                                 \
-                const int qc = qcb + qi;                                                           \
-                const uint32_t mw = HAS_IDX ? mask_s[BUF][wv][qi] : 0xffffffffu;                   \
-                const int on = (int)key_ok & (int)(qc < L) & (int)(hd < G) & (int)(mykey <= qc) &  \
-                               (int)((mw >> j) & 1u);                 /* branch-free */             \
-                const float p = fast_exp2(on ? sacc[vi] * scale_log2 - l4[e] : -INFINITY);         \
+                if (e == 0 || GSHIFT < 2) {              /* rows of one query share the mask bit */  \
+                    const int qi = row >> GSHIFT;                                                  \
+                    uint32_t mw = HAS_IDX ? mask_s[BUF][wv][qi] : 0xffffffffu;                     \
+                    if (diag) mw &= causal_bits(qcb + qi - kc);                                    \
+                    keep = bit_mask(mw, j);                                                        \
+                }                                                                                  \
+                const float p = fast_exp2(keep_or_neginf(fmaf(sacc[vi], scale_log2, -l4[e]), keep)); \
                 pv[vi] = p;                                                                        \
                 dsv[vi] = p * (pacc[vi] - d4[e]);                                                  \
             }                                                                                      \
@@ -505,46 +540,56 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv8_kernel(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
     const float scale_log2 = scale * LOG2E_F;
-    const float gamma = role ? 1.f : 0.f;                // B = p * (gamma * dP - delta'), delta' = -1 for the dV role
     const int nblocks = (L - c0 + QB - 1) / QB;          // queries c0 .. L-1
     const bool stager = tid < NCHUNK;
-    const int srow = tid / CPR, sch = tid % CPR;
+    const int srow = (tid % NCHUNK) / CPR, sch = tid % CPR;   // non-staging threads re-read a staged chunk and drop it
 
     u32x4 qst[2], dost[2];
-    float aux_st[2] = {0.f, 0.f};
-    // aux staging threads: 0..31 lse of row tid; 32..63 delta of row tid-32; 64..64+4*QB-1 mask words
+    // Per-block side data, one 32-bit word per staging thread, loaded raw and interpreted at STORE time:
+    //   tid 0..31: lse of row tid;  32..63: delta of row tid-32;  64..64+4*QB-1: selection word of
+    //   (key group w, query qi);  the rest re-read a valid word and drop it.
+    const uint32_t *aux_base;
+    int aux_q = 0, aux_stride = 1;                       // word index = aux_stride * min(block start + aux_q, L-1)
+    bool aux_mask_ok = false;
+    if (tid < 64) {
+        const int row = tid & 31;
+        const int hd = min(row & (Gp - 1), G - 1);
+        aux_q = row >> GSHIFT;
+        aux_base = reinterpret_cast<const uint32_t *>((tid < 32 ? lse : delta) + (int64_t)(kvh * G + hd) * T + s0);
+    } else if (HAS_IDX && tid < 64 + 4 * QB) {
+        const int w = (tid - 64) / QB;
+        aux_q = (tid - 64) % QB;
+        aux_stride = ldw;
+        aux_mask_ok = (c0 >> 5) + w < ldw;
+        aux_base = bitmap + (int64_t)s0 * ldw + (aux_mask_ok ? (c0 >> 5) + w : 0);
+    } else {
+        aux_base = reinterpret_cast<const uint32_t *>(lse);
+    }
+    uint32_t aux_st[2] = {0u, 0u};
 #define DKV8_LOAD(SET, BLK)                                                                         \
     {                                                                                              \
         const int qcb = c0 + (BLK) * QB;                                                           \
-        if (stager) {                                                                              \
-            const int qc = min(qcb + (srow >> GSHIFT), L - 1);                                     \
-            const int hd = min(srow & (Gp - 1), G - 1);                                            \
-            const int64_t off = ((int64_t)(s0 + qc) * Hq + kvh * G + hd) * D + sch * 8;            \
-            qst[SET] = *reinterpret_cast<const u32x4 *>(q + off);                                  \
-            dost[SET] = *reinterpret_cast<const u32x4 *>(dout + off);                              \
-        }                                                                                          \
-        if (tid < 64) {                                                                            \
-            const int row = tid & 31;                                                              \
-            const int qc = min(qcb + (row >> GSHIFT), L - 1);                                      \
-            const int hd = min(row & (Gp - 1), G - 1);                                             \
-            const int64_t o = (int64_t)(kvh * G + hd) * T + s0 + qc;                               \
-            aux_st[SET] = (tid < 32) ? lse[o] * LOG2E_F : delta[o];                                \
-        } else if (HAS_IDX && tid < 64 + 4 * QB) {                                                 \
-            const int w = (tid - 64) / QB, qi = (tid - 64) % QB;                                   \
-            const int qc = qcb + qi;                                                               \
-            const uint32_t m = (qc < L && (c0 >> 5) + w < ldw) ? bitmap[(int64_t)(s0 + qc) * ldw + (c0 >> 5) + w] : 0u; \
-            aux_st[SET] = __uint_as_float(m);                                                      \
-        }                                                                                          \
+        const int qc = min(qcb + (srow >> GSHIFT), L - 1);                                         \
+        const int hd = min(srow & (Gp - 1), G - 1);                                                \
+        const int64_t off = ((int64_t)(s0 + qc) * Hq + kvh * G + hd) * D + sch * 8;                \
+        qst[SET] = *reinterpret_cast<const u32x4 *>(q + off);                                      \
+        dost[SET] = *reinterpret_cast<const u32x4 *>(dout + off);                                  \
+        aux_st[SET] = aux_base[(int64_t)aux_stride * min(qcb + aux_q, L - 1)];                     \
     }
-#define DKV8_STORE(SET, BUF)                                                                        \
+#define DKV8_STORE(SET, BUF, BLK)                                                                   \
     {                                                                                              \
+        const int qcb = c0 + (BLK) * QB;                                                           \
         if (stager) {                                                                              \
-            *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(srow, sch)]) = qst[SET];           \
-            *reinterpret_cast<u32x4 *>(&lds[BUF][1][tile_off<D>(srow, sch)]) = dost[SET];          \
+            /* rows past the segment and padded heads are zeroed: they add nothing to dK, dV */     \
+            const bool live = qcb + (srow >> GSHIFT) < L && (srow & (Gp - 1)) < G;                 \
+            const u32x4 z4 = {0u, 0u, 0u, 0u};                                                     \
+            *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(srow, sch)]) = live ? qst[SET] : z4;  \
+            *reinterpret_cast<u32x4 *>(&lds[BUF][1][tile_off<D>(srow, sch)]) = live ? dost[SET] : z4; \
         }                                                                                          \
-        if (tid < 32) lse_s[BUF][tid] = aux_st[SET];                                               \
-        else if (tid < 64) dlt_s[BUF][tid - 32] = aux_st[SET];                                     \
-        else if (HAS_IDX && tid < 64 + 4 * QB) mask_s[BUF][(tid - 64) / QB][(tid - 64) % QB] = __float_as_uint(aux_st[SET]); \
+        if (tid < 32) lse_s[BUF][tid] = __uint_as_float(aux_st[SET]) * LOG2E_F;                    \
+        else if (tid < 64) dlt_s[BUF][tid - 32] = __uint_as_float(aux_st[SET]);                    \
+        else if (HAS_IDX && tid < 64 + 4 * QB)                                                     \
+            mask_s[BUF][(tid - 64) / QB][(tid - 64) % QB] = (aux_mask_ok && qcb + aux_q < L) ? aux_st[SET] : 0u; \
     }
 #define DKV8_COMPUTE(BLK, BUF)                                                                      \
     {                                                                                              \
@@ -559,19 +604,21 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv8_kernel(
                 pacc = mfma32(tile_rowop<D>(dot, j, ks, h), vB[ks], pacc);                         \
         }                                                                                          \
         float bv[16];                                                                              \
+        const bool diag = qcb < kc + 32;                /* wave-uniform: block touches the diagonal */ \
         _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {                                         \
             const f32x4 l4 = *reinterpret_cast<const f32x4 *>(&lse_s[BUF][8 * g4 + 4 * h]);        \
             const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&dlt_s[BUF][8 * g4 + 4 * h]);        \
+            uint32_t keep = 0u;                                                                    \
             _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                        \
                 const int vi = 4 * g4 + e, row = 8 * g4 + 4 * h + e;                               \
-                const int qi = row >> GSHIFT, hd = row & (Gp - 1);                                 \
-                const int qc = qcb + qi;                                                           \
-                const uint32_t mw = HAS_IDX ? mask_s[BUF][kg][qi] : 0xffffffffu;                   \
-                const int on = (int)key_ok & (int)(qc < L) & (int)(hd < G) & (int)(mykey <= qc) &  \
-                               (int)((mw >> j) & 1u);                                              \
-                const float p = fast_exp2(on ? sacc[vi] * scale_log2 - l4[e] : -INFINITY);         \
-                const float dl = role ? d4[e] : -1.f;                                              \
-                bv[vi] = p * (gamma * pacc[vi] - dl);                                              \
+                if (e == 0 || GSHIFT < 2) {              /* rows of one query share the mask bit */  \
+                    const int qi = row >> GSHIFT;                                                  \
+                    uint32_t mw = HAS_IDX ? mask_s[BUF][kg][qi] : 0xffffffffu;                     \
+                    if (diag) mw &= causal_bits(qcb + qi - kc);                                    \
+                    keep = bit_mask(mw, j);                                                        \
+                }                                                                                  \
+                const float p = fast_exp2(keep_or_neginf(fmaf(sacc[vi], scale_log2, -l4[e]), keep)); \
+                bv[vi] = role ? p * (pacc[vi] - d4[e]) : p;                                        \
             }                                                                                      \
         }                                                                                          \
         const bf16x8 b0 = pack8(bv), b1 = pack8(bv + 8);                                           \
