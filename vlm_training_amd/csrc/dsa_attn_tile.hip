@@ -55,6 +55,19 @@ __device__ __forceinline__ float keep_or_neginf(float x, uint32_t keep) {
 }
 // bits j <= d of a 32-key tile (keys at or before the diagonal when d = query column - tile start)
 __device__ __forceinline__ uint32_t causal_bits(int d) { return d >= 31 ? 0xffffffffu : (d < 0 ? 0u : ((2u << d) - 1u)); }
+// Issue order for a chain of NM MFMAs that each consume RPM LDS reads: keep AHEAD MFMAs' worth of reads
+// in flight (the machine scheduler otherwise sinks every read next to its use and the chain runs at
+// LDS latency).  Applies to the instructions of the enclosing basic block, in program order.
+template <int NM, int AHEAD, int RPM>
+__device__ __forceinline__ void sched_reads_ahead() {
+    __builtin_amdgcn_sched_group_barrier(0x100, AHEAD * RPM, 0);
+#pragma unroll
+    for (int i = 0; i < NM - AHEAD; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, RPM, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
+}
 __device__ __forceinline__ bf16x8 pack8(const float *x) {
     const u32x4 w = {pack2bf(x[0], x[1]), pack2bf(x[2], x[3]), pack2bf(x[4], x[5]), pack2bf(x[6], x[7])};
     return __builtin_bit_cast(bf16x8, w);
@@ -184,8 +197,12 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
         if (!HAS_IDX) word = row_ok ? causal_bits(qcol - kc0) : 0u;                                \
         word >>= 4 * h;                                  /* element vi then sits at bit 8*(vi/4) + vi%4 */ \
         f32x16 sacc = zero16();                                                                    \
-        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                          \
-            sacc = mfma32(tile_rowop<D>(kt, j, ks, h), qB[ks], sacc);                              \
+        {                                                /* all K operands in flight before the first MFMA */ \
+            bf16x8 ka[KS];                                                                         \
+            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) ka[ks] = tile_rowop<D>(kt, j, ks, h); \
+            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) sacc = mfma32(ka[ks], qB[ks], sacc); \
+            sched_reads_ahead<KS, 4, 1>();                                                         \
+        }                                                                                          \
         float s2[16], mloc = -INFINITY;                                                            \
         _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
             s2[vi] = keep_or_neginf(sacc[vi], bit_mask(word, 8 * (vi >> 2) + (vi & 3)));           \
@@ -215,6 +232,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
             mfma32_acc(oacc[dt], tile_trop<D>(vt, 4 * h, m0, lane), pB0);                          \
             mfma32_acc(oacc[dt], tile_trop<D>(vt, 16 + 4 * h, m0, lane), pB1);                     \
         }                                                                                          \
+        sched_reads_ahead<2 * DT, 3, 2>();                                                         \
     }
     TILE_PIPELINE(ntiles, FWD_LOAD, FWD_STORE, FWD_COMPUTE)
 #undef FWD_LOAD
@@ -313,6 +331,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
             sacc = mfma32(tile_rowop<D>(kt, j, ks, h), qB[ks], sacc);                              \
             pacc = mfma32(tile_rowop<D>(vt, j, ks, h), doB[ks], pacc);                             \
         }                                                                                          \
+        sched_reads_ahead<2 * KS, 4, 1>();                                                         \
         float ds[16];                                                                              \
         _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
             const float x = keep_or_neginf(fmaf(sacc[vi], scale_log2, -lse2),                      \
@@ -325,6 +344,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
             mfma32_acc(acc[dt], tile_trop<D>(kt, 4 * h, m0, lane), dB0);                           \
             mfma32_acc(acc[dt], tile_trop<D>(kt, 16 + 4 * h, m0, lane), dB1);                      \
         }                                                                                          \
+        sched_reads_ahead<2 * DT, 3, 2>();                                                         \
     }
     TILE_PIPELINE(ntiles, DQ_LOAD, DQ_STORE, DQ_COMPUTE)
 #undef DQ_LOAD
@@ -599,9 +619,11 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv8_kernel(
         f32x16 sacc = zero16(), pacc = zero16();                                                   \
         _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                          \
             sacc = mfma32(tile_rowop<D>(qt, j, ks, h), kB[ks], sacc);                              \
+        sched_reads_ahead<KS, 4, 1>();                                                             \
         if (role) {                                     /* wave-uniform */                          \
             _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                      \
                 pacc = mfma32(tile_rowop<D>(dot, j, ks, h), vB[ks], pacc);                         \
+            sched_reads_ahead<KS, 4, 1>();                                                         \
         }                                                                                          \
         float bv[16];                                                                              \
         const bool diag = qcb < kc + 32;                /* wave-uniform: block touches the diagonal */ \
@@ -627,6 +649,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv8_kernel(
             acc[dt] = mfma32(tile_trop<D>(t2, 4 * h, m0, lane), b0, acc[dt]);                      \
             acc[dt] = mfma32(tile_trop<D>(t2, 16 + 4 * h, m0, lane), b1, acc[dt]);                 \
         }                                                                                          \
+        sched_reads_ahead<2 * DT, 3, 2>();                                                         \
     }
     TILE_PIPELINE(nblocks, DKV8_LOAD, DKV8_STORE, DKV8_COMPUTE)
 #undef DKV8_LOAD
