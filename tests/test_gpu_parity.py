@@ -167,6 +167,25 @@ def test_tile_and_gather_paths_agree_with_the_oracle(crossover, name, segs, K):
         a += L
 
 
+def test_headline_geometry_with_full_top_k():
+    """C3 head geometry with its real top_k = 2048 on segments long enough to have sparse rows spanning
+    many bitmap words, plus an image-patch run (clustered selections)."""
+    _log("C3 K=2048")
+    _run_case(W.scaled(W.C3, (3000, 2304), top_k=2048, name="C3-k2048"))
+
+
+@pytest.mark.parametrize("Hq,Hkv,D", [(6, 2, 128), (4, 4, 64), (16, 1, 128), (2, 1, 256)])
+def test_sparse_path_odd_head_groups(Hq, Hkv, D):
+    """Group sizes that are not the configs': G = 3 (padded to 4), 1, 16 and 2, through tiles and gather."""
+    _log(f"odd groups {Hq}/{Hkv}/{D}")
+    base = W.Workload("odd", torch.bfloat16, (333, 140, 515), Hq, Hkv, D, 8, 32, 48, 0.5, 77)
+    old = ops.set_tile_crossover(3)                      # rows before pos 256 on tiles, the rest gathered
+    try:
+        _run_case(base)
+    finally:
+        ops.set_tile_crossover(old)
+
+
 def test_dense_path_equals_reference_semantics():
     _log("dense path")
     g = torch.Generator().manual_seed(11)
