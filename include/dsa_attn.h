@@ -81,10 +81,12 @@ int dsa_index_topk(const void *q_idx, const void *k_idx, const void *w_idx, cons
  * segment when idx == NULL: that case is the drop-in for varlen_attn(..., window_size=(-1,0))
  * (train/model_attention.py:123-132; models/qwen3_vl/model.py:41-46; models/qwen3_5/model.py:93-98).
  * q head h reads kv head h / (Hq/Hkv) (models/qwen3/model.py:125-129).  softmax in fp32.
+ * causal == 0 (only with idx == NULL) attends every key of the own segment: the vision towers' call,
+ * varlen_attn(..., window_size=(-1,-1)) (models/qwen3_vl/model.py:423-428, models/qwen3_5/model.py:388-393).
  */
 int dsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
                  const int32_t *cu_seqlens, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
-                 int dtype, int max_seqlen, void *out, float *lse, void *ws, size_t ws_bytes, void *stream);
+                 int dtype, int max_seqlen, int causal, void *out, float *lse, void *ws, size_t ws_bytes, void *stream);
 
 /* Bytes of workspace dsa_attn_fwd needs (the inverted selection bitmap; 0 without idx). */
 size_t dsa_attn_fwd_workspace_bytes(int T, int max_seqlen, int has_idx);
@@ -107,8 +109,8 @@ size_t dsa_attn_bwd_workspace_bytes(int T, int Hq, int max_seqlen, int has_idx);
  */
 int dsa_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out, const float *lse,
                  const int32_t *idx, const int32_t *n, const int32_t *cu_seqlens, int T, int N, int Hq, int Hkv,
-                 int D, int K, float softmax_scale, int dtype, int max_seqlen, void *dq, void *dk, void *dv,
-                 void *ws, size_t ws_bytes, void *stream);
+                 int D, int K, float softmax_scale, int dtype, int max_seqlen, int causal, void *dq, void *dk,
+                 void *dv, void *ws, size_t ws_bytes, void *stream);
 
 /*
  * Measurement hook: dsa_attn_bwd restricted to the kernels named in `parts`, so that each can be
@@ -123,8 +125,8 @@ int dsa_attn_bwd(const void *dout, const void *q, const void *k, const void *v, 
 #define DSA_BWD_ALL 15
 int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k, const void *v, const void *out,
                        const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu_seqlens, int T, int N,
-                       int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen, void *dq, void *dk,
-                       void *dv, void *ws, size_t ws_bytes, int parts, void *stream);
+                       int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen, int causal,
+                       void *dq, void *dk, void *dv, void *ws, size_t ws_bytes, int parts, void *stream);
 
 #ifdef __cplusplus
 }

@@ -45,7 +45,7 @@ def test_workspace_sizes_without_a_gpu():
 
 def test_argument_errors_are_reported_not_thrown():
     lib = _lib.load()
-    rc = lib.dsa_attn_fwd(None, None, None, None, None, None, 8, 1, 4, 3, 64, 0, 1.0, 0, 8, None, None, None, 0, None)
+    rc = lib.dsa_attn_fwd(None, None, None, None, None, None, 8, 1, 4, 3, 64, 0, 1.0, 0, 8, 1, None, None, None, 0, None)
     assert rc == -1 and b"cu_seqlens" in lib.dsa_last_error()
     with pytest.raises(ValueError):
         _lib.check(rc, "dsa_attn_fwd")

@@ -208,6 +208,35 @@ def test_dense_path_equals_reference_semantics():
         assert_close_bf16(vd.grad, vr.grad, "dv")
 
 
+def test_non_causal_packed_attention_for_the_vision_towers():
+    """causal=False: every key of the own segment (models/qwen3_vl/model.py:423-428 calls
+    dispatch_varlen_attention(..., causal=False) with cu_seqlens built from grid_thw)."""
+    _log("non-causal")
+    import vlm_training_amd as M
+    g = torch.Generator().manual_seed(21)
+    cu = [0, 64, 64, 320, 401, 977]
+    T = cu[-1]
+    for Hq, Hkv, D in ((16, 16, 64), (4, 2, 128), (2, 1, 256)):
+        q = (torch.randn(T, Hq, D, generator=g) * 0.6).bfloat16()
+        k = (torch.randn(T, Hkv, D, generator=g) * 0.6).bfloat16()
+        v = (torch.randn(T, Hkv, D, generator=g) * 0.6).bfloat16()
+        do = torch.randn(T, Hq, D, generator=g).bfloat16()
+        qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+        out = M.dispatch_varlen_attention(qd, kd, vd, torch.tensor(cu, dtype=torch.int32, device=DEV), 576, causal=False)
+        out.backward(do.to(DEV))
+        qr, kr, vr = (x.float().requires_grad_(True) for x in (q, k, v))
+        ref = R.dense_varlen_causal(qr, kr, vr, cu, causal=False)
+        ref.backward(do.float())
+        assert_close_bf16(out, ref, f"out {Hq}/{Hkv}/{D}")
+        assert_close_bf16(qd.grad, qr.grad, "dq")
+        assert_close_bf16(kd.grad, kr.grad, "dk")
+        assert_close_bf16(vd.grad, vr.grad, "dv")
+    with pytest.raises(ValueError):
+        ops.dsa_varlen_attn(qd, kd, vd, torch.tensor(cu, dtype=torch.int32, device=DEV), 576, causal=False,
+                            indexer_q=torch.zeros(T, 2, 32, device=DEV), indexer_k=torch.zeros(T, 32, device=DEV),
+                            indexer_w=torch.zeros(T, 2, device=DEV), top_k=8)
+
+
 def test_topk_at_least_longest_segment_is_dense():
     _log("K >= L")
     w = W.scaled(W.C2, (300, 120, 77), top_k=512, name="C2-dense")

@@ -87,6 +87,19 @@ def test_dense_first_token_is_v_and_rows_are_convex():
     assert torch.allclose(R.dense_varlen_causal(q, k, v1, cu), torch.ones_like(q), atol=1e-6)
 
 
+def test_non_causal_dense_matches_bruteforce():
+    cu = [0, 6, 15]
+    q, k, v = rnd(15, 2, 4, seed=41), rnd(15, 1, 4, seed=42), rnd(15, 1, 4, seed=43)
+    got = R.dense_varlen_causal(q, k, v, cu, causal=False)
+    want = torch.zeros(15, 2, 4, dtype=torch.float64)
+    for a, b in zip(cu[:-1], cu[1:]):
+        for t in range(a, b):
+            for h in range(2):
+                w = torch.softmax(torch.stack([torch.dot(q[t, h].double(), k[s, 0].double()) / 2.0 for s in range(a, b)]), 0)
+                want[t, h] = sum(w[i] * v[a + i, 0].double() for i in range(b - a))
+    assert torch.allclose(got.double(), want, atol=1e-5)
+
+
 def test_gqa_head_mapping_is_h_div_g():
     # kv head 1 carries a marker value; only q heads 2,3 (G=2) may see it
     T = 6

@@ -24,13 +24,13 @@ hipError_t dsa_launch_gather_dq(const void *dout, const void *q, const void *k, 
                                 hipStream_t stream);
 hipError_t dsa_launch_tile_fwd(const void *q, const void *k, const void *v, const uint32_t *bitmap, int ldw,
                                const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale, int pos_split,
-                               void *out, float *lse, hipStream_t stream);
+                               int causal, void *out, float *lse, hipStream_t stream);
 hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const void *k, const void *v, const float *lse,
                               const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T,
-                              int Hq, int Hkv, int D, float scale, int pos_split, void *dq, hipStream_t stream);
+                              int Hq, int Hkv, int D, float scale, int pos_split, int causal, void *dq, hipStream_t stream);
 hipError_t dsa_launch_tile_dkv(const void *dout, const void *q, const void *k, const void *v, const float *lse,
                                const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T,
-                               int Hq, int Hkv, int D, float scale, void *dk, void *dv, hipStream_t stream);
+                               int Hq, int Hkv, int D, float scale, int causal, void *dk, void *dv, hipStream_t stream);
 }
 
 static thread_local char g_err[512] = "";
@@ -160,8 +160,10 @@ extern "C" size_t dsa_attn_fwd_workspace_bytes(int T, int max_seqlen, int has_id
 
 extern "C" int dsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
                             const int32_t *cu, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
-                            int dtype, int max_seqlen, void *out, float *lse, void *ws, size_t ws_bytes, void *stream) {
+                            int dtype, int max_seqlen, int causal, void *out, float *lse, void *ws, size_t ws_bytes,
+                            void *stream) {
     if (int rc = check_attn(T, N, cu, Hq, Hkv, D, K, dtype, idx, n)) return rc;
+    if (!causal && idx) return fail(DSA_ERR_ARG, "a key selection (idx) implies causal attention");
     if (!q || !k || !v || !out || !lse) return fail(DSA_ERR_ARG, "null tensor pointer");
     if (max_seqlen < 1 || max_seqlen > (T > 0 ? T : 1)) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
     if (T == 0) return DSA_OK;
@@ -179,7 +181,7 @@ extern "C" int dsa_attn_fwd(const void *q, const void *k, const void *v, const i
             e = dsa_launch_bitmap(idx, n, cu, N, T, K, ldw, bitmap, st);
             if (e != hipSuccess) return hip_fail(e, "bitmap launch");
         }
-        e = dsa_launch_tile_fwd(q, k, v, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, split, out, lse, st);
+        e = dsa_launch_tile_fwd(q, k, v, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, split, causal, out, lse, st);
         if (e != hipSuccess) return hip_fail(e, "tile forward launch");
     }
     if (max_seqlen > split) {
@@ -199,8 +201,10 @@ extern "C" size_t dsa_attn_bwd_workspace_bytes(int T, int Hq, int max_seqlen, in
 extern "C" int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k, const void *v, const void *out,
                                   const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu, int T,
                                   int N, int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen,
-                                  void *dq, void *dk, void *dv, void *ws, size_t ws_bytes, int parts, void *stream) {
+                                  int causal, void *dq, void *dk, void *dv, void *ws, size_t ws_bytes, int parts,
+                                  void *stream) {
     if (int rc = check_attn(T, N, cu, Hq, Hkv, D, K, dtype, idx, n)) return rc;
+    if (!causal && idx) return fail(DSA_ERR_ARG, "a key selection (idx) implies causal attention");
     if (!dout || !q || !k || !v || !out || !lse || !dq || !dk || !dv) return fail(DSA_ERR_ARG, "null tensor pointer");
     if (max_seqlen < 1 || max_seqlen > (T > 0 ? T : 1)) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
     if (T == 0) return DSA_OK;
@@ -223,7 +227,7 @@ extern "C" int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k
     }
     if (parts & DSA_BWD_DQ) {
         if (split > 0) {
-            e = dsa_launch_tile_dq(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, split, dq, st);
+            e = dsa_launch_tile_dq(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, split, causal, dq, st);
             if (e != hipSuccess) return hip_fail(e, "tile dq launch");
         }
         if (max_seqlen > split) {
@@ -232,7 +236,7 @@ extern "C" int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k
         }
     }
     if (parts & DSA_BWD_DKV) {
-        e = dsa_launch_tile_dkv(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, dk, dv, st);
+        e = dsa_launch_tile_dkv(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, causal, dk, dv, st);
         if (e != hipSuccess) return hip_fail(e, "tile dkv launch");
     }
     return DSA_OK;
@@ -240,8 +244,8 @@ extern "C" int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k
 
 extern "C" int dsa_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
                             const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu, int T, int N,
-                            int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen, void *dq,
-                            void *dk, void *dv, void *ws, size_t ws_bytes, void *stream) {
+                            int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen, int causal,
+                            void *dq, void *dk, void *dv, void *ws, size_t ws_bytes, void *stream) {
     return dsa_attn_bwd_parts(dout, q, k, v, out, lse, idx, n, cu, T, N, Hq, Hkv, D, K, softmax_scale, dtype, max_seqlen,
-                              dq, dk, dv, ws, ws_bytes, DSA_BWD_ALL, stream);
+                              causal, dq, dk, dv, ws, ws_bytes, DSA_BWD_ALL, stream);
 }

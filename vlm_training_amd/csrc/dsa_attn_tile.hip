@@ -140,7 +140,7 @@ template <int D, bool HAS_IDX, int GSHIFT>
 __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
     const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
-    float scale_log2, int pos_split, bf16_t *__restrict__ out, float *__restrict__ lse) {
+    float scale_log2, int pos_split, int causal, bf16_t *__restrict__ out, float *__restrict__ lse) {
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2, LOADS = 32 * CPR / 256;
     constexpr int NBUF = (D > 128) ? 1 : 2;           // double buffering where 64 KiB of static LDS allow it
     constexpr int Gp = 1 << GSHIFT, QBW = 128 >> GSHIFT;
@@ -163,7 +163,8 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
         qB[ks] = row_ok ? load_bf16x8(q + ((int64_t)t * Hq + hq) * D + 16 * ks + 8 * h) : zero_bf16x8();
-    const int ntiles = min(qc0 + QBW - 1, L - 1) / 32 + 1;
+    const int ntiles = (causal ? min(qc0 + QBW - 1, L - 1) : L - 1) / 32 + 1;
+    const int klim = causal ? qcol : L - 1;             // last key column this row may attend (dense mode)
     const uint32_t *wrow = bitmap + (int64_t)t * ldw;
 
     u32x4 kst[2][LOADS], vst[2][LOADS];
@@ -194,7 +195,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
         const unsigned char *kt = lds[BUF][0], *vt = lds[BUF][1];                                  \
         uint32_t word = row_ok ? word_next : 0u;                                                   \
         if (HAS_IDX) word_next = wrow[min((TILE) + 1, ntiles - 1)];                                \
-        if (!HAS_IDX) word = row_ok ? causal_bits(qcol - kc0) : 0u;                                \
+        if (!HAS_IDX) word = row_ok ? causal_bits(klim - kc0) : 0u;                                \
         word >>= 4 * h;                                  /* element vi then sits at bit 8*(vi/4) + vi%4 */ \
         f32x16 sacc = zero16();                                                                    \
         {                                                /* all K operands in flight before the first MFMA */ \
@@ -266,7 +267,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
     const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
-    float scale, int pos_split, bf16_t *__restrict__ dq) {
+    float scale, int pos_split, int causal, bf16_t *__restrict__ dq) {
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2, LOADS = 32 * CPR / 256;
     constexpr int NBUF = (D > 128) ? 1 : 2;
     constexpr int Gp = 1 << GSHIFT, QBW = 128 >> GSHIFT;
@@ -294,7 +295,8 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
     }
     const float lse2 = lse[(int64_t)hq * T + t] * LOG2E_F;
     const float dlt = delta[(int64_t)hq * T + t];
-    const int ntiles = min(qc0 + QBW - 1, L - 1) / 32 + 1;
+    const int ntiles = (causal ? min(qc0 + QBW - 1, L - 1) : L - 1) / 32 + 1;
+    const int klim = causal ? qcol : L - 1;             // last key column this row may attend (dense mode)
     const uint32_t *wrow = bitmap + (int64_t)t * ldw;
 
     u32x4 kst[2][LOADS], vst[2][LOADS];
@@ -324,7 +326,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
         const unsigned char *kt = lds[BUF][0], *vt = lds[BUF][1];                                  \
         uint32_t word = row_ok ? word_next : 0u;                                                   \
         if (HAS_IDX) word_next = wrow[min((TILE) + 1, ntiles - 1)];                                \
-        if (!HAS_IDX) word = row_ok ? causal_bits(qcol - kc0) : 0u;                                \
+        if (!HAS_IDX) word = row_ok ? causal_bits(klim - kc0) : 0u;                                \
         word >>= 4 * h;                                                                            \
         f32x16 sacc = zero16(), pacc = zero16();                                                   \
         _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
@@ -378,7 +380,7 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
     const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
-    float scale, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    float scale, int causal, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2, LOADS = 32 * CPR / 256;
     constexpr int NBUF = (D > 128) ? 1 : 2;
     constexpr int Gp = 1 << GSHIFT, QB = 32 >> GSHIFT;                           // queries per block
@@ -405,7 +407,8 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) { dkacc[dt] = zero16(); dvacc[dt] = zero16(); }
     const float scale_log2 = scale * LOG2E_F;
-    const int nblocks = (L - c0 + QB - 1) / QB;          // queries c0 .. L-1
+    const int q0 = causal ? c0 : 0;                      // first query column that can see this key tile
+    const int nblocks = (L - q0 + QB - 1) / QB;          // queries q0 .. L-1
 
     u32x4 qst[2][LOADS], dost[2][LOADS];
     // Per-block side data, one 32-bit word per staging thread, loaded raw and interpreted at STORE time:
@@ -431,7 +434,7 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
     uint32_t aux_st[2] = {0u, 0u};
 #define DKV_LOAD(SET, BLK)                                                                          \
     {                                                                                              \
-        const int qcb = c0 + (BLK) * QB;                                                           \
+        const int qcb = q0 + (BLK) * QB;                                                           \
         _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                        \
             const int c = i * 256 + tid;                                                           \
             const int row = c / CPR, ch = c % CPR;                                                 \
@@ -445,7 +448,7 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
     }
 #define DKV_STORE(SET, BUF, BLK)                                                                    \
     {                                                                                              \
-        const int qcb = c0 + (BLK) * QB;                                                           \
+        const int qcb = q0 + (BLK) * QB;                                                           \
         const u32x4 z4 = {0u, 0u, 0u, 0u};                                                         \
         _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                        \
             const int c = i * 256 + tid;                                                           \
@@ -462,7 +465,7 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
     }
 #define DKV_COMPUTE(BLK, BUF)                                                                       \
     {                                                                                              \
-        const int qcb = c0 + (BLK) * QB;                                                           \
+        const int qcb = q0 + (BLK) * QB;                                                           \
         const unsigned char *qt = lds[BUF][0], *dot = lds[BUF][1];                                 \
         f32x16 sacc = zero16(), pacc = zero16();                                                   \
         _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
@@ -470,7 +473,7 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
             pacc = mfma32(tile_rowop<D>(dot, j, ks, h), vB[ks], pacc);                             \
         }                                                                                          \
         float pv[16], dsv[16];                                                                     \
-        const bool diag = qcb < kc + 32;                /* wave-uniform: block touches the diagonal */ \
+        const bool diag = causal && qcb < kc + 32;      /* wave-uniform: block touches the diagonal */ \
         _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {                                         \
             const f32x4 l4 = *reinterpret_cast<const f32x4 *>(&lse_s[BUF][8 * g4 + 4 * h]);        \
             const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&dlt_s[BUF][8 * g4 + 4 * h]);        \
@@ -530,7 +533,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv8_kernel(
     const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
-    float scale, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    float scale, int causal, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2;
     constexpr int NCHUNK = 32 * CPR;                     // 16-byte chunks per staged operand (<= 512 threads)
     constexpr int NBUF = 2;
@@ -560,7 +563,8 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv8_kernel(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
     const float scale_log2 = scale * LOG2E_F;
-    const int nblocks = (L - c0 + QB - 1) / QB;          // queries c0 .. L-1
+    const int q0 = causal ? c0 : 0;                      // first query column that can see this key tile
+    const int nblocks = (L - q0 + QB - 1) / QB;          // queries q0 .. L-1
     const bool stager = tid < NCHUNK;
     const int srow = (tid % NCHUNK) / CPR, sch = tid % CPR;   // non-staging threads re-read a staged chunk and drop it
 
@@ -588,7 +592,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv8_kernel(
     uint32_t aux_st[2] = {0u, 0u};
 #define DKV8_LOAD(SET, BLK)                                                                         \
     {                                                                                              \
-        const int qcb = c0 + (BLK) * QB;                                                           \
+        const int qcb = q0 + (BLK) * QB;                                                           \
         const int qc = min(qcb + (srow >> GSHIFT), L - 1);                                         \
         const int hd = min(srow & (Gp - 1), G - 1);                                                \
         const int64_t off = ((int64_t)(s0 + qc) * Hq + kvh * G + hd) * D + sch * 8;                \
@@ -598,7 +602,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv8_kernel(
     }
 #define DKV8_STORE(SET, BUF, BLK)                                                                   \
     {                                                                                              \
-        const int qcb = c0 + (BLK) * QB;                                                           \
+        const int qcb = q0 + (BLK) * QB;                                                           \
         if (stager) {                                                                              \
             /* rows past the segment and padded heads are zeroed: they add nothing to dK, dV */     \
             const bool live = qcb + (srow >> GSHIFT) < L && (srow & (Gp - 1)) < G;                 \
@@ -613,7 +617,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv8_kernel(
     }
 #define DKV8_COMPUTE(BLK, BUF)                                                                      \
     {                                                                                              \
-        const int qcb = c0 + (BLK) * QB;                                                           \
+        const int qcb = q0 + (BLK) * QB;                                                           \
         const unsigned char *qt = lds[BUF][0], *dot = lds[BUF][1];                                 \
         const unsigned char *t2 = role ? qt : dot;      /* operand of the second GEMM */            \
         f32x16 sacc = zero16(), pacc = zero16();                                                   \
@@ -626,7 +630,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv8_kernel(
             sched_reads_ahead<KS, 4, 1>();                                                         \
         }                                                                                          \
         float bv[16];                                                                              \
-        const bool diag = qcb < kc + 32;                /* wave-uniform: block touches the diagonal */ \
+        const bool diag = causal && qcb < kc + 32;      /* wave-uniform: block touches the diagonal */ \
         _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {                                         \
             const f32x4 l4 = *reinterpret_cast<const f32x4 *>(&lse_s[BUF][8 * g4 + 4 * h]);        \
             const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&dlt_s[BUF][8 * g4 + 4 * h]);        \
@@ -683,30 +687,30 @@ static inline int group_shift(int Hq, int Hkv) {
 template <int D, bool HAS_IDX, int GS>
 static void launch_fwd_i(dim3 grid, hipStream_t stream, const void *q, const void *k, const void *v,
                          const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T, int Hq, int Hkv, float sl2,
-                         int pos_split, void *out, float *lse) {
+                         int pos_split, int causal, void *out, float *lse) {
     hipLaunchKernelGGL((dsa_tile_fwd_kernel<D, HAS_IDX, GS>), grid, dim3(256), 0, stream, (const bf16_t *)q,
-                       (const bf16_t *)k, (const bf16_t *)v, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, pos_split, (bf16_t *)out, lse);
+                       (const bf16_t *)k, (const bf16_t *)v, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, pos_split, causal, (bf16_t *)out, lse);
 }
 template <int D, bool HAS_IDX, int GS>
 static void launch_dq_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
                         const float *lse, const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N,
-                        int T, int Hq, int Hkv, float scale, int pos_split, void *dq) {
+                        int T, int Hq, int Hkv, float scale, int pos_split, int causal, void *dq) {
     hipLaunchKernelGGL((dsa_tile_dq_kernel<D, HAS_IDX, GS>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
                        (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv,
-                       scale, pos_split, (bf16_t *)dq);
+                       scale, pos_split, causal, (bf16_t *)dq);
 }
 template <int D, bool HAS_IDX, int GS>
 static void launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
                          const float *lse, const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N,
-                         int T, int Hq, int Hkv, float scale, void *dk, void *dv) {
+                         int T, int Hq, int Hkv, float scale, int causal, void *dk, void *dv) {
     if constexpr (D <= 128)
         hipLaunchKernelGGL((dsa_tile_dkv8_kernel<D, HAS_IDX, GS>), grid, dim3(512), 0, stream, (const bf16_t *)dout,
                            (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T, Hq,
-                           Hkv, scale, (bf16_t *)dk, (bf16_t *)dv);
+                           Hkv, scale, causal, (bf16_t *)dk, (bf16_t *)dv);
     else
         hipLaunchKernelGGL((dsa_tile_dkv_kernel<D, HAS_IDX, GS>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
                            (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T, Hq,
-                           Hkv, scale, (bf16_t *)dk, (bf16_t *)dv);
+                           Hkv, scale, causal, (bf16_t *)dk, (bf16_t *)dv);
 }
 
 #define GS_SWITCH(FN, DD, HI, ...)                                    \
@@ -727,27 +731,27 @@ static void launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, const 
 
 extern "C" hipError_t dsa_launch_tile_fwd(const void *q, const void *k, const void *v, const uint32_t *bitmap, int ldw,
                                           const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale,
-                                          int pos_split, void *out, float *lse, hipStream_t stream) {
+                                          int pos_split, int causal, void *out, float *lse, hipStream_t stream) {
     const int gs = group_shift(Hq, Hkv);
     const dim3 grid((unsigned)(((int64_t)T / (128 >> gs) + N + 1) * Hkv));
-    TILE_SWITCH(launch_fwd_i, grid, stream, q, k, v, bitmap, ldw, cu, N, T, Hq, Hkv, scale * LOG2E_F, pos_split, out, lse)
+    TILE_SWITCH(launch_fwd_i, grid, stream, q, k, v, bitmap, ldw, cu, N, T, Hq, Hkv, scale * LOG2E_F, pos_split, causal, out, lse)
     return hipGetLastError();
 }
 extern "C" hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const void *k, const void *v,
                                          const float *lse, const float *delta, const uint32_t *bitmap, int ldw,
                                          const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale,
-                                         int pos_split, void *dq, hipStream_t stream) {
+                                         int pos_split, int causal, void *dq, hipStream_t stream) {
     const int gs = group_shift(Hq, Hkv);
     const dim3 grid((unsigned)(((int64_t)T / (128 >> gs) + N + 1) * Hkv));
-    TILE_SWITCH(launch_dq_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, pos_split, dq)
+    TILE_SWITCH(launch_dq_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, pos_split, causal, dq)
     return hipGetLastError();
 }
 extern "C" hipError_t dsa_launch_tile_dkv(const void *dout, const void *q, const void *k, const void *v,
                                           const float *lse, const float *delta, const uint32_t *bitmap, int ldw,
-                                          const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale, void *dk,
-                                          void *dv, hipStream_t stream) {
+                                          const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale, int causal,
+                                          void *dk, void *dv, hipStream_t stream) {
     const int gs = group_shift(Hq, Hkv);
     const dim3 grid((unsigned)(((int64_t)T / 128 + N + 1) * Hkv));
-    TILE_SWITCH(launch_dkv_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, dk, dv)
+    TILE_SWITCH(launch_dkv_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, causal, dk, dv)
     return hipGetLastError();
 }

@@ -36,11 +36,9 @@ def varlen_attn(query, key, value, cu_seq_q, cu_seq_k, max_q, max_k, is_causal=N
         causal = right == 0
     else:
         causal = True if is_causal is None else bool(is_causal)
-    if not causal:
-        raise NotImplementedError("non-causal (vision tower) packed attention is not built yet")
     if return_aux is not None:
         raise NotImplementedError("return_aux is not supported")
-    return dsa_varlen_attn(query, key, value, cu_seq_q, int(max_q), softmax_scale=scale, **dsa)
+    return dsa_varlen_attn(query, key, value, cu_seq_q, int(max_q), softmax_scale=scale, causal=causal, **dsa)
 
 
 def dispatch_varlen_attention(q, k, v, cu_seqlens, max_seqlen, causal: bool = True, **dsa):

@@ -128,7 +128,7 @@ def set_tile_crossover(crossover: int) -> int:
     return old
 
 
-def attn_fwd(q, k, v, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float):
+def attn_fwd(q, k, v, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float, causal: bool = True):
     T, Hq, Hkv, D = _check_qkv(q, k, v)
     cu = _check_cu(cu_seqlens, T)
     out = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=q.device)
@@ -138,14 +138,14 @@ def attn_fwd(q, k, v, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float)
     ws_bytes = lib.dsa_attn_fwd_workspace_bytes(T, max_seqlen, 1 if idx is not None else 0)
     ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q.device)
     rc = lib.dsa_attn_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(idx), _ptr(n), _ptr(cu), T, cu.numel() - 1, Hq, Hkv, D, K,
-                          softmax_scale, _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
+                          softmax_scale, _lib.DSA_DTYPE_BF16, max_seqlen, 1 if causal else 0, _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
                           _stream(q.device))
     _lib.check(rc, "dsa_attn_fwd")
     return out, lse
 
 
 def attn_bwd(dout, q, k, v, out, lse, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float,
-             parts: int = 15, buffers=None):
+             parts: int = 15, buffers=None, causal: bool = True):
     """Stage D4.  ``parts``/``buffers`` exist for per-kernel timing: ``buffers=(dq, dk, dv, ws)`` reuses
     the outputs and workspace of an earlier full call."""
     T, Hq, Hkv, D = _check_qkv(q, k, v)
@@ -160,7 +160,8 @@ def attn_bwd(dout, q, k, v, out, lse, idx, n, cu_seqlens, max_seqlen: int, softm
         dq, dk, dv, ws = buffers
     rc = lib.dsa_attn_bwd_parts(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(idx), _ptr(n),
                                 _ptr(cu), T, cu.numel() - 1, Hq, Hkv, D, K, softmax_scale, _lib.DSA_DTYPE_BF16,
-                                max_seqlen, _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), ws_bytes, parts, _stream(q.device))
+                                max_seqlen, 1 if causal else 0, _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), ws_bytes, parts,
+                                _stream(q.device))
     _lib.check(rc, "dsa_attn_bwd")
     return (dq, dk, dv) if buffers is None else (dq, dk, dv, ws)
 
@@ -190,7 +191,7 @@ class _DsaVarlenAttn(torch.autograd.Function):
     Other dtypes / larger head_dim are rounded to bf16 once."""
 
     @staticmethod
-    def forward(ctx, q, k, v, cu_seqlens, max_seqlen, idx, n, softmax_scale):
+    def forward(ctx, q, k, v, cu_seqlens, max_seqlen, idx, n, softmax_scale, causal=True):
         in_dtype = q.dtype
         D = q.shape[-1]
         split = in_dtype == torch.float32 and 4 * D <= 256
@@ -199,7 +200,8 @@ class _DsaVarlenAttn(torch.autograd.Function):
             qb, kb, vb = _stack((qh, ql, qh), D), _stack((kh, kh, kl), D), _stack((vh, vl, vh), D)
         else:
             qb, kb, vb = _as_bf16(q), _as_bf16(k), _as_bf16(v)
-        out, lse = attn_fwd(qb, kb, vb, idx, n, cu_seqlens, int(max_seqlen), softmax_scale)
+        out, lse = attn_fwd(qb, kb, vb, idx, n, cu_seqlens, int(max_seqlen), softmax_scale, causal)
+        ctx.causal = bool(causal)
         ctx.save_for_backward(qb, kb, vb, out, lse, cu_seqlens, *(() if idx is None else (idx, n)))
         ctx.has_idx = idx is not None
         ctx.max_seqlen = int(max_seqlen)
@@ -222,19 +224,20 @@ class _DsaVarlenAttn(torch.autograd.Function):
             db = _stack((gh, gh, gl), D)
         else:
             db = _as_bf16(dout)
-        dq, dk, dv = attn_bwd(db, qb, kb, vb, out, lse, idx, n, cu, ctx.max_seqlen, ctx.softmax_scale)
+        dq, dk, dv = attn_bwd(db, qb, kb, vb, out, lse, idx, n, cu, ctx.max_seqlen, ctx.softmax_scale,
+                              causal=ctx.causal)
         if ctx.split:
             dq = dq[..., :D].float() + dq[..., 2 * D:3 * D].float()
             dk = dk[..., :D].float() + dk[..., D:2 * D].float()
             dv = dv[..., :D].float() + dv[..., 2 * D:3 * D].float()
         elif ctx.in_dtype != torch.bfloat16:
             dq, dk, dv = dq.to(ctx.in_dtype), dk.to(ctx.in_dtype), dv.to(ctx.in_dtype)
-        return dq, dk, dv, None, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None, None
 
 
 def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: int, *, indexer_q=None, indexer_k=None, indexer_w=None,
                     top_k: Optional[int] = None, index_scale: Optional[float] = None,
-                    softmax_scale: Optional[float] = None, return_indices: bool = False):
+                    softmax_scale: Optional[float] = None, return_indices: bool = False, causal: bool = True):
     """Packed causal attention over ``cu_seqlens`` segments, optionally sparsified by the DSA indexer.
 
     q (T,Hq,D), k/v (T,Hkv,D) contiguous, cu_seqlens (N+1,) int32 on the device, max_seqlen host int
@@ -242,7 +245,8 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: int, *, indexer_q=None, ind
     every causal key of the token's own segment is attended (the reference's behaviour).  With
     ``indexer_q (T,Hi,Di)``, ``indexer_k (T,Di)``, ``indexer_w (T,Hi)`` and ``top_k`` each query keeps
     the top_k keys of its causal window under (indexer score descending, key index ascending).
-    Gradients flow to q, k, v only.
+    Gradients flow to q, k, v only.  ``causal=False`` (dense only) attends every key of the own segment, the
+    vision towers' form of the call (models/qwen3_vl/model.py:423-428).
     """
     _require_cuda(q, k, v, cu_seqlens)
     T, Hq, Hkv, D = _check_qkv(q, k, v)
@@ -250,6 +254,8 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: int, *, indexer_q=None, ind
     scale = float(softmax_scale) if softmax_scale is not None else D ** -0.5
     sparse = indexer_q is not None or indexer_k is not None or indexer_w is not None
     idx = n = None
+    if sparse and not causal:
+        raise ValueError("DSA key selection is defined for causal attention only")
     if sparse:
         if indexer_q is None or indexer_k is None or indexer_w is None or top_k is None:
             raise ValueError("DSA needs indexer_q, indexer_k, indexer_w and top_k together")
@@ -259,5 +265,6 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: int, *, indexer_q=None, ind
             idx, n = index_topk(indexer_q, indexer_k, indexer_w, cu, int(max_seqlen), int(top_k), index_scale)
     elif return_indices:
         raise ValueError("return_indices needs the indexer inputs")
-    out = _DsaVarlenAttn.apply(q.contiguous(), k.contiguous(), v.contiguous(), cu, int(max_seqlen), idx, n, scale)
+    out = _DsaVarlenAttn.apply(q.contiguous(), k.contiguous(), v.contiguous(), cu, int(max_seqlen), idx, n, scale,
+                               bool(causal))
     return (out, idx, n) if return_indices else out
