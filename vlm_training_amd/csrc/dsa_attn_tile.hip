@@ -675,6 +675,204 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv8_kernel(
 }
 
 // ==================================================================================================
+// dK, dV for head_dim <= 128, producer/consumer form.  A workgroup owns a 128-key tile (4 groups of 32
+// keys) of one segment and kv head and walks the later queries in blocks of 32 (query, head) rows.
+//   waves 0-3 (producers, one per key group): S = Q K^T and dP = dO V^T against the group's K / V rows
+//     held in registers, then P and dS = P * (dP - delta) in bf16, written to LDS in MFMA B layout;
+//   waves 4-7 (consumers, one per key group): dV^T += dO^T P and dK^T += Q^T dS for the previous block,
+//     A operands read transposed from the staged q / dO block, B operands read back from LDS.
+// Producer w and consumer w+4 share a SIMD: the softmax arithmetic of one overlaps the MFMAs of the
+// other, nothing is computed twice (32 MFMAs per 32x32 block pair), each wave stays under 256 registers.
+// LDS (dynamic, ~85 KiB): q/dO blocks in a ring of three (block b+1 being staged, b read row-wise by
+// the producers, b-1 read transposed by the consumers), P/dS in a ring of two.  One barrier per block.
+// ==================================================================================================
+template <int D, bool HAS_IDX, int GSHIFT>
+__global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
+    const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
+    const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
+    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
+    float scale, int causal, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2;
+    constexpr int NCHUNK = 32 * CPR;                     // 16-byte chunks per staged operand (<= 512)
+    constexpr int Gp = 1 << GSHIFT, QB = 32 >> GSHIFT;
+    constexpr int QD_SLOT = 2 * TILE_B;                  // q block | dO block
+    constexpr int PD_SLOT = 4 * 4 * 1024;                // 4 key groups x {P lo, P hi, dS lo, dS hi} x 64 lanes x 16 B
+    constexpr int AUX_SLOT = (32 + 32 + 4 * 32) * 4;     // lse | delta | selection words [key group][query]
+    static_assert(NCHUNK <= 512, "one chunk per thread");
+    extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
+    unsigned char *const qd_ring = dyn_lds;                          // 3 slots
+    unsigned char *const pd_ring = dyn_lds + 3 * QD_SLOT;            // 2 slots
+    unsigned char *const aux_ring = pd_ring + 2 * PD_SLOT;           // 3 slots
+
+    const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5, j = lane & 31;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);         // wave-uniform for the compiler too
+    const int kg = wv & 3;
+    const bool consumer = wv >= 4;
+    const int G = Hq / Hkv;
+    const int kvh = blockIdx.x % Hkv;
+    int s0, L, blk;
+    if (!locate_block(cu, N, blockIdx.x / Hkv, 128, false, s0, L, blk)) return;
+    const int c0 = blk * 128, kc = c0 + kg * 32;
+    const int mykey = kc + j;
+    const bool key_ok = mykey < L;
+    const int64_t krow = (int64_t)(s0 + min(mykey, L - 1)) * Hkv + kvh;
+    const float scale_log2 = scale * LOG2E_F;
+    const int q0 = causal ? c0 : 0;                      // first query column that can see this key tile
+    const int nblocks = (L - q0 + QB - 1) / QB;          // queries q0 .. L-1
+
+    // ---- staging (all 512 threads): one 16-byte chunk of q and of dO per block, one side word ----------
+    const bool stager = tid < NCHUNK;
+    const int srow = (tid % NCHUNK) / CPR, sch = tid % CPR;
+    const uint32_t *aux_base;
+    int aux_q = 0, aux_stride = 1;
+    bool aux_mask_ok = false;
+    if (tid < 64) {                                      // 0..31: lse of row tid, 32..63: delta of row tid-32
+        const int row = tid & 31;
+        const int hd = min(row & (Gp - 1), G - 1);
+        aux_q = row >> GSHIFT;
+        aux_base = reinterpret_cast<const uint32_t *>((tid < 32 ? lse : delta) + (int64_t)(kvh * G + hd) * T + s0);
+    } else if (HAS_IDX && tid < 64 + 4 * QB) {           // selection word of (key group w, query qi)
+        const int w = (tid - 64) / QB;
+        aux_q = (tid - 64) % QB;
+        aux_stride = ldw;
+        aux_mask_ok = (c0 >> 5) + w < ldw;
+        aux_base = bitmap + (int64_t)s0 * ldw + (aux_mask_ok ? (c0 >> 5) + w : 0);
+    } else {
+        aux_base = reinterpret_cast<const uint32_t *>(lse);
+    }
+    u32x4 qst, dost;
+    uint32_t aux_st;
+    auto gload = [&](int b) {                            // block index clamped by the caller
+        const int qcb = q0 + b * QB;
+        const int qc = min(qcb + (srow >> GSHIFT), L - 1);
+        const int hd = min(srow & (Gp - 1), G - 1);
+        const int64_t off = ((int64_t)(s0 + qc) * Hq + kvh * G + hd) * D + sch * 8;
+        qst = *reinterpret_cast<const u32x4 *>(q + off);
+        dost = *reinterpret_cast<const u32x4 *>(dout + off);
+        aux_st = aux_base[(int64_t)aux_stride * min(qcb + aux_q, L - 1)];
+    };
+    auto lstore = [&](int b) {                           // registers -> ring slot b % 3
+        const int qcb = q0 + b * QB;
+        unsigned char *slot = qd_ring + (b % 3) * QD_SLOT;
+        float *lse_s = reinterpret_cast<float *>(aux_ring + (b % 3) * AUX_SLOT);
+        float *dlt_s = lse_s + 32;
+        uint32_t *mask_s = reinterpret_cast<uint32_t *>(dlt_s + 32);
+        if (stager) {
+            // rows past the segment and padded heads are zeroed: they add nothing to dK, dV
+            const bool live = qcb + (srow >> GSHIFT) < L && (srow & (Gp - 1)) < G;
+            const u32x4 z4 = {0u, 0u, 0u, 0u};
+            *reinterpret_cast<u32x4 *>(slot + tile_off<D>(srow, sch)) = live ? qst : z4;
+            *reinterpret_cast<u32x4 *>(slot + TILE_B + tile_off<D>(srow, sch)) = live ? dost : z4;
+        }
+        if (tid < 32) lse_s[tid] = __uint_as_float(aux_st) * LOG2E_F;
+        else if (tid < 64) dlt_s[tid - 32] = __uint_as_float(aux_st);
+        else if (HAS_IDX && tid < 64 + 4 * QB)
+            mask_s[((tid - 64) / QB) * 32 + (tid - 64) % QB] = (aux_mask_ok && qcb + aux_q < L) ? aux_st : 0u;
+    };
+
+    gload(0);
+    lstore(0);
+    gload(min(1, nblocks - 1));
+    __syncthreads();
+
+    if (!consumer) {
+        // ================= producer: P and dS of block b into the P/dS ring =================
+        bf16x8 kB[KS], vB[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            kB[ks] = load_bf16x8(k + krow * D + 16 * ks + 8 * h);
+            vB[ks] = load_bf16x8(v + krow * D + 16 * ks + 8 * h);
+        }
+        for (int b = 0; b <= nblocks; ++b) {
+            lstore(b + 1);                               // registers hold block b+1; slot (b+1)%3 is free since the last barrier
+            gload(min(b + 2, nblocks - 1));
+            if (b < nblocks) {
+                const int qcb = q0 + b * QB;
+                const unsigned char *qt = qd_ring + (b % 3) * QD_SLOT, *dot = qt + TILE_B;
+                const float *lse_s = reinterpret_cast<const float *>(aux_ring + (b % 3) * AUX_SLOT);
+                const float *dlt_s = lse_s + 32;
+                const uint32_t *mask_s = reinterpret_cast<const uint32_t *>(dlt_s + 32) + kg * 32;
+                f32x16 sacc = zero16(), pacc = zero16();
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    sacc = mfma32(tile_rowop<D>(qt, j, ks, h), kB[ks], sacc);
+                    pacc = mfma32(tile_rowop<D>(dot, j, ks, h), vB[ks], pacc);
+                }
+                sched_reads_ahead<2 * KS, 4, 1>();
+                float pv[16], dsv[16];
+                const bool diag = causal && qcb < kc + 32;   // wave-uniform: block touches the diagonal
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const f32x4 l4 = *reinterpret_cast<const f32x4 *>(&lse_s[8 * g4 + 4 * h]);
+                    const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&dlt_s[8 * g4 + 4 * h]);
+                    uint32_t keep = 0u;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int vi = 4 * g4 + e, row = 8 * g4 + 4 * h + e;
+                        if (e == 0 || GSHIFT < 2) {          // rows of one query share the mask bit
+                            const int qi = row >> GSHIFT;
+                            uint32_t mw = HAS_IDX ? mask_s[qi] : 0xffffffffu;
+                            if (diag) mw &= causal_bits(qcb + qi - kc);
+                            keep = bit_mask(mw, j);
+                        }
+                        const float p = fast_exp2(keep_or_neginf(fmaf(sacc[vi], scale_log2, -l4[e]), keep));
+                        pv[vi] = p;
+                        dsv[vi] = p * (pacc[vi] - d4[e]);
+                    }
+                }
+                unsigned char *pd = pd_ring + (b & 1) * PD_SLOT + kg * 4096 + lane * 16;
+                *reinterpret_cast<bf16x8 *>(pd) = pack8(pv);
+                *reinterpret_cast<bf16x8 *>(pd + 1024) = pack8(pv + 8);
+                *reinterpret_cast<bf16x8 *>(pd + 2048) = pack8(dsv);
+                *reinterpret_cast<bf16x8 *>(pd + 3072) = pack8(dsv + 8);
+            }
+            __syncthreads();
+        }
+    } else {
+        // ================= consumer: dV^T, dK^T of block b-1 =================
+        f32x16 dkacc[DT], dvacc[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) { dkacc[dt] = zero16(); dvacc[dt] = zero16(); }
+        for (int b = 0; b <= nblocks; ++b) {
+            lstore(b + 1);
+            gload(min(b + 2, nblocks - 1));
+            if (b >= 1) {
+                const unsigned char *qt = qd_ring + ((b - 1) % 3) * QD_SLOT, *dot = qt + TILE_B;
+                const unsigned char *pd = pd_ring + ((b - 1) & 1) * PD_SLOT + kg * 4096 + lane * 16;
+                const bf16x8 pB0 = *reinterpret_cast<const bf16x8 *>(pd), pB1 = *reinterpret_cast<const bf16x8 *>(pd + 1024);
+                const bf16x8 dB0 = *reinterpret_cast<const bf16x8 *>(pd + 2048), dB1 = *reinterpret_cast<const bf16x8 *>(pd + 3072);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;
+                    dvacc[dt] = mfma32(tile_trop<D>(dot, 4 * h, m0, lane), pB0, dvacc[dt]);
+                    dvacc[dt] = mfma32(tile_trop<D>(dot, 16 + 4 * h, m0, lane), pB1, dvacc[dt]);
+                    dkacc[dt] = mfma32(tile_trop<D>(qt, 4 * h, m0, lane), dB0, dkacc[dt]);
+                    dkacc[dt] = mfma32(tile_trop<D>(qt, 16 + 4 * h, m0, lane), dB1, dkacc[dt]);
+                }
+                sched_reads_ahead<4 * DT, 3, 2>();
+            }
+            __syncthreads();
+        }
+        if (key_ok) {
+            bf16_t *pk = dk + krow * D + 4 * h, *pv_ = dv + krow * D + 4 * h;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const u32x2 wk = {pack2bf(dkacc[dt][4 * g4] * scale, dkacc[dt][4 * g4 + 1] * scale),
+                                      pack2bf(dkacc[dt][4 * g4 + 2] * scale, dkacc[dt][4 * g4 + 3] * scale)};
+                    const u32x2 wvv = {pack2bf(dvacc[dt][4 * g4], dvacc[dt][4 * g4 + 1]),
+                                       pack2bf(dvacc[dt][4 * g4 + 2], dvacc[dt][4 * g4 + 3])};
+                    *reinterpret_cast<u32x2 *>(pk + dt * 32 + 8 * g4) = wk;
+                    *reinterpret_cast<u32x2 *>(pv_ + dt * 32 + 8 * g4) = wvv;
+                }
+        }
+    }
+}
+template <int D>
+constexpr size_t dkvpc_lds_bytes() { return 3 * (2 * 32 * D * 2) + 2 * (4 * 4 * 1024) + 3 * ((32 + 32 + 4 * 32) * 4); }
+
+// ==================================================================================================
 // launchers: instantiate per head_dim, mask kind and (power-of-two padded) group size
 // ==================================================================================================
 static inline int group_shift(int Hq, int Hkv) {
@@ -703,10 +901,17 @@ template <int D, bool HAS_IDX, int GS>
 static void launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
                          const float *lse, const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N,
                          int T, int Hq, int Hkv, float scale, int causal, void *dk, void *dv) {
-    if constexpr (D <= 128)
-        hipLaunchKernelGGL((dsa_tile_dkv8_kernel<D, HAS_IDX, GS>), grid, dim3(512), 0, stream, (const bf16_t *)dout,
-                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T, Hq,
-                           Hkv, scale, causal, (bf16_t *)dk, (bf16_t *)dv);
+    if constexpr (D <= 128) {
+        static bool configured = false;                  // LDS above 64 KiB has to be requested once per kernel
+        if (!configured) {
+            hipFuncSetAttribute(reinterpret_cast<const void *>(&dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkvpc_lds_bytes<D>());
+            configured = true;
+        }
+        hipLaunchKernelGGL((dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>), grid, dim3(512), dkvpc_lds_bytes<D>(), stream,
+                           (const bf16_t *)dout, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap,
+                           ldw, cu, N, T, Hq, Hkv, scale, causal, (bf16_t *)dk, (bf16_t *)dv);
+    }
     else
         hipLaunchKernelGGL((dsa_tile_dkv_kernel<D, HAS_IDX, GS>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
                            (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T, Hq,
