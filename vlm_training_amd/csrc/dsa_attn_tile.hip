@@ -68,6 +68,55 @@ __device__ __forceinline__ void sched_reads_ahead() {
     }
     __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
 }
+// Per-lane LDS byte offsets of the two read patterns, computed once per kernel so that every operand
+// read in the loops is "tile base + lane offset + immediate" (the swizzle only XORs chunk bits 0-2, so
+// k-step / d-tile indices move the address by a lane constant plus a compile-time multiple of 128 B).
+typedef __attribute__((address_space(3))) unsigned char lds_u8;
+template <int D>
+struct LaneOffsets {
+    int row[4];      // row-wise operand of row j: k-steps ks with ks % 4 == c
+    int tr_e[4];     // transposed operand, even d-tiles: rows 4h + s/4 + {0, 8, 16, 24}
+    int tr_o[4];     // same for odd d-tiles
+    __device__ __forceinline__ void init(int lane) {
+        const int h = lane >> 5, j = lane & 31, s = lane & 15;
+        const int swj = tile_sw(j);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) row[c] = j * (D * 2) + ((((c ^ (swj >> 1)) << 1) | (h ^ (swj & 1))) << 4);
+        const int low = ((lane >> 4) & 1) * 2 + ((s & 3) >> 1), sub = (s & 1) << 3;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int r = 4 * h + (s >> 2) + 8 * v, sw = tile_sw(r);
+            const int lo = low ^ (sw & 3), f = sw & 4;
+            tr_e[v] = r * (D * 2) + ((lo | f) << 4) + sub;
+            tr_o[v] = r * (D * 2) + ((lo | (4 ^ f)) << 4) + sub;
+        }
+    }
+    // row-wise A operand of k-step ks (elements [16ks + 8h, +8) of row j)
+    __device__ __forceinline__ bf16x8 rowop(const unsigned char *tile, int ks) const {
+        return *reinterpret_cast<const bf16x8 *>(tile + row[ks & 3] + (ks >> 2) * 128);
+    }
+    // same with the lane addresses already formed (pe/po = tile + tr_e/tr_o): one immediate per read
+    __device__ __forceinline__ static bf16x8 trop_at(lds_u8 *const *pe, lds_u8 *const *po, int pair, int dt, int imm) {
+        lds_u8 *const *t = (dt & 1) ? po : pe;
+        lds_u8 *p0 = t[2 * pair] + (dt >> 1) * 128 + imm, *p1 = t[2 * pair + 1] + (dt >> 1) * 128 + imm;
+        const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p0);
+        const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p1);
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        const s16x8 r = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+        return __builtin_bit_cast(bf16x8, r);
+    }
+    // transposed A operand of d-tile dt over rows {R..R+3, R+8..R+11}, R = 4h (pair 0) or 16 + 4h (pair 1)
+    __device__ __forceinline__ bf16x8 trop(const unsigned char *tile, int pair, int dt) const {
+        const int *t = (dt & 1) ? tr_o : tr_e;
+        const unsigned char *p0 = tile + t[2 * pair] + (dt >> 1) * 128;
+        const unsigned char *p1 = tile + t[2 * pair + 1] + (dt >> 1) * 128;
+        const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p0);
+        const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p1);
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        const s16x8 r = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+        return __builtin_bit_cast(bf16x8, r);
+    }
+};
 __device__ __forceinline__ bf16x8 pack8(const float *x) {
     const u32x4 w = {pack2bf(x[0], x[1]), pack2bf(x[2], x[3]), pack2bf(x[4], x[5]), pack2bf(x[6], x[7])};
     return __builtin_bit_cast(bf16x8, w);
@@ -148,6 +197,8 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
     __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];   // [buffer][K|V]
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
+    LaneOffsets<D> lo;
+    lo.init(lane);
     const int G = Hq / Hkv;
     const int kvh = blockIdx.x % Hkv;
     int s0, L, blk;
@@ -200,7 +251,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
         f32x16 sacc = zero16();                                                                    \
         {                                                /* all K operands in flight before the first MFMA */ \
             bf16x8 ka[KS];                                                                         \
-            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) ka[ks] = tile_rowop<D>(kt, j, ks, h); \
+            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) ka[ks] = lo.rowop(kt, ks); \
             _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) sacc = mfma32(ka[ks], qB[ks], sacc); \
             sched_reads_ahead<KS, 4, 1>();                                                         \
         }                                                                                          \
@@ -229,9 +280,8 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
         lsum += psum;                                                                              \
         const bf16x8 pB0 = pack8(s2), pB1 = pack8(s2 + 8);                                         \
         _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
-            const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;                                       \
-            mfma32_acc(oacc[dt], tile_trop<D>(vt, 4 * h, m0, lane), pB0);                          \
-            mfma32_acc(oacc[dt], tile_trop<D>(vt, 16 + 4 * h, m0, lane), pB1);                     \
+            mfma32_acc(oacc[dt], lo.trop(vt, 0, dt), pB0);                          \
+            mfma32_acc(oacc[dt], lo.trop(vt, 1, dt), pB1);                     \
         }                                                                                          \
         sched_reads_ahead<2 * DT, 3, 2>();                                                         \
     }
@@ -274,6 +324,8 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
     __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
+    LaneOffsets<D> lo;
+    lo.init(lane);
     const int G = Hq / Hkv;
     const int kvh = blockIdx.x % Hkv;
     int s0, L, blk;
@@ -330,8 +382,8 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
         word >>= 4 * h;                                                                            \
         f32x16 sacc = zero16(), pacc = zero16();                                                   \
         _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
-            sacc = mfma32(tile_rowop<D>(kt, j, ks, h), qB[ks], sacc);                              \
-            pacc = mfma32(tile_rowop<D>(vt, j, ks, h), doB[ks], pacc);                             \
+            sacc = mfma32(lo.rowop(kt, ks), qB[ks], sacc);                              \
+            pacc = mfma32(lo.rowop(vt, ks), doB[ks], pacc);                             \
         }                                                                                          \
         sched_reads_ahead<2 * KS, 4, 1>();                                                         \
         float ds[16];                                                                              \
@@ -342,9 +394,8 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
         }                                                                                          \
         const bf16x8 dB0 = pack8(ds), dB1 = pack8(ds + 8);                                         \
         _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
-            const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;                                       \
-            mfma32_acc(acc[dt], tile_trop<D>(kt, 4 * h, m0, lane), dB0);                           \
-            mfma32_acc(acc[dt], tile_trop<D>(kt, 16 + 4 * h, m0, lane), dB1);                      \
+            mfma32_acc(acc[dt], lo.trop(kt, 0, dt), dB0);                           \
+            mfma32_acc(acc[dt], lo.trop(kt, 1, dt), dB1);                      \
         }                                                                                          \
         sched_reads_ahead<2 * DT, 3, 2>();                                                         \
     }
@@ -389,6 +440,8 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
     __shared__ uint32_t mask_s[NBUF][4][32];                                      // [buffer][wave][query in block]
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
+    LaneOffsets<D> lo;
+    lo.init(lane);
     const int G = Hq / Hkv;
     const int kvh = blockIdx.x % Hkv;
     int s0, L, blk;
@@ -469,8 +522,8 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
         const unsigned char *qt = lds[BUF][0], *dot = lds[BUF][1];                                 \
         f32x16 sacc = zero16(), pacc = zero16();                                                   \
         _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
-            sacc = mfma32(tile_rowop<D>(qt, j, ks, h), kB[ks], sacc);                              \
-            pacc = mfma32(tile_rowop<D>(dot, j, ks, h), vB[ks], pacc);                             \
+            sacc = mfma32(lo.rowop(qt, ks), kB[ks], sacc);                              \
+            pacc = mfma32(lo.rowop(dot, ks), vB[ks], pacc);                             \
         }                                                                                          \
         float pv[16], dsv[16];                                                                     \
         const bool diag = causal && qcb < kc + 32;      /* wave-uniform: block touches the diagonal */ \
@@ -493,11 +546,10 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
         }                                                                                          \
         const bf16x8 pB0 = pack8(pv), pB1 = pack8(pv + 8), dB0 = pack8(dsv), dB1 = pack8(dsv + 8); \
         _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
-            const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;                                       \
-            mfma32_acc(dvacc[dt], tile_trop<D>(dot, 4 * h, m0, lane), pB0);                        \
-            mfma32_acc(dvacc[dt], tile_trop<D>(dot, 16 + 4 * h, m0, lane), pB1);                   \
-            mfma32_acc(dkacc[dt], tile_trop<D>(qt, 4 * h, m0, lane), dB0);                         \
-            mfma32_acc(dkacc[dt], tile_trop<D>(qt, 16 + 4 * h, m0, lane), dB1);                    \
+            mfma32_acc(dvacc[dt], lo.trop(dot, 0, dt), pB0);                        \
+            mfma32_acc(dvacc[dt], lo.trop(dot, 1, dt), pB1);                   \
+            mfma32_acc(dkacc[dt], lo.trop(qt, 0, dt), dB0);                         \
+            mfma32_acc(dkacc[dt], lo.trop(qt, 1, dt), dB1);                    \
         }                                                                                          \
     }
     TILE_PIPELINE(nblocks, DKV_LOAD, DKV_STORE, DKV_COMPUTE)
@@ -517,159 +569,6 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
                                    pack2bf(dvacc[dt][4 * g4 + 2], dvacc[dt][4 * g4 + 3])};
                 *reinterpret_cast<u32x2 *>(pk + dt * 32 + 8 * g4) = wk;
                 *reinterpret_cast<u32x2 *>(pv_ + dt * 32 + 8 * g4) = wvv;
-            }
-    }
-}
-
-// ==================================================================================================
-// dK, dV for head_dim <= 128: the same key-stationary walk with 8 waves per workgroup.  Waves 0-3
-// accumulate dV^T for the four 32-key groups of the tile, waves 4-7 accumulate dK^T for the same
-// groups, so one wave holds a single D x 32 fp32 accumulator, everything fits the 256 registers that
-// two waves per SIMD allow, and the softmax arithmetic of one wave overlaps the MFMAs of the other.
-// (S is computed by both roles: 40 MFMAs per 32x32 block pair instead of 32.)
-// ==================================================================================================
-template <int D, bool HAS_IDX, int GSHIFT>
-__global__ __launch_bounds__(512, 1) void dsa_tile_dkv8_kernel(
-    const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
-    const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
-    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
-    float scale, int causal, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
-    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2;
-    constexpr int NCHUNK = 32 * CPR;                     // 16-byte chunks per staged operand (<= 512 threads)
-    constexpr int NBUF = 2;
-    constexpr int Gp = 1 << GSHIFT, QB = 32 >> GSHIFT;
-    static_assert(NCHUNK <= 512, "one chunk per thread");
-    __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];   // [buffer][q|dO]
-    __shared__ __attribute__((aligned(16))) float lse_s[NBUF][32], dlt_s[NBUF][32];
-    __shared__ uint32_t mask_s[NBUF][4][32];                                      // [buffer][key group][query in block]
-
-    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
-    const int kg = wv & 3, role = wv >> 2;               // role 0: dV, role 1: dK
-    const int G = Hq / Hkv;
-    const int kvh = blockIdx.x % Hkv;
-    int s0, L, blk;
-    if (!locate_block(cu, N, blockIdx.x / Hkv, 128, false, s0, L, blk)) return;
-    const int c0 = blk * 128, kc = c0 + kg * 32;
-    const int mykey = kc + j;
-    const bool key_ok = mykey < L;
-    const int64_t krow = (int64_t)(s0 + min(mykey, L - 1)) * Hkv + kvh;
-    bf16x8 kB[KS], vB[KS];
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        kB[ks] = load_bf16x8(k + krow * D + 16 * ks + 8 * h);
-        vB[ks] = load_bf16x8(v + krow * D + 16 * ks + 8 * h);
-    }
-    f32x16 acc[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
-    const float scale_log2 = scale * LOG2E_F;
-    const int q0 = causal ? c0 : 0;                      // first query column that can see this key tile
-    const int nblocks = (L - q0 + QB - 1) / QB;          // queries q0 .. L-1
-    const bool stager = tid < NCHUNK;
-    const int srow = (tid % NCHUNK) / CPR, sch = tid % CPR;   // non-staging threads re-read a staged chunk and drop it
-
-    u32x4 qst[2], dost[2];
-    // Per-block side data, one 32-bit word per staging thread, loaded raw and interpreted at STORE time:
-    //   tid 0..31: lse of row tid;  32..63: delta of row tid-32;  64..64+4*QB-1: selection word of
-    //   (key group w, query qi);  the rest re-read a valid word and drop it.
-    const uint32_t *aux_base;
-    int aux_q = 0, aux_stride = 1;                       // word index = aux_stride * min(block start + aux_q, L-1)
-    bool aux_mask_ok = false;
-    if (tid < 64) {
-        const int row = tid & 31;
-        const int hd = min(row & (Gp - 1), G - 1);
-        aux_q = row >> GSHIFT;
-        aux_base = reinterpret_cast<const uint32_t *>((tid < 32 ? lse : delta) + (int64_t)(kvh * G + hd) * T + s0);
-    } else if (HAS_IDX && tid < 64 + 4 * QB) {
-        const int w = (tid - 64) / QB;
-        aux_q = (tid - 64) % QB;
-        aux_stride = ldw;
-        aux_mask_ok = (c0 >> 5) + w < ldw;
-        aux_base = bitmap + (int64_t)s0 * ldw + (aux_mask_ok ? (c0 >> 5) + w : 0);
-    } else {
-        aux_base = reinterpret_cast<const uint32_t *>(lse);
-    }
-    uint32_t aux_st[2] = {0u, 0u};
-#define DKV8_LOAD(SET, BLK)                                                                         \
-    {                                                                                              \
-        const int qcb = q0 + (BLK) * QB;                                                           \
-        const int qc = min(qcb + (srow >> GSHIFT), L - 1);                                         \
-        const int hd = min(srow & (Gp - 1), G - 1);                                                \
-        const int64_t off = ((int64_t)(s0 + qc) * Hq + kvh * G + hd) * D + sch * 8;                \
-        qst[SET] = *reinterpret_cast<const u32x4 *>(q + off);                                      \
-        dost[SET] = *reinterpret_cast<const u32x4 *>(dout + off);                                  \
-        aux_st[SET] = aux_base[(int64_t)aux_stride * min(qcb + aux_q, L - 1)];                     \
-    }
-#define DKV8_STORE(SET, BUF, BLK)                                                                   \
-    {                                                                                              \
-        const int qcb = q0 + (BLK) * QB;                                                           \
-        if (stager) {                                                                              \
-            /* rows past the segment and padded heads are zeroed: they add nothing to dK, dV */     \
-            const bool live = qcb + (srow >> GSHIFT) < L && (srow & (Gp - 1)) < G;                 \
-            const u32x4 z4 = {0u, 0u, 0u, 0u};                                                     \
-            *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(srow, sch)]) = live ? qst[SET] : z4;  \
-            *reinterpret_cast<u32x4 *>(&lds[BUF][1][tile_off<D>(srow, sch)]) = live ? dost[SET] : z4; \
-        }                                                                                          \
-        if (tid < 32) lse_s[BUF][tid] = __uint_as_float(aux_st[SET]) * LOG2E_F;                    \
-        else if (tid < 64) dlt_s[BUF][tid - 32] = __uint_as_float(aux_st[SET]);                    \
-        else if (HAS_IDX && tid < 64 + 4 * QB)                                                     \
-            mask_s[BUF][(tid - 64) / QB][(tid - 64) % QB] = (aux_mask_ok && qcb + aux_q < L) ? aux_st[SET] : 0u; \
-    }
-#define DKV8_COMPUTE(BLK, BUF)                                                                      \
-    {                                                                                              \
-        const int qcb = q0 + (BLK) * QB;                                                           \
-        const unsigned char *qt = lds[BUF][0], *dot = lds[BUF][1];                                 \
-        const unsigned char *t2 = role ? qt : dot;      /* operand of the second GEMM */            \
-        f32x16 sacc = zero16(), pacc = zero16();                                                   \
-        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                          \
-            sacc = mfma32(tile_rowop<D>(qt, j, ks, h), kB[ks], sacc);                              \
-        sched_reads_ahead<KS, 4, 1>();                                                             \
-        if (role) {                                     /* wave-uniform */                          \
-            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                      \
-                pacc = mfma32(tile_rowop<D>(dot, j, ks, h), vB[ks], pacc);                         \
-            sched_reads_ahead<KS, 4, 1>();                                                         \
-        }                                                                                          \
-        float bv[16];                                                                              \
-        const bool diag = causal && qcb < kc + 32;      /* wave-uniform: block touches the diagonal */ \
-        _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {                                         \
-            const f32x4 l4 = *reinterpret_cast<const f32x4 *>(&lse_s[BUF][8 * g4 + 4 * h]);        \
-            const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&dlt_s[BUF][8 * g4 + 4 * h]);        \
-            uint32_t keep = 0u;                                                                    \
-            _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                        \
-                const int vi = 4 * g4 + e, row = 8 * g4 + 4 * h + e;                               \
-                if (e == 0 || GSHIFT < 2) {              /* rows of one query share the mask bit */  \
-                    const int qi = row >> GSHIFT;                                                  \
-                    uint32_t mw = HAS_IDX ? mask_s[BUF][kg][qi] : 0xffffffffu;                     \
-                    if (diag) mw &= causal_bits(qcb + qi - kc);                                    \
-                    keep = bit_mask(mw, j);                                                        \
-                }                                                                                  \
-                const float p = fast_exp2(keep_or_neginf(fmaf(sacc[vi], scale_log2, -l4[e]), keep)); \
-                bv[vi] = role ? p * (pacc[vi] - d4[e]) : p;                                        \
-            }                                                                                      \
-        }                                                                                          \
-        const bf16x8 b0 = pack8(bv), b1 = pack8(bv + 8);                                           \
-        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
-            const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;                                       \
-            acc[dt] = mfma32(tile_trop<D>(t2, 4 * h, m0, lane), b0, acc[dt]);                      \
-            acc[dt] = mfma32(tile_trop<D>(t2, 16 + 4 * h, m0, lane), b1, acc[dt]);                 \
-        }                                                                                          \
-        sched_reads_ahead<2 * DT, 3, 2>();                                                         \
-    }
-    TILE_PIPELINE(nblocks, DKV8_LOAD, DKV8_STORE, DKV8_COMPUTE)
-#undef DKV8_LOAD
-#undef DKV8_STORE
-#undef DKV8_COMPUTE
-
-    if (key_ok) {
-        bf16_t *po = (role ? dk : dv) + krow * D + 4 * h;
-        const float osc = role ? scale : 1.f;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                const u32x2 w2 = {pack2bf(acc[dt][4 * g4] * osc, acc[dt][4 * g4 + 1] * osc),
-                                  pack2bf(acc[dt][4 * g4 + 2] * osc, acc[dt][4 * g4 + 3] * osc)};
-                *reinterpret_cast<u32x2 *>(po + dt * 32 + 8 * g4) = w2;
             }
     }
 }
@@ -705,6 +604,8 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     unsigned char *const aux_ring = pd_ring + 2 * PD_SLOT;           // 3 slots
 
     const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5, j = lane & 31;
+    LaneOffsets<D> lo;
+    lo.init(lane);
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);         // wave-uniform for the compiler too
     const int kg = wv & 3;
     const bool consumer = wv >= 4;
@@ -795,8 +696,8 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
                 f32x16 sacc = zero16(), pacc = zero16();
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    sacc = mfma32(tile_rowop<D>(qt, j, ks, h), kB[ks], sacc);
-                    pacc = mfma32(tile_rowop<D>(dot, j, ks, h), vB[ks], pacc);
+                    sacc = mfma32(lo.rowop(qt, ks), kB[ks], sacc);
+                    pacc = mfma32(lo.rowop(dot, ks), vB[ks], pacc);
                 }
                 sched_reads_ahead<2 * KS, 4, 1>();
                 float pv[16], dsv[16];
@@ -837,17 +738,23 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
             lstore(b + 1);
             gload(min(b + 2, nblocks - 1));
             if (b >= 1) {
-                const unsigned char *qt = qd_ring + ((b - 1) % 3) * QD_SLOT, *dot = qt + TILE_B;
+                const unsigned char *qt = qd_ring + ((b - 1) % 3) * QD_SLOT;
+                lds_u8 *pe[4], *po[4];      // lane addresses in the q block; the dO block sits TILE_B behind
+#pragma unroll
+                for (int vv = 0; vv < 4; ++vv) {
+                    pe[vv] = (lds_u8 *)qt + lo.tr_e[vv];
+                    po[vv] = (lds_u8 *)qt + lo.tr_o[vv];
+                    asm volatile("" : "+v"(pe[vv]), "+v"(po[vv]));   // keep "address + immediate" reads: no re-association
+                }
                 const unsigned char *pd = pd_ring + ((b - 1) & 1) * PD_SLOT + kg * 4096 + lane * 16;
                 const bf16x8 pB0 = *reinterpret_cast<const bf16x8 *>(pd), pB1 = *reinterpret_cast<const bf16x8 *>(pd + 1024);
                 const bf16x8 dB0 = *reinterpret_cast<const bf16x8 *>(pd + 2048), dB1 = *reinterpret_cast<const bf16x8 *>(pd + 3072);
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const int m0 = dt * 32 + ((lane >> 4) & 1) * 16;
-                    dvacc[dt] = mfma32(tile_trop<D>(dot, 4 * h, m0, lane), pB0, dvacc[dt]);
-                    dvacc[dt] = mfma32(tile_trop<D>(dot, 16 + 4 * h, m0, lane), pB1, dvacc[dt]);
-                    dkacc[dt] = mfma32(tile_trop<D>(qt, 4 * h, m0, lane), dB0, dkacc[dt]);
-                    dkacc[dt] = mfma32(tile_trop<D>(qt, 16 + 4 * h, m0, lane), dB1, dkacc[dt]);
+                    dvacc[dt] = mfma32(LaneOffsets<D>::trop_at(pe, po, 0, dt, TILE_B), pB0, dvacc[dt]);
+                    dvacc[dt] = mfma32(LaneOffsets<D>::trop_at(pe, po, 1, dt, TILE_B), pB1, dvacc[dt]);
+                    dkacc[dt] = mfma32(LaneOffsets<D>::trop_at(pe, po, 0, dt, 0), dB0, dkacc[dt]);
+                    dkacc[dt] = mfma32(LaneOffsets<D>::trop_at(pe, po, 1, dt, 0), dB1, dkacc[dt]);
                 }
                 sched_reads_ahead<4 * DT, 3, 2>();
             }
