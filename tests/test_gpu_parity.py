@@ -151,7 +151,7 @@ def test_scaled_configs(name, segs, K):
     ("C1", (300, 200), 16),
 ])
 def test_tile_and_gather_paths_agree_with_the_oracle(crossover, name, segs, K):
-    """crossover 0 = gather kernels only, 1<<20 = tile kernels only, 2 = rows split at pos 2K (rounded to 128)."""
+    """crossover 0 = gather kernels only, 1<<20 = tile kernels only, 2 = rows split at pos 2K (rounded to 256)."""
     _log(f"paths {name}")
     w = W.scaled(W.WORKLOADS[name], segs, top_k=K, name=name + "-paths")
     outs = {}
@@ -159,7 +159,7 @@ def test_tile_and_gather_paths_agree_with_the_oracle(crossover, name, segs, K):
         crossover(c)
         outs[c] = _run_case(w).detach().float()
     assert (outs[0] - outs[1 << 20]).abs().max().item() < 2e-2
-    split = (2 * K + 127) // 128 * 128            # mixed run: tile rows before the split, gather rows after
+    split = (2 * K + 255) // 256 * 256            # mixed run: tile rows before the split, gather rows after
     a = 0
     for L in segs:
         assert torch.equal(outs[2][a:a + min(L, split)], outs[1 << 20][a:a + min(L, split)])

@@ -150,7 +150,7 @@ static int pos_split_for(const int32_t *idx, int K) {
     if (!idx) return INT32_MAX;                       // dense causal: tiles everywhere
     const int64_t p = (int64_t)K * g_tile_crossover;
     if (p >= INT32_MAX - 256) return INT32_MAX;
-    return (int)((p + 127) / 128 * 128);
+    return (int)((p + 255) / 256 * 256);          // a multiple of every tile kernel's query block
 }
 
 extern "C" size_t dsa_attn_fwd_workspace_bytes(int T, int max_seqlen, int has_idx) {

@@ -13,36 +13,23 @@
 //   The second GEMM of each chain takes its B operand straight from the C layout of the first
 //   (the contraction order over the 32 keys/rows of a tile is permuted identically on both operands).
 #include "dsa_common.h"
+#include <type_traits>
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }   // v_exp_f32; exp2(-inf) = 0
 
-// ---- swizzled LDS tile: rows of D bf16 (D*2 bytes, no padding); chunk = 16 bytes -----------------
-__device__ __forceinline__ int tile_sw(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
+// ---- LDS tile: 32 rows of D bf16 with a pitch of D*2 + 64 bytes; chunk = 16 bytes ------------------
+// The LDS of gfx950 has 64 four-byte banks (256 B per clock).  A 16-byte read is served 16 lanes at a
+// time and a transposed 8-byte read 32 lanes at a time, so a row-wise operand read (16 consecutive rows,
+// same chunk) and a transposed read (4 consecutive rows x 64 B) must each cover all banks once.  The
+// 64-byte skew per row separates 4 consecutive rows, the XOR of the chunk's two low bits with row bits
+// 2-3 separates rows 4 apart: both read patterns and the row-wise staging writes are conflict-free.
+template <int D> constexpr int tile_pitch() { return D * 2 + 64; }
+template <int D> constexpr int tile_bytes() { return 32 * tile_pitch<D>(); }
+__device__ __forceinline__ int tile_sw(int row) { return (row >> 2) & 3; }
 template <int D>
-__device__ __forceinline__ int tile_off(int row, int chunk) { return row * (D * 2) + ((chunk ^ tile_sw(row)) << 4); }
+__device__ __forceinline__ int tile_off(int row, int chunk) { return row * tile_pitch<D>() + ((chunk ^ tile_sw(row)) << 4); }
 
-// A operand of mfma32 read row-wise: lane (i = row, h) takes elements [16*ks + 8h, +8) of row i
-template <int D>
-__device__ __forceinline__ bf16x8 tile_rowop(const unsigned char *tile, int row, int ks, int h) {
-    return *reinterpret_cast<const bf16x8 *>(tile + tile_off<D>(row, 2 * ks + h));
-}
-// A operand of mfma32 read transposed: lane l takes column c = m0 + (l & 15) and the 8 rows
-// {R0..R0+3, R0+8..R0+11}.  ds_read_b64_tr_b16: within 16 lanes, lane s supplies the address of 4
-// consecutive elements of row R0 + s/4 at column m0 + 4*(s%4); lane s receives rows R0..R0+3 of column m0+s.
-template <int D>
-__device__ __forceinline__ bf16x8 tile_trop(const unsigned char *tile, int R0, int m0, int lane) {
-    const int s = lane & 15;
-    const int row = R0 + (s >> 2), col = m0 + ((s & 3) << 2);
-    const int sub = ((col >> 2) & 1) << 3;
-    const unsigned char *p0 = tile + tile_off<D>(row, col >> 3) + sub;
-    const unsigned char *p1 = tile + tile_off<D>(row + 8, col >> 3) + sub;
-    const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p0);
-    const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p1);
-    typedef short s16x8 __attribute__((ext_vector_type(8)));
-    const s16x8 r = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
-    return __builtin_bit_cast(bf16x8, r);
-}
 // accumulate in place (kept as a function so that the accumulation sites read alike)
 __device__ __forceinline__ void mfma32_acc(f32x16 &c, bf16x8 a, bf16x8 b) { c = mfma32(a, b, c); }
 // all-ones if bit `b` of `word` is set, else 0 (v_bfe_i32 when b is a compile-time constant)
@@ -58,9 +45,9 @@ __device__ __forceinline__ uint32_t causal_bits(int d) { return d >= 31 ? 0xffff
 // Issue order for a chain of NM MFMAs that each consume RPM LDS reads: keep AHEAD MFMAs' worth of reads
 // in flight (the machine scheduler otherwise sinks every read next to its use and the chain runs at
 // LDS latency).  Applies to the instructions of the enclosing basic block, in program order.
-template <int NM, int AHEAD, int RPM>
+template <int NM, int AHEAD, int RPM, int FIRST = 0>
 __device__ __forceinline__ void sched_reads_ahead() {
-    __builtin_amdgcn_sched_group_barrier(0x100, AHEAD * RPM, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, FIRST + AHEAD * RPM, 0);   // FIRST: other reads issued up front
 #pragma unroll
     for (int i = 0; i < NM - AHEAD; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -69,36 +56,34 @@ __device__ __forceinline__ void sched_reads_ahead() {
     __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
 }
 // Per-lane LDS byte offsets of the two read patterns, computed once per kernel so that every operand
-// read in the loops is "tile base + lane offset + immediate" (the swizzle only XORs chunk bits 0-2, so
-// k-step / d-tile indices move the address by a lane constant plus a compile-time multiple of 128 B).
+// read in the loops is "tile base + lane offset + immediate" (the swizzle only XORs chunk bits 0-1, so
+// k-step / d-tile indices move the address by a lane constant plus a compile-time multiple of 64 B).
+//   row-wise A operand of mfma32: lane (i = row j, h) takes elements [16*ks + 8h, +8) of row j
+//   transposed A operand: lane l takes column c = 32*dt + (l & 31)... of the 8 rows {R..R+3, R+8..R+11}.
+//   ds_read_b64_tr_b16: within 16 lanes, lane s supplies the address of 4 consecutive elements of row
+//   R + s/4 at column m0 + 4*(s%4); lane s receives rows R..R+3 of column m0 + s.
 typedef __attribute__((address_space(3))) unsigned char lds_u8;
 template <int D>
 struct LaneOffsets {
-    int row[4];      // row-wise operand of row j: k-steps ks with ks % 4 == c
-    int tr_e[4];     // transposed operand, even d-tiles: rows 4h + s/4 + {0, 8, 16, 24}
-    int tr_o[4];     // same for odd d-tiles
+    int row[2];      // row-wise operand of row j: k-steps ks with ks % 2 == c
+    int tr[4];       // transposed operand: rows 4h + s/4 + {0, 8, 16, 24}
     __device__ __forceinline__ void init(int lane) {
         const int h = lane >> 5, j = lane & 31, s = lane & 15;
         const int swj = tile_sw(j);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) row[c] = j * (D * 2) + ((((c ^ (swj >> 1)) << 1) | (h ^ (swj & 1))) << 4);
+        for (int c = 0; c < 2; ++c) row[c] = j * tile_pitch<D>() + ((((c ^ (swj >> 1)) << 1) | (h ^ (swj & 1))) << 4);
         const int low = ((lane >> 4) & 1) * 2 + ((s & 3) >> 1), sub = (s & 1) << 3;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-            const int r = 4 * h + (s >> 2) + 8 * v, sw = tile_sw(r);
-            const int lo = low ^ (sw & 3), f = sw & 4;
-            tr_e[v] = r * (D * 2) + ((lo | f) << 4) + sub;
-            tr_o[v] = r * (D * 2) + ((lo | (4 ^ f)) << 4) + sub;
+            const int r = 4 * h + (s >> 2) + 8 * v;
+            tr[v] = r * tile_pitch<D>() + ((low ^ tile_sw(r)) << 4) + sub;
         }
     }
     // row-wise A operand of k-step ks (elements [16ks + 8h, +8) of row j)
     __device__ __forceinline__ bf16x8 rowop(const unsigned char *tile, int ks) const {
-        return *reinterpret_cast<const bf16x8 *>(tile + row[ks & 3] + (ks >> 2) * 128);
+        return *reinterpret_cast<const bf16x8 *>(tile + row[ks & 1] + (ks >> 1) * 64);
     }
-    // same with the lane addresses already formed (pe/po = tile + tr_e/tr_o): one immediate per read
-    __device__ __forceinline__ static bf16x8 trop_at(lds_u8 *const *pe, lds_u8 *const *po, int pair, int dt, int imm) {
-        lds_u8 *const *t = (dt & 1) ? po : pe;
-        lds_u8 *p0 = t[2 * pair] + (dt >> 1) * 128 + imm, *p1 = t[2 * pair + 1] + (dt >> 1) * 128 + imm;
+    __device__ __forceinline__ static bf16x8 tr_pair(lds_u8 *p0, lds_u8 *p1) {
         const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p0);
         const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p1);
         typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -107,14 +92,11 @@ struct LaneOffsets {
     }
     // transposed A operand of d-tile dt over rows {R..R+3, R+8..R+11}, R = 4h (pair 0) or 16 + 4h (pair 1)
     __device__ __forceinline__ bf16x8 trop(const unsigned char *tile, int pair, int dt) const {
-        const int *t = (dt & 1) ? tr_o : tr_e;
-        const unsigned char *p0 = tile + t[2 * pair] + (dt >> 1) * 128;
-        const unsigned char *p1 = tile + t[2 * pair + 1] + (dt >> 1) * 128;
-        const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p0);
-        const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p1);
-        typedef short s16x8 __attribute__((ext_vector_type(8)));
-        const s16x8 r = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
-        return __builtin_bit_cast(bf16x8, r);
+        return tr_pair((lds_u8 *)tile + tr[2 * pair] + dt * 64, (lds_u8 *)tile + tr[2 * pair + 1] + dt * 64);
+    }
+    // same with the lane addresses already formed (p[v] = tile + tr[v]): one immediate per read
+    __device__ __forceinline__ static bf16x8 trop_at(lds_u8 *const *p, int pair, int dt, int imm) {
+        return tr_pair(p[2 * pair] + dt * 64 + imm, p[2 * pair + 1] + dt * 64 + imm);
     }
 };
 __device__ __forceinline__ bf16x8 pack8(const float *x) {
@@ -190,7 +172,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
     const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
     float scale_log2, int pos_split, int causal, bf16_t *__restrict__ out, float *__restrict__ lse) {
-    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2, LOADS = 32 * CPR / 256;
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / 256;
     constexpr int NBUF = (D > 128) ? 1 : 2;           // double buffering where 64 KiB of static LDS allow it
     constexpr int Gp = 1 << GSHIFT, QBW = 128 >> GSHIFT;
     static_assert(LOADS >= 1, "tile must give every thread a chunk");
@@ -318,7 +300,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
     float scale, int pos_split, int causal, bf16_t *__restrict__ dq) {
-    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2, LOADS = 32 * CPR / 256;
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / 256;
     constexpr int NBUF = (D > 128) ? 1 : 2;
     constexpr int Gp = 1 << GSHIFT, QBW = 128 >> GSHIFT;
     __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];
@@ -432,7 +414,7 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
     float scale, int causal, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
-    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2, LOADS = 32 * CPR / 256;
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / 256;
     constexpr int NBUF = (D > 128) ? 1 : 2;
     constexpr int Gp = 1 << GSHIFT, QB = 32 >> GSHIFT;                           // queries per block
     __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];   // [buffer][q|dO]
@@ -577,13 +559,17 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
 // dK, dV for head_dim <= 128, producer/consumer form.  A workgroup owns a 128-key tile (4 groups of 32
 // keys) of one segment and kv head and walks the later queries in blocks of 32 (query, head) rows.
 //   waves 0-3 (producers, one per key group): S = Q K^T and dP = dO V^T against the group's K / V rows
-//     held in registers, then P and dS = P * (dP - delta) in bf16, written to LDS in MFMA B layout;
-//   waves 4-7 (consumers, one per key group): dV^T += dO^T P and dK^T += Q^T dS for the previous block,
-//     A operands read transposed from the staged q / dO block, B operands read back from LDS.
-// Producer w and consumer w+4 share a SIMD: the softmax arithmetic of one overlaps the MFMAs of the
-// other, nothing is computed twice (32 MFMAs per 32x32 block pair), each wave stays under 256 registers.
-// LDS (dynamic, ~85 KiB): q/dO blocks in a ring of three (block b+1 being staged, b read row-wise by
-// the producers, b-1 read transposed by the consumers), P/dS in a ring of two.  One barrier per block.
+//     held in registers, then P and dS = P * (dP - delta) in bf16, written to LDS in MFMA B layout.
+//     The two GEMMs of block b+1 are issued between the softmax arithmetic of block b: a SIMD overlaps
+//     matrix and vector instructions of one instruction stream far better than those of two waves.
+//   waves 4-7 (consumers, one per key group): dV^T += dO^T P and dK^T += Q^T dS for block b-1,
+//     A operands read transposed from the staged q / dO block, B operands read back from LDS.  They
+//     also do all the staging (global -> registers one block ahead -> LDS), so the producers' stream
+//     holds nothing but the GEMMs and the softmax.
+// Nothing is computed twice (32 MFMAs per 32x32 block pair), each wave stays under 256 registers.
+// LDS (dynamic, ~115 KiB): q/dO blocks in a ring of four (b+2 being staged, b+1 read row-wise by the
+// producers, b-1 read transposed by the consumers), P/dS in a ring of two, row statistics and
+// selection words in a ring of four.  One barrier per block.
 // ==================================================================================================
 template <int D, bool HAS_IDX, int GSHIFT>
 __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
@@ -591,17 +577,18 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
     float scale, int causal, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
-    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = 32 * D * 2;
-    constexpr int NCHUNK = 32 * CPR;                     // 16-byte chunks per staged operand (<= 512)
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>();
+    constexpr int NCHUNK = 32 * CPR;                     // 16-byte chunks per staged operand
+    constexpr int CPT = NCHUNK / 256;                    // chunks per consumer thread and operand
     constexpr int Gp = 1 << GSHIFT, QB = 32 >> GSHIFT;
     constexpr int QD_SLOT = 2 * TILE_B;                  // q block | dO block
     constexpr int PD_SLOT = 4 * 4 * 1024;                // 4 key groups x {P lo, P hi, dS lo, dS hi} x 64 lanes x 16 B
     constexpr int AUX_SLOT = (32 + 32 + 4 * 32) * 4;     // lse | delta | selection words [key group][query]
-    static_assert(NCHUNK <= 512, "one chunk per thread");
+    static_assert(CPT >= 1 && NCHUNK % 256 == 0, "every consumer thread stages whole chunks");
     extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
-    unsigned char *const qd_ring = dyn_lds;                          // 3 slots
-    unsigned char *const pd_ring = dyn_lds + 3 * QD_SLOT;            // 2 slots
-    unsigned char *const aux_ring = pd_ring + 2 * PD_SLOT;           // 3 slots
+    unsigned char *const qd_ring = dyn_lds;                          // 4 slots
+    unsigned char *const pd_ring = dyn_lds + 4 * QD_SLOT;            // 2 slots
+    unsigned char *const aux_ring = pd_ring + 2 * PD_SLOT;           // 4 slots
 
     const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5, j = lane & 31;
     LaneOffsets<D> lo;
@@ -621,142 +608,94 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     const int q0 = causal ? c0 : 0;                      // first query column that can see this key tile
     const int nblocks = (L - q0 + QB - 1) / QB;          // queries q0 .. L-1
 
-    // ---- staging (all 512 threads): one 16-byte chunk of q and of dO per block, one side word ----------
-    const bool stager = tid < NCHUNK;
-    const int srow = (tid % NCHUNK) / CPR, sch = tid % CPR;
-    const uint32_t *aux_base;
-    int aux_q = 0, aux_stride = 1;
-    bool aux_mask_ok = false;
-    if (tid < 64) {                                      // 0..31: lse of row tid, 32..63: delta of row tid-32
-        const int row = tid & 31;
-        const int hd = min(row & (Gp - 1), G - 1);
-        aux_q = row >> GSHIFT;
-        aux_base = reinterpret_cast<const uint32_t *>((tid < 32 ? lse : delta) + (int64_t)(kvh * G + hd) * T + s0);
-    } else if (HAS_IDX && tid < 64 + 4 * QB) {           // selection word of (key group w, query qi)
-        const int w = (tid - 64) / QB;
-        aux_q = (tid - 64) % QB;
-        aux_stride = ldw;
-        aux_mask_ok = (c0 >> 5) + w < ldw;
-        aux_base = bitmap + (int64_t)s0 * ldw + (aux_mask_ok ? (c0 >> 5) + w : 0);
-    } else {
-        aux_base = reinterpret_cast<const uint32_t *>(lse);
-    }
-    u32x4 qst, dost;
-    uint32_t aux_st;
-    auto gload = [&](int b) {                            // block index clamped by the caller
-        const int qcb = q0 + b * QB;
-        const int qc = min(qcb + (srow >> GSHIFT), L - 1);
-        const int hd = min(srow & (Gp - 1), G - 1);
-        const int64_t off = ((int64_t)(s0 + qc) * Hq + kvh * G + hd) * D + sch * 8;
-        qst = *reinterpret_cast<const u32x4 *>(q + off);
-        dost = *reinterpret_cast<const u32x4 *>(dout + off);
-        aux_st = aux_base[(int64_t)aux_stride * min(qcb + aux_q, L - 1)];
-    };
-    auto lstore = [&](int b) {                           // registers -> ring slot b % 3
-        const int qcb = q0 + b * QB;
-        unsigned char *slot = qd_ring + (b % 3) * QD_SLOT;
-        float *lse_s = reinterpret_cast<float *>(aux_ring + (b % 3) * AUX_SLOT);
-        float *dlt_s = lse_s + 32;
-        uint32_t *mask_s = reinterpret_cast<uint32_t *>(dlt_s + 32);
-        if (stager) {
-            // rows past the segment and padded heads are zeroed: they add nothing to dK, dV
-            const bool live = qcb + (srow >> GSHIFT) < L && (srow & (Gp - 1)) < G;
-            const u32x4 z4 = {0u, 0u, 0u, 0u};
-            *reinterpret_cast<u32x4 *>(slot + tile_off<D>(srow, sch)) = live ? qst : z4;
-            *reinterpret_cast<u32x4 *>(slot + TILE_B + tile_off<D>(srow, sch)) = live ? dost : z4;
+    if (consumer) {
+        // ================= consumers: stage block b+2, then dV^T, dK^T of block b-1 =================
+        const int ctid = tid - 256;
+        const uint32_t *aux_base;
+        int aux_q = 0, aux_stride = 1;
+        bool aux_mask_ok = false;
+        if (ctid < 64) {                                 // 0..31: lse of row ctid, 32..63: delta of row ctid-32
+            const int row = ctid & 31;
+            const int hd = min(row & (Gp - 1), G - 1);
+            aux_q = row >> GSHIFT;
+            aux_base = reinterpret_cast<const uint32_t *>((ctid < 32 ? lse : delta) + (int64_t)(kvh * G + hd) * T + s0);
+        } else if (HAS_IDX && ctid < 64 + 4 * QB) {      // selection word of (key group w, query qi)
+            const int w = (ctid - 64) / QB;
+            aux_q = (ctid - 64) % QB;
+            aux_stride = ldw;
+            aux_mask_ok = (c0 >> 5) + w < ldw;
+            aux_base = bitmap + (int64_t)s0 * ldw + (aux_mask_ok ? (c0 >> 5) + w : 0);
+        } else {
+            aux_base = reinterpret_cast<const uint32_t *>(lse);
         }
-        if (tid < 32) lse_s[tid] = __uint_as_float(aux_st) * LOG2E_F;
-        else if (tid < 64) dlt_s[tid - 32] = __uint_as_float(aux_st);
-        else if (HAS_IDX && tid < 64 + 4 * QB)
-            mask_s[((tid - 64) / QB) * 32 + (tid - 64) % QB] = (aux_mask_ok && qcb + aux_q < L) ? aux_st : 0u;
-    };
-
-    gload(0);
-    lstore(0);
-    gload(min(1, nblocks - 1));
-    __syncthreads();
-
-    if (!consumer) {
-        // ================= producer: P and dS of block b into the P/dS ring =================
-        bf16x8 kB[KS], vB[KS];
+        u32x4 qst[CPT], dost[CPT];
+        uint32_t aux_st;
+        auto gload = [&](int b) {                        // block index clamped by the caller
+            const int qcb = q0 + b * QB;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            kB[ks] = load_bf16x8(k + krow * D + 16 * ks + 8 * h);
-            vB[ks] = load_bf16x8(v + krow * D + 16 * ks + 8 * h);
-        }
-        for (int b = 0; b <= nblocks; ++b) {
-            lstore(b + 1);                               // registers hold block b+1; slot (b+1)%3 is free since the last barrier
-            gload(min(b + 2, nblocks - 1));
-            if (b < nblocks) {
-                const int qcb = q0 + b * QB;
-                const unsigned char *qt = qd_ring + (b % 3) * QD_SLOT, *dot = qt + TILE_B;
-                const float *lse_s = reinterpret_cast<const float *>(aux_ring + (b % 3) * AUX_SLOT);
-                const float *dlt_s = lse_s + 32;
-                const uint32_t *mask_s = reinterpret_cast<const uint32_t *>(dlt_s + 32) + kg * 32;
-                f32x16 sacc = zero16(), pacc = zero16();
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    sacc = mfma32(lo.rowop(qt, ks), kB[ks], sacc);
-                    pacc = mfma32(lo.rowop(dot, ks), vB[ks], pacc);
-                }
-                sched_reads_ahead<2 * KS, 4, 1>();
-                float pv[16], dsv[16];
-                const bool diag = causal && qcb < kc + 32;   // wave-uniform: block touches the diagonal
-#pragma unroll
-                for (int g4 = 0; g4 < 4; ++g4) {
-                    const f32x4 l4 = *reinterpret_cast<const f32x4 *>(&lse_s[8 * g4 + 4 * h]);
-                    const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&dlt_s[8 * g4 + 4 * h]);
-                    uint32_t keep = 0u;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int vi = 4 * g4 + e, row = 8 * g4 + 4 * h + e;
-                        if (e == 0 || GSHIFT < 2) {          // rows of one query share the mask bit
-                            const int qi = row >> GSHIFT;
-                            uint32_t mw = HAS_IDX ? mask_s[qi] : 0xffffffffu;
-                            if (diag) mw &= causal_bits(qcb + qi - kc);
-                            keep = bit_mask(mw, j);
-                        }
-                        const float p = fast_exp2(keep_or_neginf(fmaf(sacc[vi], scale_log2, -l4[e]), keep));
-                        pv[vi] = p;
-                        dsv[vi] = p * (pacc[vi] - d4[e]);
-                    }
-                }
-                unsigned char *pd = pd_ring + (b & 1) * PD_SLOT + kg * 4096 + lane * 16;
-                *reinterpret_cast<bf16x8 *>(pd) = pack8(pv);
-                *reinterpret_cast<bf16x8 *>(pd + 1024) = pack8(pv + 8);
-                *reinterpret_cast<bf16x8 *>(pd + 2048) = pack8(dsv);
-                *reinterpret_cast<bf16x8 *>(pd + 3072) = pack8(dsv + 8);
+            for (int i = 0; i < CPT; ++i) {
+                const int c = i * 256 + ctid, srow = c / CPR, sch = c % CPR;
+                const int qc = min(qcb + (srow >> GSHIFT), L - 1);
+                const int hd = min(srow & (Gp - 1), G - 1);
+                const int64_t off = ((int64_t)(s0 + qc) * Hq + kvh * G + hd) * D + sch * 8;
+                qst[i] = *reinterpret_cast<const u32x4 *>(q + off);
+                dost[i] = *reinterpret_cast<const u32x4 *>(dout + off);
             }
-            __syncthreads();
-        }
-    } else {
-        // ================= consumer: dV^T, dK^T of block b-1 =================
+            aux_st = aux_base[(int64_t)aux_stride * min(qcb + aux_q, L - 1)];
+        };
+        auto lstore = [&](int b) {                       // registers -> ring slot b % 4
+            const int qcb = q0 + b * QB;
+            unsigned char *slot = qd_ring + (b & 3) * QD_SLOT;
+            float *lse_s = reinterpret_cast<float *>(aux_ring + (b & 3) * AUX_SLOT);
+            float *dlt_s = lse_s + 32;
+            uint32_t *mask_s = reinterpret_cast<uint32_t *>(dlt_s + 32);
+#pragma unroll
+            for (int i = 0; i < CPT; ++i) {
+                const int c = i * 256 + ctid, srow = c / CPR, sch = c % CPR;
+                // rows past the segment and padded heads are zeroed: they add nothing to dK, dV
+                const bool live = qcb + (srow >> GSHIFT) < L && (srow & (Gp - 1)) < G;
+                const u32x4 z4 = {0u, 0u, 0u, 0u};
+                *reinterpret_cast<u32x4 *>(slot + tile_off<D>(srow, sch)) = live ? qst[i] : z4;
+                *reinterpret_cast<u32x4 *>(slot + TILE_B + tile_off<D>(srow, sch)) = live ? dost[i] : z4;
+            }
+            if (ctid < 32) lse_s[ctid] = __uint_as_float(aux_st) * LOG2E_F;
+            else if (ctid < 64) dlt_s[ctid - 32] = __uint_as_float(aux_st);
+            else if (HAS_IDX && ctid < 64 + 4 * QB)
+                mask_s[((ctid - 64) / QB) * 32 + (ctid - 64) % QB] = (aux_mask_ok && qcb + aux_q < L) ? aux_st : 0u;
+        };
+        const int last = nblocks - 1;
+        gload(0);
+        lstore(0);
+        gload(min(1, last));
+        lstore(1);
+        gload(min(2, last));
+        __syncthreads();                                 // blocks 0 and 1 staged
+
         f32x16 dkacc[DT], dvacc[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) { dkacc[dt] = zero16(); dvacc[dt] = zero16(); }
         for (int b = 0; b <= nblocks; ++b) {
-            lstore(b + 1);
-            gload(min(b + 2, nblocks - 1));
+            lstore(b + 2);                               // slot (b+2)%4 was last read (as block b-2) before the previous barrier
+            gload(min(b + 3, last));
             if (b >= 1) {
-                const unsigned char *qt = qd_ring + ((b - 1) % 3) * QD_SLOT;
-                lds_u8 *pe[4], *po[4];      // lane addresses in the q block; the dO block sits TILE_B behind
+                const unsigned char *qt = qd_ring + ((b - 1) & 3) * QD_SLOT;
+                lds_u8 *pt[4];              // lane addresses in the q block; the dO block sits TILE_B behind
 #pragma unroll
                 for (int vv = 0; vv < 4; ++vv) {
-                    pe[vv] = (lds_u8 *)qt + lo.tr_e[vv];
-                    po[vv] = (lds_u8 *)qt + lo.tr_o[vv];
-                    asm volatile("" : "+v"(pe[vv]), "+v"(po[vv]));   // keep "address + immediate" reads: no re-association
+                    pt[vv] = (lds_u8 *)qt + lo.tr[vv];
+                    asm volatile("" : "+v"(pt[vv]));     // keep "address + immediate" reads: no re-association
                 }
                 const unsigned char *pd = pd_ring + ((b - 1) & 1) * PD_SLOT + kg * 4096 + lane * 16;
                 const bf16x8 pB0 = *reinterpret_cast<const bf16x8 *>(pd), pB1 = *reinterpret_cast<const bf16x8 *>(pd + 1024);
                 const bf16x8 dB0 = *reinterpret_cast<const bf16x8 *>(pd + 2048), dB1 = *reinterpret_cast<const bf16x8 *>(pd + 3072);
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    dvacc[dt] = mfma32(LaneOffsets<D>::trop_at(pe, po, 0, dt, TILE_B), pB0, dvacc[dt]);
-                    dvacc[dt] = mfma32(LaneOffsets<D>::trop_at(pe, po, 1, dt, TILE_B), pB1, dvacc[dt]);
-                    dkacc[dt] = mfma32(LaneOffsets<D>::trop_at(pe, po, 0, dt, 0), dB0, dkacc[dt]);
-                    dkacc[dt] = mfma32(LaneOffsets<D>::trop_at(pe, po, 1, dt, 0), dB1, dkacc[dt]);
+                    dvacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 0, dt, TILE_B), pB0, dvacc[dt]);
+                    dkacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 0, dt, 0), dB0, dkacc[dt]);
+                    dvacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 1, dt, TILE_B), pB1, dvacc[dt]);
+                    dkacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 1, dt, 0), dB1, dkacc[dt]);
                 }
-                sched_reads_ahead<4 * DT, 3, 2>();
+                sched_reads_ahead<4 * DT, 3, 2, 4>();
             }
             __syncthreads();
         }
@@ -774,10 +713,132 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
                     *reinterpret_cast<u32x2 *>(pv_ + dt * 32 + 8 * g4) = wvv;
                 }
         }
+        return;
     }
+
+    // ================= producers: S, dP of block b+1 between the softmax of block b =================
+    bf16x8 kB[KS], vB[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        kB[ks] = load_bf16x8(k + krow * D + 16 * ks + 8 * h);
+        vB[ks] = load_bf16x8(v + krow * D + 16 * ks + 8 * h);
+    }
+    // row statistics and selection words of a block are read from LDS one block ahead
+    f32x4 l4[4], d4[4];
+    uint32_t mw[16];
+    auto read_aux = [&](int b) {
+        const float *lse_s = reinterpret_cast<const float *>(aux_ring + (b & 3) * AUX_SLOT);
+        const float *dlt_s = lse_s + 32;
+        const uint32_t *mask_s = reinterpret_cast<const uint32_t *>(dlt_s + 32) + kg * 32;
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            l4[g4] = *reinterpret_cast<const f32x4 *>(&lse_s[8 * g4 + 4 * h]);
+            d4[g4] = *reinterpret_cast<const f32x4 *>(&dlt_s[8 * g4 + 4 * h]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (HAS_IDX && (e == 0 || GSHIFT < 2)) mw[4 * g4 + e] = mask_s[(8 * g4 + 4 * h + e) >> GSHIFT];
+        }
+    };
+    auto gemms = [&](int b, f32x16 &sacc, f32x16 &pacc) {            // S and dP of block b
+        const unsigned char *qt = qd_ring + (b & 3) * QD_SLOT, *dot = qt + TILE_B;
+        sacc = zero16();
+        pacc = zero16();
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            sacc = mfma32(lo.rowop(qt, ks), kB[ks], sacc);
+            pacc = mfma32(lo.rowop(dot, ks), vB[ks], pacc);
+        }
+        sched_reads_ahead<2 * KS, 4, 1>();
+    };
+    // P and dS of element vi (C layout) of block b from its S and dP accumulators
+    auto element = [&](auto may_diag, int b, int vi, const f32x16 &sacc, const f32x16 &pacc, float sl2, uint32_t &keep,
+                       float *pv, float *dsv) {
+        const int g4 = vi >> 2, e = vi & 3, row = 8 * g4 + 4 * h + e;
+        if (e == 0 || GSHIFT < 2) {                      // rows of one query share the mask bit
+            const int qcb = q0 + b * QB, qi = row >> GSHIFT;
+            uint32_t w = HAS_IDX ? mw[vi] : 0xffffffffu;
+            if (decltype(may_diag)::value && causal && qcb < kc + 32) w &= causal_bits(qcb + qi - kc);
+            keep = bit_mask(w, j);
+        }
+        const float p = fast_exp2(keep_or_neginf(fmaf(sacc[vi], sl2, -l4[g4][e]), keep));
+        pv[vi] = p;
+        dsv[vi] = p * (pacc[vi] - d4[g4][e]);
+    };
+    auto store_pd = [&](int b, const float *pv, const float *dsv) {  // -> ring slot b % 2, MFMA B layout
+        unsigned char *pd = pd_ring + (b & 1) * PD_SLOT + kg * 4096 + lane * 16;
+        *reinterpret_cast<bf16x8 *>(pd) = pack8(pv);
+        *reinterpret_cast<bf16x8 *>(pd + 1024) = pack8(pv + 8);
+        *reinterpret_cast<bf16x8 *>(pd + 2048) = pack8(dsv);
+        *reinterpret_cast<bf16x8 *>(pd + 3072) = pack8(dsv + 8);
+    };
+    auto softmax = [&](auto may_diag, int b, const f32x16 &sacc, const f32x16 &pacc) {
+        float pv[16], dsv[16];
+        uint32_t keep = 0u;
+#pragma unroll
+        for (int vi = 0; vi < 16; ++vi) element(may_diag, b, vi, sacc, pacc, scale_log2, keep, pv, dsv);
+        store_pd(b, pv, dsv);
+    };
+    // GEMMs of block b+1 into (sn, pn) with the softmax of block b from (sc, pc) between them: after
+    // every MFMA the vector work of 16 / (2 KS) elements, operand reads four MFMAs ahead.  The order
+    // is fixed by hand: every step ends in an empty asm statement that the step's results, the next
+    // MFMA's operand and the scale used by the next step's arithmetic pass through.
+    auto fused = [&](auto may_diag, int b, const f32x16 &sc, const f32x16 &pc, f32x16 &sn, f32x16 &pn) {
+        constexpr int NM = 2 * KS, EPM = 16 / NM;
+        const unsigned char *qt = qd_ring + ((b + 1) & 3) * QD_SLOT, *dot = qt + TILE_B;
+        float pv[16], dsv[16], sl2 = scale_log2;
+        uint32_t keep = 0u;
+        bf16x8 a[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[i] = lo.rowop((i & 1) ? dot : qt, i >> 1);
+        sn = zero16();
+        pn = zero16();
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+            if (i & 1) pn = mfma32(a[i & 3], vB[i >> 1], pn);
+            else sn = mfma32(a[i & 3], kB[i >> 1], sn);
+            if (i + 4 < NM) a[i & 3] = lo.rowop((i & 1) ? dot : qt, (i + 4) >> 1);
+#pragma unroll
+            for (int u = 0; u < EPM; ++u) element(may_diag, b, i * EPM + u, sc, pc, sl2, keep, pv, dsv);
+            if (EPM == 1)
+                asm volatile("" : "+v"(sl2), "+v"(pv[i]), "+v"(dsv[i]), "+v"(a[(i + 1) & 3]) : : "memory");
+            else
+                asm volatile("" : "+v"(sl2), "+v"(pv[2 * i]), "+v"(dsv[2 * i]), "+v"(pv[2 * i + 1]), "+v"(dsv[2 * i + 1]),
+                             "+v"(a[(i + 1) & 3]) : : "memory");
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        store_pd(b, pv, dsv);
+    };
+    // one producer step
+#define DKV_PRODUCER_STEP(B, SC, PC, SN, PN, MAY_DIAG)                                              \
+    {                                                                                              \
+        if ((B) + 1 < nblocks) fused(MAY_DIAG, B, SC, PC, SN, PN);                                 \
+        else if ((B) < nblocks) softmax(MAY_DIAG, B, SC, PC);                                      \
+        if ((B) + 1 < nblocks) read_aux((B) + 1);                                                  \
+        __syncthreads();                                                                           \
+    }
+    f32x16 s_a, p_a, s_b, p_b;
+    __syncthreads();                                     // blocks 0 and 1 staged
+    gemms(0, s_a, p_a);
+    read_aux(0);
+    // blocks that can touch the causal diagonal come first (rounded up to a pair of steps); the steady
+    // loop after them has no mask arithmetic besides the selection bits and is one basic block
+    const std::true_type diag_y;
+    const std::false_type diag_n;
+    const int nb_diag = causal ? ((kc + 32 - q0 + QB - 1) / QB + 1) & ~1 : 0;
+    int b = 0;
+    for (; b < nb_diag && b + 1 <= nblocks; b += 2) {
+        DKV_PRODUCER_STEP(b, s_a, p_a, s_b, p_b, diag_y)
+        DKV_PRODUCER_STEP(b + 1, s_b, p_b, s_a, p_a, diag_y)
+    }
+    for (; b + 1 <= nblocks; b += 2) {
+        DKV_PRODUCER_STEP(b, s_a, p_a, s_b, p_b, diag_n)
+        DKV_PRODUCER_STEP(b + 1, s_b, p_b, s_a, p_a, diag_n)
+    }
+    if (b <= nblocks) DKV_PRODUCER_STEP(b, s_a, p_a, s_b, p_b, diag_y)
+#undef DKV_PRODUCER_STEP
 }
 template <int D>
-constexpr size_t dkvpc_lds_bytes() { return 3 * (2 * 32 * D * 2) + 2 * (4 * 4 * 1024) + 3 * ((32 + 32 + 4 * 32) * 4); }
+constexpr size_t dkvpc_lds_bytes() { return 4 * (2 * tile_bytes<D>()) + 2 * (4 * 4 * 1024) + 4 * ((32 + 32 + 4 * 32) * 4); }
 
 // ==================================================================================================
 // launchers: instantiate per head_dim, mask kind and (power-of-two padded) group size
@@ -811,7 +872,7 @@ static void launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, const 
     if constexpr (D <= 128) {
         static bool configured = false;                  // LDS above 64 KiB has to be requested once per kernel
         if (!configured) {
-            hipFuncSetAttribute(reinterpret_cast<const void *>(&dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>),
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkvpc_lds_bytes<D>());
             configured = true;
         }
