@@ -628,47 +628,85 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
         } else {
             aux_base = reinterpret_cast<const uint32_t *>(lse);
         }
+        // Per-thread element offsets of block 0 and what the last block adds to them (its rows past the
+        // segment end re-read row L-1); in between a block moves every address by the same stride, so
+        // the loop does no index arithmetic per row.
+        const int last = nblocks - 1;
+        const int64_t blk_bytes = (int64_t)QB * Hq * D * 2;
+        const unsigned char *qp[CPT], *dp[CPT];          // this thread's chunks of the block loaded last
+        int64_t dlast[CPT];
+        int lds_off[CPT];
+        bool row_dead_last[CPT], head_ok[CPT];
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const int c = i * 256 + ctid, srow = c / CPR, sch = c % CPR;
+            const int hd = min(srow & (Gp - 1), G - 1);
+            const int qr = srow >> GSHIFT;
+            const int over0 = max(q0 + qr - (L - 1), 0);                 // block 0 may already be the last one
+            const int64_t off = ((int64_t)(s0 + q0 + qr - over0) * Hq + kvh * G + hd) * D + sch * 8;
+            qp[i] = reinterpret_cast<const unsigned char *>(q + off);
+            dp[i] = reinterpret_cast<const unsigned char *>(dout + off);
+            const int over = max(q0 + last * QB + qr - (L - 1), 0);      // rows past the end in the last block
+            dlast[i] = -(int64_t)over * Hq * D * 2;
+            row_dead_last[i] = over > 0;
+            head_ok[i] = (srow & (Gp - 1)) < G;
+            lds_off[i] = tile_off<D>(srow, sch);
+        }
+        const int64_t aux_blk_bytes = (int64_t)aux_stride * QB * 4;
+        const int aux_over = max(q0 + last * QB + aux_q - (L - 1), 0);
+        const int64_t aux_dlast = -(int64_t)aux_stride * aux_over * 4;
+        const unsigned char *ap = reinterpret_cast<const unsigned char *>(aux_base + (int64_t)aux_stride * min(q0 + aux_q, L - 1));
         u32x4 qst[CPT], dost[CPT];
         uint32_t aux_st;
-        auto gload = [&](int b) {                        // block index clamped by the caller
-            const int qcb = q0 + b * QB;
+        // loads block b, called with b = 0, 1, 2, ... in turn; past the last block it reads the last one again
+        auto gload = [&](int b) {
+            if (b >= 1 && b <= last) {
+#pragma unroll
+                for (int i = 0; i < CPT; ++i) { qp[i] += blk_bytes; dp[i] += blk_bytes; }
+                ap += aux_blk_bytes;
+                if (b == last && last >= 1) {
+#pragma unroll
+                    for (int i = 0; i < CPT; ++i) { qp[i] += dlast[i]; dp[i] += dlast[i]; }
+                    ap += aux_dlast;
+                }
+            }
 #pragma unroll
             for (int i = 0; i < CPT; ++i) {
-                const int c = i * 256 + ctid, srow = c / CPR, sch = c % CPR;
-                const int qc = min(qcb + (srow >> GSHIFT), L - 1);
-                const int hd = min(srow & (Gp - 1), G - 1);
-                const int64_t off = ((int64_t)(s0 + qc) * Hq + kvh * G + hd) * D + sch * 8;
-                qst[i] = *reinterpret_cast<const u32x4 *>(q + off);
-                dost[i] = *reinterpret_cast<const u32x4 *>(dout + off);
+                qst[i] = *reinterpret_cast<const u32x4 *>(qp[i]);
+                dost[i] = *reinterpret_cast<const u32x4 *>(dp[i]);
             }
-            aux_st = aux_base[(int64_t)aux_stride * min(qcb + aux_q, L - 1)];
+            aux_st = *reinterpret_cast<const uint32_t *>(ap);
         };
         auto lstore = [&](int b) {                       // registers -> ring slot b % 4
-            const int qcb = q0 + b * QB;
             unsigned char *slot = qd_ring + (b & 3) * QD_SLOT;
             float *lse_s = reinterpret_cast<float *>(aux_ring + (b & 3) * AUX_SLOT);
             float *dlt_s = lse_s + 32;
             uint32_t *mask_s = reinterpret_cast<uint32_t *>(dlt_s + 32);
+            // rows past the segment (last block only) and padded heads are zeroed: they add nothing to dK, dV
+            const bool tail = b >= last;
 #pragma unroll
             for (int i = 0; i < CPT; ++i) {
-                const int c = i * 256 + ctid, srow = c / CPR, sch = c % CPR;
-                // rows past the segment and padded heads are zeroed: they add nothing to dK, dV
-                const bool live = qcb + (srow >> GSHIFT) < L && (srow & (Gp - 1)) < G;
-                const u32x4 z4 = {0u, 0u, 0u, 0u};
-                *reinterpret_cast<u32x4 *>(slot + tile_off<D>(srow, sch)) = live ? qst[i] : z4;
-                *reinterpret_cast<u32x4 *>(slot + TILE_B + tile_off<D>(srow, sch)) = live ? dost[i] : z4;
+                u32x4 qv = qst[i], dv4 = dost[i];
+                if (tail || G != Gp) {
+                    const bool live = head_ok[i] && !(b > last || (b == last && row_dead_last[i]));
+                    const u32x4 z4 = {0u, 0u, 0u, 0u};
+                    qv = live ? qv : z4;
+                    dv4 = live ? dv4 : z4;
+                }
+                *reinterpret_cast<u32x4 *>(slot + lds_off[i]) = qv;
+                *reinterpret_cast<u32x4 *>(slot + TILE_B + lds_off[i]) = dv4;
             }
             if (ctid < 32) lse_s[ctid] = __uint_as_float(aux_st) * LOG2E_F;
             else if (ctid < 64) dlt_s[ctid - 32] = __uint_as_float(aux_st);
             else if (HAS_IDX && ctid < 64 + 4 * QB)
-                mask_s[((ctid - 64) / QB) * 32 + (ctid - 64) % QB] = (aux_mask_ok && qcb + aux_q < L) ? aux_st : 0u;
+                mask_s[((ctid - 64) / QB) * 32 + (ctid - 64) % QB] =
+                    (aux_mask_ok && !(b > last || (b == last && aux_over > 0))) ? aux_st : 0u;
         };
-        const int last = nblocks - 1;
         gload(0);
         lstore(0);
-        gload(min(1, last));
+        gload(1);
         lstore(1);
-        gload(min(2, last));
+        gload(2);
         __syncthreads();                                 // blocks 0 and 1 staged
 
         f32x16 dkacc[DT], dvacc[DT];
@@ -676,7 +714,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
         for (int dt = 0; dt < DT; ++dt) { dkacc[dt] = zero16(); dvacc[dt] = zero16(); }
         for (int b = 0; b <= nblocks; ++b) {
             lstore(b + 2);                               // slot (b+2)%4 was last read (as block b-2) before the previous barrier
-            gload(min(b + 3, last));
+            gload(b + 3);
             if (b >= 1) {
                 const unsigned char *qt = qd_ring + ((b - 1) & 3) * QD_SLOT;
                 lds_u8 *pt[4];              // lane addresses in the q block; the dO block sits TILE_B behind
