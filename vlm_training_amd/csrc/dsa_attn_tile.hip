@@ -557,7 +557,9 @@ __global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
 
 // ==================================================================================================
 // dK, dV for head_dim <= 128, producer/consumer form.  A workgroup owns a 128-key tile (4 groups of 32
-// keys) of one segment and kv head and walks the later queries in blocks of 32 (query, head) rows.
+// keys) of one segment and kv head and walks the later queries in blocks of 32 (query, head) rows,
+// from the end of the segment down to the key tile: workgroups that run side by side then read the
+// same q / dO rows at about the same time and share them in L2.
 //   waves 0-3 (producers, one per key group): S = Q K^T and dP = dO V^T against the group's K / V rows
 //     held in registers, then P and dS = P * (dP - delta) in bf16, written to LDS in MFMA B layout.
 //     The two GEMMs of block b+1 are issued between the softmax arithmetic of block b: a SIMD overlaps
@@ -642,11 +644,10 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
             const int c = i * 256 + ctid, srow = c / CPR, sch = c % CPR;
             const int hd = min(srow & (Gp - 1), G - 1);
             const int qr = srow >> GSHIFT;
-            const int over0 = max(q0 + qr - (L - 1), 0);                 // block 0 may already be the last one
-            const int64_t off = ((int64_t)(s0 + q0 + qr - over0) * Hq + kvh * G + hd) * D + sch * 8;
+            const int over = max(q0 + last * QB + qr - (L - 1), 0);      // rows past the end in the last block
+            const int64_t off = ((int64_t)(s0 + q0 + last * QB + qr - over) * Hq + kvh * G + hd) * D + sch * 8;
             qp[i] = reinterpret_cast<const unsigned char *>(q + off);
             dp[i] = reinterpret_cast<const unsigned char *>(dout + off);
-            const int over = max(q0 + last * QB + qr - (L - 1), 0);      // rows past the end in the last block
             dlast[i] = -(int64_t)over * Hq * D * 2;
             row_dead_last[i] = over > 0;
             head_ok[i] = (srow & (Gp - 1)) < G;
@@ -655,19 +656,21 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
         const int64_t aux_blk_bytes = (int64_t)aux_stride * QB * 4;
         const int aux_over = max(q0 + last * QB + aux_q - (L - 1), 0);
         const int64_t aux_dlast = -(int64_t)aux_stride * aux_over * 4;
-        const unsigned char *ap = reinterpret_cast<const unsigned char *>(aux_base + (int64_t)aux_stride * min(q0 + aux_q, L - 1));
+        const unsigned char *ap =
+            reinterpret_cast<const unsigned char *>(aux_base + (int64_t)aux_stride * (q0 + last * QB + aux_q - aux_over));
         u32x4 qst[CPT], dost[CPT];
         uint32_t aux_st;
-        // loads block b, called with b = 0, 1, 2, ... in turn; past the last block it reads the last one again
+        // loads the block of step b (block last - b), called with b = 0, 1, 2, ... in turn; past step
+        // `last` it reads block 0 again
         auto gload = [&](int b) {
             if (b >= 1 && b <= last) {
 #pragma unroll
-                for (int i = 0; i < CPT; ++i) { qp[i] += blk_bytes; dp[i] += blk_bytes; }
-                ap += aux_blk_bytes;
-                if (b == last && last >= 1) {
+                for (int i = 0; i < CPT; ++i) { qp[i] -= blk_bytes; dp[i] -= blk_bytes; }
+                ap -= aux_blk_bytes;
+                if (b == 1) {                            // leaving the last block: undo its row clamp
 #pragma unroll
-                    for (int i = 0; i < CPT; ++i) { qp[i] += dlast[i]; dp[i] += dlast[i]; }
-                    ap += aux_dlast;
+                    for (int i = 0; i < CPT; ++i) { qp[i] -= dlast[i]; dp[i] -= dlast[i]; }
+                    ap -= aux_dlast;
                 }
             }
 #pragma unroll
@@ -677,18 +680,18 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
             }
             aux_st = *reinterpret_cast<const uint32_t *>(ap);
         };
-        auto lstore = [&](int b) {                       // registers -> ring slot b % 4
+        auto lstore = [&](int b) {                       // registers (step b) -> ring slot b % 4
             unsigned char *slot = qd_ring + (b & 3) * QD_SLOT;
             float *lse_s = reinterpret_cast<float *>(aux_ring + (b & 3) * AUX_SLOT);
             float *dlt_s = lse_s + 32;
             uint32_t *mask_s = reinterpret_cast<uint32_t *>(dlt_s + 32);
             // rows past the segment (last block only) and padded heads are zeroed: they add nothing to dK, dV
-            const bool tail = b >= last;
+            const bool tail = b == 0 || b > last;
 #pragma unroll
             for (int i = 0; i < CPT; ++i) {
                 u32x4 qv = qst[i], dv4 = dost[i];
                 if (tail || G != Gp) {
-                    const bool live = head_ok[i] && !(b > last || (b == last && row_dead_last[i]));
+                    const bool live = head_ok[i] && !(b > last || (b == 0 && row_dead_last[i]));
                     const u32x4 z4 = {0u, 0u, 0u, 0u};
                     qv = live ? qv : z4;
                     dv4 = live ? dv4 : z4;
@@ -700,7 +703,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
             else if (ctid < 64) dlt_s[ctid - 32] = __uint_as_float(aux_st);
             else if (HAS_IDX && ctid < 64 + 4 * QB)
                 mask_s[((ctid - 64) / QB) * 32 + (ctid - 64) % QB] =
-                    (aux_mask_ok && !(b > last || (b == last && aux_over > 0))) ? aux_st : 0u;
+                    (aux_mask_ok && !(b > last || (b == 0 && aux_over > 0))) ? aux_st : 0u;
         };
         gload(0);
         lstore(0);
@@ -793,7 +796,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
                        float *pv, float *dsv) {
         const int g4 = vi >> 2, e = vi & 3, row = 8 * g4 + 4 * h + e;
         if (e == 0 || GSHIFT < 2) {                      // rows of one query share the mask bit
-            const int qcb = q0 + b * QB, qi = row >> GSHIFT;
+            const int qcb = q0 + (nblocks - 1 - b) * QB, qi = row >> GSHIFT;
             uint32_t w = HAS_IDX ? mw[vi] : 0xffffffffu;
             if (decltype(may_diag)::value && causal && qcb < kc + 32) w &= causal_bits(qcb + qi - kc);
             keep = bit_mask(w, j);
@@ -858,19 +861,20 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     __syncthreads();                                     // blocks 0 and 1 staged
     gemms(0, s_a, p_a);
     read_aux(0);
-    // blocks that can touch the causal diagonal come first (rounded up to a pair of steps); the steady
-    // loop after them has no mask arithmetic besides the selection bits and is one basic block
+    // The blocks that can touch the causal diagonal come last; the steady loop before them has no mask
+    // arithmetic besides the selection bits and is one basic block.
     const std::true_type diag_y;
     const std::false_type diag_n;
-    const int nb_diag = causal ? ((kc + 32 - q0 + QB - 1) / QB + 1) & ~1 : 0;
+    const int nb_diag = causal ? (kc + 32 - q0 + QB - 1) / QB : 0;
+    const int steady = max(nblocks - nb_diag, 0) & ~1;   // steps [0, steady) see blocks fully past the diagonal
     int b = 0;
-    for (; b < nb_diag && b + 1 <= nblocks; b += 2) {
-        DKV_PRODUCER_STEP(b, s_a, p_a, s_b, p_b, diag_y)
-        DKV_PRODUCER_STEP(b + 1, s_b, p_b, s_a, p_a, diag_y)
-    }
-    for (; b + 1 <= nblocks; b += 2) {
+    for (; b < steady; b += 2) {
         DKV_PRODUCER_STEP(b, s_a, p_a, s_b, p_b, diag_n)
         DKV_PRODUCER_STEP(b + 1, s_b, p_b, s_a, p_a, diag_n)
+    }
+    for (; b + 1 <= nblocks; b += 2) {
+        DKV_PRODUCER_STEP(b, s_a, p_a, s_b, p_b, diag_y)
+        DKV_PRODUCER_STEP(b + 1, s_b, p_b, s_a, p_a, diag_y)
     }
     if (b <= nblocks) DKV_PRODUCER_STEP(b, s_a, p_a, s_b, p_b, diag_y)
 #undef DKV_PRODUCER_STEP
