@@ -658,11 +658,12 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
         const int64_t aux_dlast = -(int64_t)aux_stride * aux_over * 4;
         const unsigned char *ap =
             reinterpret_cast<const unsigned char *>(aux_base + (int64_t)aux_stride * (q0 + last * QB + aux_q - aux_over));
-        u32x4 qst[CPT], dost[CPT];
-        uint32_t aux_st;
+        // two register sets: a global load has two block-times to land before its LDS store
+        u32x4 qst0[CPT], dost0[CPT], qst1[CPT], dost1[CPT];
+        uint32_t aux_st0, aux_st1;
         // loads the block of step b (block last - b), called with b = 0, 1, 2, ... in turn; past step
         // `last` it reads block 0 again
-        auto gload = [&](int b) {
+        auto gload = [&](int b, u32x4 (&qst)[CPT], u32x4 (&dost)[CPT], uint32_t &aux_st) {
             if (b >= 1 && b <= last) {
 #pragma unroll
                 for (int i = 0; i < CPT; ++i) { qp[i] -= blk_bytes; dp[i] -= blk_bytes; }
@@ -680,7 +681,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
             }
             aux_st = *reinterpret_cast<const uint32_t *>(ap);
         };
-        auto lstore = [&](int b) {                       // registers (step b) -> ring slot b % 4
+        auto lstore = [&](int b, const u32x4 (&qst)[CPT], const u32x4 (&dost)[CPT], uint32_t aux_st) {   // step b -> ring slot b % 4
             unsigned char *slot = qd_ring + (b & 3) * QD_SLOT;
             float *lse_s = reinterpret_cast<float *>(aux_ring + (b & 3) * AUX_SLOT);
             float *dlt_s = lse_s + 32;
@@ -705,41 +706,52 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
                 mask_s[((ctid - 64) / QB) * 32 + (ctid - 64) % QB] =
                     (aux_mask_ok && !(b > last || (b == 0 && aux_over > 0))) ? aux_st : 0u;
         };
-        gload(0);
-        lstore(0);
-        gload(1);
-        lstore(1);
-        gload(2);
-        __syncthreads();                                 // blocks 0 and 1 staged
+        gload(0, qst0, dost0, aux_st0);
+        gload(1, qst1, dost1, aux_st1);
+        lstore(0, qst0, dost0, aux_st0);
+        lstore(1, qst1, dost1, aux_st1);
+        gload(2, qst0, dost0, aux_st0);
+        gload(3, qst1, dost1, aux_st1);
+        __syncthreads();                                 // steps 0 and 1 staged
 
         f32x16 dkacc[DT], dvacc[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) { dkacc[dt] = zero16(); dvacc[dt] = zero16(); }
-        for (int b = 0; b <= nblocks; ++b) {
-            lstore(b + 2);                               // slot (b+2)%4 was last read (as block b-2) before the previous barrier
-            gload(b + 3);
-            if (b >= 1) {
-                const unsigned char *qt = qd_ring + ((b - 1) & 3) * QD_SLOT;
-                lds_u8 *pt[4];              // lane addresses in the q block; the dO block sits TILE_B behind
+        // one consumer step: stage step B+2 from the given register set, refill it with step B+4, then the MFMAs of step B-1
+#define DKV_CONSUMER_STEP(B, QS, DS, AS)                                                            \
+    {                                                                                              \
+        lstore((B) + 2, QS, DS, AS);    /* slot (B+2)%4 was last read (as step B-2) before the previous barrier */ \
+        gload((B) + 4, QS, DS, AS);                                                                \
+        if ((B) >= 1) consume((B) - 1);                                                            \
+        __syncthreads();                                                                           \
+    }
+        auto consume = [&](int b) {
+            const unsigned char *qt = qd_ring + (b & 3) * QD_SLOT;
+            lds_u8 *pt[4];                  // lane addresses in the q block; the dO block sits TILE_B behind
 #pragma unroll
-                for (int vv = 0; vv < 4; ++vv) {
-                    pt[vv] = (lds_u8 *)qt + lo.tr[vv];
-                    asm volatile("" : "+v"(pt[vv]));     // keep "address + immediate" reads: no re-association
-                }
-                const unsigned char *pd = pd_ring + ((b - 1) & 1) * PD_SLOT + kg * 4096 + lane * 16;
-                const bf16x8 pB0 = *reinterpret_cast<const bf16x8 *>(pd), pB1 = *reinterpret_cast<const bf16x8 *>(pd + 1024);
-                const bf16x8 dB0 = *reinterpret_cast<const bf16x8 *>(pd + 2048), dB1 = *reinterpret_cast<const bf16x8 *>(pd + 3072);
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    dvacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 0, dt, TILE_B), pB0, dvacc[dt]);
-                    dkacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 0, dt, 0), dB0, dkacc[dt]);
-                    dvacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 1, dt, TILE_B), pB1, dvacc[dt]);
-                    dkacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 1, dt, 0), dB1, dkacc[dt]);
-                }
-                sched_reads_ahead<4 * DT, 3, 2, 4>();
+            for (int vv = 0; vv < 4; ++vv) {
+                pt[vv] = (lds_u8 *)qt + lo.tr[vv];
+                asm volatile("" : "+v"(pt[vv]));         // keep "address + immediate" reads: no re-association
             }
-            __syncthreads();
+            const unsigned char *pd = pd_ring + (b & 1) * PD_SLOT + kg * 4096 + lane * 16;
+            const bf16x8 pB0 = *reinterpret_cast<const bf16x8 *>(pd), pB1 = *reinterpret_cast<const bf16x8 *>(pd + 1024);
+            const bf16x8 dB0 = *reinterpret_cast<const bf16x8 *>(pd + 2048), dB1 = *reinterpret_cast<const bf16x8 *>(pd + 3072);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                dvacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 0, dt, TILE_B), pB0, dvacc[dt]);
+                dkacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 0, dt, 0), dB0, dkacc[dt]);
+                dvacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 1, dt, TILE_B), pB1, dvacc[dt]);
+                dkacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 1, dt, 0), dB1, dkacc[dt]);
+            }
+            sched_reads_ahead<4 * DT, 3, 2, 4>();
+        };
+        int b = 0;
+        for (; b + 1 <= nblocks; b += 2) {
+            DKV_CONSUMER_STEP(b, qst0, dost0, aux_st0)
+            DKV_CONSUMER_STEP(b + 1, qst1, dost1, aux_st1)
         }
+        if (b <= nblocks) DKV_CONSUMER_STEP(b, qst0, dost0, aux_st0)
+#undef DKV_CONSUMER_STEP
         if (key_ok) {
             bf16_t *pk = dk + krow * D + 4 * h, *pv_ = dv + krow * D + 4 * h;
 #pragma unroll
