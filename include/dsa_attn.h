@@ -102,6 +102,13 @@ int dsa_get_tile_crossover(void);
 
 /* Bytes of workspace dsa_attn_bwd needs (softmax row terms + the inverted selection bitmap). */
 size_t dsa_attn_bwd_workspace_bytes(int T, int Hq, int max_seqlen, int has_idx);
+/*
+ * Byte offset of the selection bitmap inside the backward workspace.  A forward call handed
+ * `ws + offset` as its workspace leaves the bitmap where a later dsa_attn_bwd_parts on the same `ws`
+ * finds it, so that backward can be run without DSA_BWD_BITMAP (the autograd wrapper does this).
+ * No reference counterpart: the reference's attention saves no selection.
+ */
+size_t dsa_attn_bwd_bitmap_offset(int T, int Hq);
 
 /*
  * Stage D4 - gradients of D3 (the autograd backward of varlen_attn restricted to the selected keys;

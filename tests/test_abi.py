@@ -37,6 +37,7 @@ def test_workspace_sizes_without_a_gpu():
     assert lib.dsa_attn_bwd_workspace_bytes(1000, 8, 640, 0) == up(1000 * 8 * 4)
     assert lib.dsa_attn_bwd_workspace_bytes(1000, 8, 640, 1) == up(1000 * 8 * 4) + up(1000 * 20 * 4)
     assert lib.dsa_attn_fwd_workspace_bytes(1000, 640, 1) == up(1000 * 20 * 4)
+    assert lib.dsa_attn_bwd_bitmap_offset(1000, 8) == up(1000 * 8 * 4)   # forward workspace fits behind it
     assert lib.dsa_attn_fwd_workspace_bytes(1000, 640, 0) == 0
     old = lib.dsa_get_tile_crossover()
     assert old == 16 and lib.dsa_set_tile_crossover(-1) == -1 and lib.dsa_set_tile_crossover(3) == 0

@@ -328,3 +328,46 @@ def test_argument_errors_cross_the_boundary_as_exceptions():
         ops.dsa_varlen_attn(q, k, k, cu, 8)            # head_dim 96 is not covered by the kernels
     with pytest.raises(RuntimeError):
         ops.dsa_varlen_attn(q.cpu(), k.cpu(), k.cpu(), cu.cpu(), 8)
+
+
+# ------------------------------------------------------------------------------------------ golden fixtures
+def _golden(name):
+    import os
+
+    import numpy as np
+    return np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name))
+
+
+def test_golden_tie_cases_bit_exact():
+    """Selections worked out by brute force in plain Python (tests/golden/make_golden.py)."""
+    _log("golden ties")
+    z = _golden("topk_ties.npz")
+    for name in z["names"]:
+        sc = torch.from_numpy(z[f"{name}/scores"])
+        L, K = sc.shape[0], int(z[f"{name}/K"])
+        idx, n = ops.topk_from_scores(sc.to(DEV).contiguous(), torch.tensor([0, L], dtype=torch.int32, device=DEV), K)
+        torch.cuda.synchronize()
+        assert torch.equal(n.cpu(), torch.from_numpy(z[f"{name}/n"])), name
+        assert torch.equal(idx.cpu(), torch.from_numpy(z[f"{name}/idx"])), name
+
+
+def test_golden_toy_configuration():
+    """C1 against the float64 loop-level restatement: selection (where fp32 and float64 scores agree on
+    the order), then outputs and gradients on the golden selection."""
+    _log("golden C1")
+    z = _golden("c1_toy.npz")
+    w = W.C1
+    t = W.make_inputs(w, device="cpu")
+    d = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in t.items()}
+    gidx = torch.from_numpy(z["idx"].astype("int32"))
+    gn = torch.from_numpy(z["n"].astype("int32"))
+    idx, n = ops.index_topk(d["q_idx"], d["k_idx"], d["w_idx"], d["cu_seqlens"], w.max_seqlen, w.top_k)
+    assert torch.equal(n.cpu(), gn)
+    assert (idx.cpu() == gidx).all(dim=1).float().mean().item() > 0.995
+    q, k, v = (d[x].clone().requires_grad_(True) for x in ("q", "k", "v"))
+    out = ops._DsaVarlenAttn.apply(q, k, v, d["cu_seqlens"], w.max_seqlen, gidx.to(DEV), gn.to(DEV), w.D ** -0.5, True)
+    out.backward(d["dout"])
+    torch.cuda.synchronize()
+    rows = torch.from_numpy(z["rows"]).long()
+    for name, got in (("out", out), ("dq", q.grad), ("dk", k.grad), ("dv", v.grad)):
+        assert_close_bf16(got.detach().cpu()[rows], torch.from_numpy(z[name]), "golden " + name)

@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libdsa_attn.so")
 
 DSA_DTYPE_BF16 = 0
 DSA_DTYPE_FP32 = 1
+DSA_BWD_DELTA, DSA_BWD_BITMAP, DSA_BWD_DQ, DSA_BWD_DKV, DSA_BWD_ALL = 1, 2, 4, 8, 15      # parts of dsa_attn_bwd_parts
 
 _SIGNATURES = {
     "dsa_version": (c_char_p, []),
@@ -30,6 +31,7 @@ _SIGNATURES = {
     "dsa_set_tile_crossover": (c_int, [c_int]),
     "dsa_get_tile_crossover": (c_int, []),
     "dsa_attn_bwd_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "dsa_attn_bwd_bitmap_offset": (c_size_t, [c_int, c_int]),
     "dsa_attn_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                              c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p,
                              c_void_p, c_void_p, c_size_t, c_void_p]),

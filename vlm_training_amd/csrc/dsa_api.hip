@@ -198,6 +198,11 @@ extern "C" size_t dsa_attn_bwd_workspace_bytes(int T, int Hq, int max_seqlen, in
     return b;
 }
 
+extern "C" size_t dsa_attn_bwd_bitmap_offset(int T, int Hq) {
+    if (T <= 0 || Hq <= 0) return 0;
+    return align_up((size_t)T * Hq * 4, 256);
+}
+
 extern "C" int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k, const void *v, const void *out,
                                   const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu, int T,
                                   int N, int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen,
@@ -213,7 +218,7 @@ extern "C" int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k
     const int ldw = bitmap_ldw(max_seqlen);
     if (idx && (size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);
     float *delta = (float *)ws;
-    uint32_t *bitmap = idx ? (uint32_t *)((char *)ws + align_up((size_t)T * Hq * 4, 256)) : nullptr;
+    uint32_t *bitmap = idx ? (uint32_t *)((char *)ws + dsa_attn_bwd_bitmap_offset(T, Hq)) : nullptr;
     const int split = pos_split_for(idx, K);
     hipStream_t st = (hipStream_t)stream;
     hipError_t e = hipSuccess;

@@ -128,7 +128,9 @@ def set_tile_crossover(crossover: int) -> int:
     return old
 
 
-def attn_fwd(q, k, v, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float, causal: bool = True):
+def attn_fwd(q, k, v, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float, causal: bool = True, ws=None):
+    """Stage D3.  ``ws`` (optional, uint8) is used as the workspace instead of a fresh allocation; the
+    autograd wrapper passes the tail of the backward workspace so that the selection bitmap is built once."""
     T, Hq, Hkv, D = _check_qkv(q, k, v)
     cu = _check_cu(cu_seqlens, T)
     out = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=q.device)
@@ -136,7 +138,10 @@ def attn_fwd(q, k, v, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float,
     K = idx.shape[1] if idx is not None else 0
     lib = _lib.load()
     ws_bytes = lib.dsa_attn_fwd_workspace_bytes(T, max_seqlen, 1 if idx is not None else 0)
-    ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q.device)
+    if ws is None:
+        ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q.device)
+    elif ws.numel() < ws_bytes:
+        raise ValueError(f"forward workspace: have {ws.numel()} bytes, need {ws_bytes}")
     rc = lib.dsa_attn_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(idx), _ptr(n), _ptr(cu), T, cu.numel() - 1, Hq, Hkv, D, K,
                           softmax_scale, _lib.DSA_DTYPE_BF16, max_seqlen, 1 if causal else 0, _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
                           _stream(q.device))
@@ -200,7 +205,18 @@ class _DsaVarlenAttn(torch.autograd.Function):
             qb, kb, vb = _stack((qh, ql, qh), D), _stack((kh, kh, kl), D), _stack((vh, vl, vh), D)
         else:
             qb, kb, vb = _as_bf16(q), _as_bf16(k), _as_bf16(v)
-        out, lse = attn_fwd(qb, kb, vb, idx, n, cu_seqlens, int(max_seqlen), softmax_scale, causal)
+        bwd_ws = None
+        if idx is not None:
+            # one workspace for forward and backward: the bitmap the forward builds stays where the backward reads it
+            lib = _lib.load()
+            T, Hq = qb.shape[0], qb.shape[1]
+            bwd_ws = torch.empty((max(lib.dsa_attn_bwd_workspace_bytes(T, Hq, int(max_seqlen), 1), 4),), dtype=torch.uint8,
+                                 device=qb.device)
+            fwd_ws = bwd_ws[lib.dsa_attn_bwd_bitmap_offset(T, Hq):]
+            out, lse = attn_fwd(qb, kb, vb, idx, n, cu_seqlens, int(max_seqlen), softmax_scale, causal, ws=fwd_ws)
+        else:
+            out, lse = attn_fwd(qb, kb, vb, idx, n, cu_seqlens, int(max_seqlen), softmax_scale, causal)
+        ctx.bwd_ws = bwd_ws
         ctx.causal = bool(causal)
         ctx.save_for_backward(qb, kb, vb, out, lse, cu_seqlens, *(() if idx is None else (idx, n)))
         ctx.has_idx = idx is not None
@@ -224,8 +240,14 @@ class _DsaVarlenAttn(torch.autograd.Function):
             db = _stack((gh, gh, gl), D)
         else:
             db = _as_bf16(dout)
-        dq, dk, dv = attn_bwd(db, qb, kb, vb, out, lse, idx, n, cu, ctx.max_seqlen, ctx.softmax_scale,
-                              causal=ctx.causal)
+        if ctx.bwd_ws is not None:                       # the forward left the selection bitmap in the workspace
+            bufs = (torch.empty_like(qb), torch.empty_like(kb), torch.empty_like(vb), ctx.bwd_ws)
+            dq, dk, dv, _ = attn_bwd(db, qb, kb, vb, out, lse, idx, n, cu, ctx.max_seqlen, ctx.softmax_scale,
+                                     parts=_lib.DSA_BWD_ALL & ~_lib.DSA_BWD_BITMAP, buffers=bufs, causal=ctx.causal)
+            ctx.bwd_ws = None
+        else:
+            dq, dk, dv = attn_bwd(db, qb, kb, vb, out, lse, idx, n, cu, ctx.max_seqlen, ctx.softmax_scale,
+                                  causal=ctx.causal)
         if ctx.split:
             dq = dq[..., :D].float() + dq[..., 2 * D:3 * D].float()
             dk = dk[..., :D].float() + dk[..., D:2 * D].float()
