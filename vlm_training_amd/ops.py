@@ -206,9 +206,9 @@ class _DsaVarlenAttn(torch.autograd.Function):
         else:
             qb, kb, vb = _as_bf16(q), _as_bf16(k), _as_bf16(v)
         bwd_ws = None
-        if idx is not None:
+        lib = _lib.load()
+        if idx is not None and lib.dsa_get_tile_crossover() > 0:     # (crossover 0: the forward builds no bitmap)
             # one workspace for forward and backward: the bitmap the forward builds stays where the backward reads it
-            lib = _lib.load()
             T, Hq = qb.shape[0], qb.shape[1]
             bwd_ws = torch.empty((max(lib.dsa_attn_bwd_workspace_bytes(T, Hq, int(max_seqlen), 1), 4),), dtype=torch.uint8,
                                  device=qb.device)
