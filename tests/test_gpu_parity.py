@@ -376,3 +376,25 @@ def test_golden_toy_configuration():
     rows = torch.from_numpy(z["rows"]).long()
     for name, got in (("out", out), ("dq", q.grad), ("dk", k.grad), ("dv", v.grad)):
         assert_close_bf16(got.detach().cpu()[rows], torch.from_numpy(z[name]), "golden " + name)
+
+
+# ------------------------------------------------------------------------------------------ sync-free bound
+def test_any_upper_bound_of_the_longest_segment_gives_the_same_result():
+    """max_seqlen=None (bound = T, no device-to-host copy of the lengths) against the exact maximum:
+    same selection, bit-identical outputs and gradients, sparse and dense, on a packed row built the
+    way the reference's collate step builds it (padding tail as the last segment)."""
+    _log("max_seqlen bound")
+    w = W.random_packed_workload(W.scaled(W.C2, (1,), top_k=96), max_length=3072, seed=11, mean_len=500)
+    assert w.T == 3072 and len(w.seg_lens) >= 3
+    t = W.make_inputs(w, device=DEV)
+    res = []
+    for ms in (w.max_seqlen, None, 3000):
+        q, k, v = (t[x].clone().requires_grad_(True) for x in ("q", "k", "v"))
+        out, idx, n = ops.dsa_varlen_attn(q, k, v, t["cu_seqlens"], ms, indexer_q=t["q_idx"], indexer_k=t["k_idx"],
+                                          indexer_w=t["w_idx"], top_k=w.top_k, return_indices=True)
+        out.backward(t["dout"])
+        dense = ops.dsa_varlen_attn(t["q"], t["k"], t["v"], t["cu_seqlens"], ms)
+        res.append((idx, n, out.detach(), q.grad, k.grad, v.grad, dense))
+    for other in res[1:]:
+        for a, b in zip(res[0], other):
+            assert torch.equal(a, b)

@@ -341,3 +341,15 @@ def test_oracle_reproduces_the_golden_toy_configuration():
     for name, got in (("out", out), ("dq", dq), ("dk", dk), ("dv", dv)):
         want = torch.from_numpy(z[name])
         assert torch.allclose(got[rows].float(), want, atol=2e-4, rtol=1e-4), (name, (got[rows].float() - want).abs().max())
+
+
+def test_pack_lengths_follows_the_reference_collate_convention():
+    """train/energon_dataloader.py:437-446: cumulative lengths, padding appended as a last segment."""
+    from vlm_training_amd import workloads as W
+    assert W.pack_lengths([5, 7], 16).tolist() == [0, 5, 12, 16]
+    assert W.pack_lengths([8, 8], 16).tolist() == [0, 8, 16]
+    with pytest.raises(ValueError):
+        W.pack_lengths([9, 8], 16)
+    w = W.random_packed_workload(W.C2, 8192, seed=3)
+    assert w.T == 8192 and w.cu[-1] == 8192 and min(w.seg_lens) >= 1
+    assert W.random_packed_workload(W.C2, 8192, seed=3).seg_lens == w.seg_lens

@@ -38,7 +38,8 @@ def varlen_attn(query, key, value, cu_seq_q, cu_seq_k, max_q, max_k, is_causal=N
         causal = True if is_causal is None else bool(is_causal)
     if return_aux is not None:
         raise NotImplementedError("return_aux is not supported")
-    return dsa_varlen_attn(query, key, value, cu_seq_q, int(max_q), softmax_scale=scale, causal=causal, **dsa)
+    return dsa_varlen_attn(query, key, value, cu_seq_q, None if max_q is None else int(max_q), softmax_scale=scale,
+                           causal=causal, **dsa)
 
 
 def dispatch_varlen_attention(q, k, v, cu_seqlens, max_seqlen, causal: bool = True, **dsa):
@@ -67,10 +68,10 @@ def varlen_attention_forward(query, key, value, attention_mask, **dsa):
     key = key.view(-1, key.size(-2), key.size(-1))
     value = value.view(-1, value.size(-2), value.size(-1))
     cu_seqlens = attention_mask.squeeze()
-    with torch.no_grad():
-        max_seqlen = torch.diff(cu_seqlens).max().item()
-    attn_output = varlen_attn(query, key, value, cu_seq_q=cu_seqlens, cu_seq_k=cu_seqlens, max_q=max_seqlen,
-                              max_k=max_seqlen, window_size=(-1, 0), **dsa)
+    # The reference reads the longest segment back to the host here (train/model_attention.py:120-121,
+    # a device sync per layer).  The kernels only need an upper bound, so the packed length serves.
+    attn_output = varlen_attn(query, key, value, cu_seq_q=cu_seqlens, cu_seq_k=cu_seqlens, max_q=None,
+                              max_k=None, window_size=(-1, 0), **dsa)
     if isinstance(attn_output, tuple):
         return (attn_output[0].unsqueeze(0), None) + tuple(attn_output[1:])
     return attn_output.unsqueeze(0), None

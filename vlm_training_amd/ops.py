@@ -257,13 +257,15 @@ class _DsaVarlenAttn(torch.autograd.Function):
         return dq, dk, dv, None, None, None, None, None, None
 
 
-def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: int, *, indexer_q=None, indexer_k=None, indexer_w=None,
+def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, indexer_q=None, indexer_k=None, indexer_w=None,
                     top_k: Optional[int] = None, index_scale: Optional[float] = None,
                     softmax_scale: Optional[float] = None, return_indices: bool = False, causal: bool = True):
     """Packed causal attention over ``cu_seqlens`` segments, optionally sparsified by the DSA indexer.
 
     q (T,Hq,D), k/v (T,Hkv,D) contiguous, cu_seqlens (N+1,) int32 on the device, max_seqlen host int
-    (the reference's callers already hold it: models/qwen3_vl/model.py:765).  Without indexer inputs
+    (the reference's callers already hold it: models/qwen3_vl/model.py:765) - any upper bound of the
+    longest segment gives the same result, and ``None`` stands for the bound T, which needs no
+    device-to-host copy of the segment lengths (train/model_attention.py:120-121 syncs for it).  Without indexer inputs
     every causal key of the token's own segment is attended (the reference's behaviour).  With
     ``indexer_q (T,Hi,Di)``, ``indexer_k (T,Di)``, ``indexer_w (T,Hi)`` and ``top_k`` each query keeps
     the top_k keys of its causal window under (indexer score descending, key index ascending).
@@ -274,6 +276,7 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: int, *, indexer_q=None, ind
     T, Hq, Hkv, D = _check_qkv(q, k, v)
     cu = _check_cu(cu_seqlens, T)
     scale = float(softmax_scale) if softmax_scale is not None else D ** -0.5
+    max_seqlen = T if max_seqlen is None else int(max_seqlen)
     sparse = indexer_q is not None or indexer_k is not None or indexer_w is not None
     idx = n = None
     if sparse and not causal:

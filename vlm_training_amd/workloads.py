@@ -124,3 +124,36 @@ def make_inputs(w: Workload, device="cpu", with_dout: bool = True):
     out["cu_seqlens"] = torch.tensor(w.cu, dtype=torch.int32, device=device)
     out["max_seqlen"] = w.max_seqlen
     return out
+
+
+def pack_lengths(sample_lengths, max_length: int, device="cpu"):
+    """``cu_seqlens`` of one packed row as the reference's collate step builds it
+    (train/energon_dataloader.py:431-464, ``PackedBatchEncoder.pack_selected_samples``): the samples back
+    to back, then - if they do not fill ``max_length`` - the padding as one more segment, so that the
+    last entry is always ``max_length``."""
+    total = int(sum(sample_lengths))
+    if total > max_length:
+        raise ValueError(f"samples ({total} tokens) do not fit max_length={max_length}")
+    cu = [0]
+    for n in sample_lengths:
+        cu.append(cu[-1] + int(n))
+    if total < max_length:
+        cu.append(max_length)
+    return torch.tensor(cu, dtype=torch.int32, device=device)
+
+
+def random_packed_workload(w: Workload, max_length: int, seed: int, mean_len: int = 1500, name=None) -> Workload:
+    """A packed row of ``max_length`` tokens filled greedily with log-normal sample lengths (the mix the
+    reference's packer sees: many short captions, a few long documents), padding tail included as the
+    last segment.  Deterministic in ``seed``; same head geometry as ``w``."""
+    g = torch.Generator().manual_seed(seed)
+    lens, total = [], 0
+    while True:
+        n = int(torch.empty(1).log_normal_(mean=0.0, std=0.9, generator=g).item() * mean_len * 0.67) + 16
+        if total + n > max_length - 64:
+            break
+        lens.append(n)
+        total += n
+    cu = pack_lengths(lens, max_length).tolist()
+    segs = tuple(b - a for a, b in zip(cu[:-1], cu[1:]))
+    return scaled(w, segs, name=name or f"{w.name}-packed{seed}")
