@@ -62,6 +62,44 @@ def cpu_baseline(w, threads):
     }
 
 
+def prologue_stage(w, dev, iters):
+    """The fused element-wise kernels either side of the operator, at the workload's geometry: HBM-bound,
+    so each is reported as algorithmic bytes / time against the 8 TB/s peak, beside the reference's own
+    sequence of eager torch ops (F.rms_norm, transposes, apply_rope, contiguous copies) on the same GPU."""
+    from oracle import prologue_ref as P
+    from vlm_training_amd import prologue
+    T, Hq, Hkv, D = w.T, w.Hq, w.Hkv, w.D
+    g = torch.Generator(device="cpu").manual_seed(w.seed)
+    mk = lambda *s: torch.randn(*s, generator=g).bfloat16().to(dev)
+    q, k, gq, gk = mk(T, Hq, D), mk(T, Hkv, D), mk(T, Hq, D), mk(T, Hkv, D)
+    qw, kw = mk(D) * 0.1 + 1, mk(D) * 0.1 + 1
+    ang = torch.arange(T, dtype=torch.float32, device=dev)[:, None] * (
+        1.0 / 1e6 ** (torch.arange(0, D, 2, dtype=torch.float32, device=dev) / D))[None, :]
+    cos, sin = torch.cat((ang.cos(), ang.cos()), -1).bfloat16(), torch.cat((ang.sin(), ang.sin()), -1).bfloat16()
+    gate = mk(T, Hq, D)
+    e = 2
+    rows = (Hq + Hkv) * D * e
+    res = {}
+
+    def entry(ms, nbytes):
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        return {"ms": ms, "algorithmic_bytes": nbytes, "GB/s": gbs, "frac_hbm_peak": gbs / PEAK_HBM_GBS}
+
+    qr, kr = q.clone().requires_grad_(True), k.clone().requires_grad_(True)
+    qwr, kwr = qw.clone().requires_grad_(True), kw.clone().requires_grad_(True)
+    with torch.no_grad():
+        ms = timed(lambda: prologue.qk_norm_rope(q, k, qw, kw, cos, sin), iters)
+        res["qk_norm_rope_fwd"] = entry(ms, T * (2 * rows + 2 * D * e + (Hq + Hkv) * 4))
+        eager = timed(lambda: P.qk_norm_rope(q, k, qw, kw, cos, sin, eager_bf16=True), iters)
+        res["qk_norm_rope_fwd"]["eager_torch_ms"] = eager
+        ms = timed(lambda: prologue.sigmoid_gate(q, gate), iters)
+        res["sigmoid_gate_fwd"] = entry(ms, T * Hq * D * e * 3)
+    oq, ok = prologue.qk_norm_rope(qr, kr, qwr, kwr, cos, sin)
+    ms = timed(lambda: torch.autograd.grad((oq, ok), (qr, kr, qwr, kwr), (gq, gk), retain_graph=True), iters)
+    res["qk_norm_rope_bwd"] = entry(ms, T * (3 * rows + 2 * D * e + (Hq + Hkv) * 4))
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -172,6 +210,7 @@ def main():
                               "compute_only_bound_ms": (wk["F1"] + 3.5 * wk["F3"]) / (PEAK_MFMA_BF16_TFLOPS * 1e12) * 1e3},
         "device": torch.cuda.get_device_name(0),
     }
+    result["adjacent_kernels"] = prologue_stage(w, dev, it)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, torch.get_num_threads())
     print(json.dumps(result))

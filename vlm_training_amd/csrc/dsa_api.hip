@@ -33,6 +33,25 @@ hipError_t dsa_launch_tile_dkv(const void *dout, const void *q, const void *k, c
                                int Hq, int Hkv, int D, float scale, int causal, void *dk, void *dv, hipStream_t stream);
 }
 
+extern "C" {
+int dsa_prologue_bwd_blocks(int T);
+hipError_t dsa_launch_qk_norm_rope_fwd(const void *q_in, int64_t q_tok, int64_t q_head, const void *k_in, int64_t k_tok,
+                                       int64_t k_head, const float *qw, const float *kw, float eps, float w_offset,
+                                       const void *cosp, const void *sinp, int cs_f32, int R, int T, int Hq, int Hkv, int D,
+                                       void *q_out, void *k_out, float *q_rstd, float *k_rstd, hipStream_t stream);
+hipError_t dsa_launch_qk_norm_rope_bwd(const void *gq, const void *gk, const void *q_in, int64_t q_tok, int64_t q_head,
+                                       const void *k_in, int64_t k_tok, int64_t k_head, const float *qw, const float *kw,
+                                       float w_offset, const void *cosp, const void *sinp, int cs_f32, int R,
+                                       const float *q_rstd, const float *k_rstd, int T, int Hq, int Hkv, int D, void *dq_in,
+                                       int64_t dq_tok, int64_t dq_head, void *dk_in, int64_t dk_tok, int64_t dk_head,
+                                       float *dqw, float *dkw, float *part, hipStream_t stream);
+hipError_t dsa_launch_sigmoid_gate_fwd(const void *x, const void *gate, int64_t gate_tok, int64_t gate_head, int D, int H,
+                                       int64_t rows, void *y, hipStream_t stream);
+hipError_t dsa_launch_sigmoid_gate_bwd(const void *gy, const void *x, const void *gate, int64_t gate_tok, int64_t gate_head,
+                                       int D, int H, int64_t rows, void *dx, void *dgate, int64_t dgate_tok,
+                                       int64_t dgate_head, hipStream_t stream);
+}
+
 static thread_local char g_err[512] = "";
 
 static int fail(int code, const char *fmt, ...) {
@@ -253,4 +272,75 @@ extern "C" int dsa_attn_bwd(const void *dout, const void *q, const void *k, cons
                             void *dq, void *dk, void *dv, void *ws, size_t ws_bytes, void *stream) {
     return dsa_attn_bwd_parts(dout, q, k, v, out, lse, idx, n, cu, T, N, Hq, Hkv, D, K, softmax_scale, dtype, max_seqlen,
                               causal, dq, dk, dv, ws, ws_bytes, DSA_BWD_ALL, stream);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// prologue / gate
+// ---------------------------------------------------------------------------------------------------
+static int check_prologue(int T, int Hq, int Hkv, int D, int R, int cs_dtype, int64_t q_head, int64_t k_head) {
+    if (T < 0 || Hq < 1 || Hkv < 1) return fail(DSA_ERR_ARG, "T=%d Hq=%d Hkv=%d", T, Hq, Hkv);
+    if (!(D == 64 || D == 128 || D == 256)) return fail(DSA_ERR_UNSUPPORTED, "head_dim=%d: need 64, 128 or 256", D);
+    if (R < 0 || R > D || R % 16) return fail(DSA_ERR_UNSUPPORTED, "rotary width R=%d: need a multiple of 16 up to head_dim=%d", R, D);
+    if (cs_dtype != DSA_DTYPE_BF16 && cs_dtype != DSA_DTYPE_FP32) return fail(DSA_ERR_ARG, "cos/sin dtype code %d", cs_dtype);
+    if (q_head % 8 || k_head % 8) return fail(DSA_ERR_ARG, "head strides must be multiples of 8 elements (16-byte rows)");
+    return DSA_OK;
+}
+
+extern "C" size_t dsa_qk_norm_rope_bwd_workspace_bytes(int T, int D) {
+    if (T <= 0 || D <= 0) return 0;
+    return (size_t)dsa_prologue_bwd_blocks(T) * 2 * D * sizeof(float);
+}
+
+extern "C" int dsa_qk_norm_rope_fwd(const void *q_in, int64_t q_tok, int64_t q_head, const void *k_in, int64_t k_tok,
+                                    int64_t k_head, const float *qw, const float *kw, float eps, int w_offset,
+                                    const void *cosp, const void *sinp, int cs_dtype, int R, int T, int Hq, int Hkv, int D,
+                                    void *q_out, void *k_out, float *q_rstd, float *k_rstd, void *stream) {
+    if (int rc = check_prologue(T, Hq, Hkv, D, R, cs_dtype, q_head, k_head)) return rc;
+    if (!q_in || !k_in || !qw || !kw || !q_out || !k_out || !q_rstd || !k_rstd || (R > 0 && (!cosp || !sinp)))
+        return fail(DSA_ERR_ARG, "null tensor pointer");
+    if (q_tok % 8 || k_tok % 8) return fail(DSA_ERR_ARG, "token strides must be multiples of 8 elements");
+    hipError_t e = dsa_launch_qk_norm_rope_fwd(q_in, q_tok, q_head, k_in, k_tok, k_head, qw, kw, eps, w_offset ? 1.f : 0.f,
+                                               cosp, sinp, cs_dtype == DSA_DTYPE_FP32, R, T, Hq, Hkv, D, q_out, k_out, q_rstd,
+                                               k_rstd, (hipStream_t)stream);
+    return e == hipSuccess ? DSA_OK : hip_fail(e, "qk_norm_rope forward launch");
+}
+
+extern "C" int dsa_qk_norm_rope_bwd(const void *gq, const void *gk, const void *q_in, int64_t q_tok, int64_t q_head,
+                                    const void *k_in, int64_t k_tok, int64_t k_head, const float *qw, const float *kw,
+                                    int w_offset, const void *cosp, const void *sinp, int cs_dtype, int R,
+                                    const float *q_rstd, const float *k_rstd, int T, int Hq, int Hkv, int D, void *dq_in,
+                                    int64_t dq_tok, int64_t dq_head, void *dk_in, int64_t dk_tok, int64_t dk_head,
+                                    float *dqw, float *dkw, void *ws, size_t ws_bytes, void *stream) {
+    if (int rc = check_prologue(T, Hq, Hkv, D, R, cs_dtype, q_head, k_head)) return rc;
+    if (!gq || !gk || !q_in || !k_in || !qw || !kw || !q_rstd || !k_rstd || !dq_in || !dk_in || !dqw || !dkw ||
+        (R > 0 && (!cosp || !sinp)))
+        return fail(DSA_ERR_ARG, "null tensor pointer");
+    if (q_tok % 8 || k_tok % 8 || dq_tok % 8 || dk_tok % 8 || dq_head % 8 || dk_head % 8)
+        return fail(DSA_ERR_ARG, "strides must be multiples of 8 elements");
+    const size_t need = dsa_qk_norm_rope_bwd_workspace_bytes(T, D);
+    if (need && (!ws || ws_bytes < need)) return fail(DSA_ERR_WORKSPACE, "prologue backward workspace: have %zu bytes, need %zu", ws_bytes, need);
+    hipError_t e = dsa_launch_qk_norm_rope_bwd(gq, gk, q_in, q_tok, q_head, k_in, k_tok, k_head, qw, kw, w_offset ? 1.f : 0.f,
+                                               cosp, sinp, cs_dtype == DSA_DTYPE_FP32, R, q_rstd, k_rstd, T, Hq, Hkv, D, dq_in,
+                                               dq_tok, dq_head, dk_in, dk_tok, dk_head, dqw, dkw, (float *)ws,
+                                               (hipStream_t)stream);
+    return e == hipSuccess ? DSA_OK : hip_fail(e, "qk_norm_rope backward launch");
+}
+
+extern "C" int dsa_sigmoid_gate_fwd(const void *x, const void *gate, int64_t gate_tok, int64_t gate_head, int T, int H, int D,
+                                    void *y, void *stream) {
+    if (T < 0 || H < 1 || D < 8 || D % 8 || gate_tok % 8 || gate_head % 8) return fail(DSA_ERR_ARG, "T=%d H=%d D=%d or strides not multiples of 8", T, H, D);
+    if (!x || !gate || !y) return fail(DSA_ERR_ARG, "null tensor pointer");
+    hipError_t e = dsa_launch_sigmoid_gate_fwd(x, gate, gate_tok, gate_head, D, H, T, y, (hipStream_t)stream);
+    return e == hipSuccess ? DSA_OK : hip_fail(e, "sigmoid gate forward launch");
+}
+
+extern "C" int dsa_sigmoid_gate_bwd(const void *gy, const void *x, const void *gate, int64_t gate_tok, int64_t gate_head,
+                                    int T, int H, int D, void *dx, void *dgate, int64_t dgate_tok, int64_t dgate_head,
+                                    void *stream) {
+    if (T < 0 || H < 1 || D < 8 || D % 8 || gate_tok % 8 || gate_head % 8 || dgate_tok % 8 || dgate_head % 8)
+        return fail(DSA_ERR_ARG, "T=%d H=%d D=%d or strides not multiples of 8", T, H, D);
+    if (!gy || !x || !gate || !dx || !dgate) return fail(DSA_ERR_ARG, "null tensor pointer");
+    hipError_t e = dsa_launch_sigmoid_gate_bwd(gy, x, gate, gate_tok, gate_head, D, H, T, dx, dgate, dgate_tok, dgate_head,
+                                               (hipStream_t)stream);
+    return e == hipSuccess ? DSA_OK : hip_fail(e, "sigmoid gate backward launch");
 }
