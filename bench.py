@@ -42,9 +42,9 @@ def cpu_baseline(w, threads):
     """Oracle (fp32 torch, CPU) fwd+bwd on one segment of the workload, scaled by causal pairs."""
     from oracle import dsa_ref as R
     from vlm_training_amd import workloads as W
-    # sample: the shortest segment that is longer than top_k (has both dense and sparse rows)
+    # sample: one long segment (rows below and above top_k), capped so that the default run stays short
     cands = [L for L in w.seg_lens if L > w.top_k] or [max(w.seg_lens)]
-    L = min(min(cands), 3072)
+    L = min(max(cands), 6144)           # about 10 s of host work at the headline geometry
     sw = W.scaled(w, (L,), name=w.name + "-cpu-sample")
     t = W.make_inputs(sw, device="cpu")
     torch.set_num_threads(threads)

@@ -398,3 +398,52 @@ def test_any_upper_bound_of_the_longest_segment_gives_the_same_result():
     for other in res[1:]:
         for a, b in zip(res[0], other):
             assert torch.equal(a, b)
+
+
+# ------------------------------------------------------------------------------------------ full size
+def test_headline_configuration_at_full_size_by_invariants():
+    """C3 as benchmarked (32768 packed tokens), checked by statements that hold at any size:
+    selections are ascending, causal, inside the query's segment and of size min(pos+1, K);
+    softmax rows sum to one (V = 1 gives out = 1, and sum_s dV[s] = sum_t dO[t] per kv head);
+    sum <dq, q> = sum <dk, k> per kv head (both equal sum dS.S); two runs are bit-identical."""
+    _log("C3 full size")
+    w = W.C3
+    t = W.make_inputs(w, device=DEV)
+    cu = t["cu_seqlens"]
+    G = w.Hq // w.Hkv
+
+    def run(vv):
+        q, k, v = (x.clone().requires_grad_(True) for x in (t["q"], t["k"], vv))
+        out, idx, n = ops.dsa_varlen_attn(q, k, v, cu, w.max_seqlen, indexer_q=t["q_idx"], indexer_k=t["k_idx"],
+                                          indexer_w=t["w_idx"], top_k=w.top_k, return_indices=True)
+        out.backward(t["dout"])
+        return out.detach(), idx, n, q.grad, k.grad, v.grad
+
+    out, idx, n, dq, dk, dv = run(t["v"])
+    torch.cuda.synchronize()
+    # selection
+    pos = torch.cat([torch.arange(L, device=DEV) for L in w.seg_lens])
+    seg0 = torch.cat([torch.full((L,), a, device=DEV) for a, L in zip(w.cu[:-1], w.seg_lens)])
+    assert torch.equal(n.long(), torch.clamp(pos + 1, max=w.top_k))
+    col = torch.arange(w.top_k, device=DEV)[None, :]
+    valid = col < n[:, None]
+    assert bool(((idx == -1) | valid).all()) and bool((idx[valid] >= 0).all())
+    assert bool((idx >= seg0[:, None])[valid].all()) and bool((idx <= (seg0 + pos)[:, None])[valid].all())
+    inc = (idx[:, 1:] > idx[:, :-1]) | ~valid[:, 1:]
+    assert bool(inc.all())
+    # finiteness and the <dq,q> = <dk,k> identity per kv head
+    for x in (out, dq, dk, dv):
+        assert bool(torch.isfinite(x).all())
+    a = (dq.float() * t["q"].float()).sum(dim=(0, 2)).view(w.Hkv, G).sum(1)
+    b = (dk.float() * t["k"].float()).sum(dim=(0, 2))
+    assert torch.allclose(a, b, rtol=2e-2, atol=2e-2 * float(a.abs().max())), (a, b)
+    # rows of P sum to one
+    want = t["dout"].float().sum(0).view(w.Hkv, G, w.D).sum(1)
+    got = dv.float().sum(0)
+    assert torch.allclose(got, want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+    out1 = run(torch.ones_like(t["v"]))[0]
+    assert float((out1.float() - 1).abs().max()) <= 2 ** -7
+    # determinism
+    again = run(t["v"])
+    for x, y in zip((out, idx, n, dq, dk, dv), again):
+        assert torch.equal(x, y)
