@@ -12,11 +12,18 @@
 // than top-k are skipped altogether.
 #include "dsa_common.h"
 
+__device__ __forceinline__ f32x16 zero_acc() {
+    f32x16 z;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) z[v] = 0.f;
+    return z;
+}
+
 #define IDX_WAVES 4
 #define IDX_BK 64
 
 template <int HT, int DI>
-__global__ __launch_bounds__(IDX_WAVES * 64) void dsa_indexer_scores_kernel(
+__global__ __launch_bounds__(IDX_WAVES * 64, 2) void dsa_indexer_scores_kernel(
     const bf16_t *__restrict__ q_idx, const bf16_t *__restrict__ k_idx, const bf16_t *__restrict__ w_idx,
     const int32_t *__restrict__ cu, int N, int T, int Hi, float scale, int row_begin, int row_end, int skip_dense_k,
     float *__restrict__ scores, int64_t ld) {
@@ -92,30 +99,59 @@ __global__ __launch_bounds__(IDX_WAVES * 64) void dsa_indexer_scores_kernel(
         if (it + 1 < ntiles) load_tile(kt + IDX_BK);
         const unsigned char *buf = lds[it & 1];
         if (active) {
+            // key operands of sub-tile `sub` (32 keys): all KS reads issued together
+            auto read_b = [&](int sub, bf16x8 (&b)[KS]) {
 #pragma unroll
-            for (int sub = 0; sub < IDX_BK / 32; ++sub) {
-                const int kb = kt + sub * 32;
-                if (kb > t || kb + 31 < s0) continue;        // wave-uniform
-                f32x16 acc[HT];
+                for (int ks = 0; ks < KS; ++ks)
+                    b[ks] = *reinterpret_cast<const bf16x8 *>(buf + (sub * 32 + (lane & 31)) * ROW_B + (ks * 16 + (lane >> 5) * 8) * 2);
+            };
+            auto gemm = [&](const bf16x8 (&b)[KS], f32x16 (&acc)[HT]) {
 #pragma unroll
-                for (int ht = 0; ht < HT; ++ht)
+                for (int ht = 0; ht < HT; ++ht) acc[ht] = zero_acc();
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[ht][v] = 0.f;
+                for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    const bf16x8 b = *reinterpret_cast<const bf16x8 *>(
-                        buf + (sub * 32 + (lane & 31)) * ROW_B + (ks * 16 + (lane >> 5) * 8) * 2);
-#pragma unroll
-                    for (int ht = 0; ht < HT; ++ht) acc[ht] = mfma32(a[ht][ks], b, acc[ht]);
-                }
+                    for (int ht = 0; ht < HT; ++ht) acc[ht] = mfma32(a[ht][ks], b[ks], acc[ht]);
+            };
+            // ReLU (one integer max on the bit pattern: negative floats are negative integers; fmaxf would
+            // cost a second instruction to quiet NaNs), head weights, sum over heads, store
+            auto epilogue = [&](int kb, const f32x16 (&acc)[HT]) {
                 float sum = 0.f;
 #pragma unroll
                 for (int ht = 0; ht < HT; ++ht)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) sum += wreg[ht][v] * fmaxf(acc[ht][v], 0.f);
+                    for (int v = 0; v < 16; ++v) sum += wreg[ht][v] * __int_as_float(max(__float_as_int(acc[ht][v]), 0));
                 sum += wave_xor_f(sum, 32);
                 const int s = kb + (lane & 31);
                 if (lane < 32 && s >= s0 && s <= t) orow[s - s0] = sum * scale;
+            };
+            const bool on0 = !(kt > t || kt + 31 < s0), on1 = !(kt + 32 > t || kt + 63 < s0);   // wave-uniform
+            if (on0 && on1) {
+                // both halves of the tile: the second GEMM is issued between the first half's epilogue
+                bf16x8 b0[KS], b1[KS];
+                f32x16 acc0[HT], acc1[HT];
+                read_b(0, b0);
+                read_b(1, b1);
+                gemm(b0, acc0);
+                gemm(b1, acc1);
+                epilogue(kt, acc0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2 * KS, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, KS * HT, 0);
+#pragma unroll
+                for (int i = 0; i < KS * HT; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, (32 * HT * 2 + KS * HT - 1) / (KS * HT), 0);
+                }
+                epilogue(kt + 32, acc1);
+            } else if (on0 || on1) {
+                const int sub = on0 ? 0 : 1;
+                bf16x8 b[KS];
+                f32x16 acc[HT];
+                read_b(sub, b);
+                gemm(b, acc);
+                __builtin_amdgcn_sched_group_barrier(0x100, KS, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, KS * HT, 0);
+                epilogue(kt + 32 * sub, acc);
             }
         }
         if (it + 1 < ntiles) store_tile((it + 1) & 1);
