@@ -109,8 +109,6 @@ __device__ __forceinline__ f32x16 zero16() {
     for (int v = 0; v < 16; ++v) z[v] = 0.f;
     return z;
 }
-// key / row index inside a 32-tile held by accumulator element v of lane half h (C layout of mfma32)
-__device__ __forceinline__ int c_row(int v, int h) { return 8 * (v >> 2) + 4 * h + (v & 3); }
 
 // slot -> (segment, block) for blocks of `blk` columns handed out segment by segment; within a segment
 // the blocks are numbered from the end when `reverse` (heaviest causal blocks first).  Returns false
@@ -400,186 +398,43 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
 }
 
 // ==================================================================================================
-// dK, dV: key-stationary ("scatter by key": every key row is reduced by exactly one wave, in query
-// order, so the result needs no atomics and is bit-reproducible).  Workgroup = 4 waves x 32 keys = one
-// 128-key tile of a segment and one kv head; walks the queries from the tile's first column to the end
-// of the segment in blocks of 32 (query, head) rows staged in LDS (same two-ahead pipeline).
-//   S[row,key] = Q K^T, dP = dO V^T     (A = q / dO block row-wise, B = K^T / V^T in registers)
-//   dV^T[d,key] += dO^T[d,row] P[row,key]   dK^T[d,key] += Q^T[d,row] dS[row,key]
-//                                           (A = dO / q block transposed, B = P / dS from the C layout)
-// ==================================================================================================
-template <int D, bool HAS_IDX, int GSHIFT>
-__global__ __launch_bounds__(256) void dsa_tile_dkv_kernel(
-    const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
-    const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
-    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
-    float scale, int causal, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
-    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / 256;
-    constexpr int NBUF = (D > 128) ? 1 : 2;
-    constexpr int Gp = 1 << GSHIFT, QB = 32 >> GSHIFT;                           // queries per block
-    __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];   // [buffer][q|dO]
-    __shared__ __attribute__((aligned(16))) float lse_s[NBUF][32], dlt_s[NBUF][32];
-    __shared__ uint32_t mask_s[NBUF][4][32];                                      // [buffer][wave][query in block]
-
-    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
-    LaneOffsets<D> lo;
-    lo.init(lane);
-    const int G = Hq / Hkv;
-    const int kvh = blockIdx.x % Hkv;
-    int s0, L, blk;
-    if (!locate_block(cu, N, blockIdx.x / Hkv, 128, false, s0, L, blk)) return;
-    const int c0 = blk * 128, kc = c0 + wv * 32;
-    const int mykey = kc + j;
-    const bool key_ok = mykey < L;
-    const int64_t krow = (int64_t)(s0 + min(mykey, L - 1)) * Hkv + kvh;
-    bf16x8 kB[KS], vB[KS];
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        kB[ks] = load_bf16x8(k + krow * D + 16 * ks + 8 * h);
-        vB[ks] = load_bf16x8(v + krow * D + 16 * ks + 8 * h);
-    }
-    f32x16 dkacc[DT], dvacc[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) { dkacc[dt] = zero16(); dvacc[dt] = zero16(); }
-    const float scale_log2 = scale * LOG2E_F;
-    const int q0 = causal ? c0 : 0;                      // first query column that can see this key tile
-    const int nblocks = (L - q0 + QB - 1) / QB;          // queries q0 .. L-1
-
-    u32x4 qst[2][LOADS], dost[2][LOADS];
-    // Per-block side data, one 32-bit word per staging thread, loaded raw and interpreted at STORE time:
-    //   tid 0..31: lse of row tid;  32..63: delta of row tid-32;  64..64+4*QB-1: selection word of
-    //   (key group w, query qi);  the rest re-read a valid word and drop it.
-    const uint32_t *aux_base;
-    int aux_q = 0, aux_stride = 1;                       // word index = aux_stride * min(block start + aux_q, L-1)
-    bool aux_mask_ok = false;
-    if (tid < 64) {
-        const int row = tid & 31;
-        const int hd = min(row & (Gp - 1), G - 1);
-        aux_q = row >> GSHIFT;
-        aux_base = reinterpret_cast<const uint32_t *>((tid < 32 ? lse : delta) + (int64_t)(kvh * G + hd) * T + s0);
-    } else if (HAS_IDX && tid < 64 + 4 * QB) {
-        const int w = (tid - 64) / QB;
-        aux_q = (tid - 64) % QB;
-        aux_stride = ldw;
-        aux_mask_ok = (c0 >> 5) + w < ldw;
-        aux_base = bitmap + (int64_t)s0 * ldw + (aux_mask_ok ? (c0 >> 5) + w : 0);
-    } else {
-        aux_base = reinterpret_cast<const uint32_t *>(lse);
-    }
-    uint32_t aux_st[2] = {0u, 0u};
-#define DKV_LOAD(SET, BLK)                                                                          \
-    {                                                                                              \
-        const int qcb = q0 + (BLK) * QB;                                                           \
-        _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                        \
-            const int c = i * 256 + tid;                                                           \
-            const int row = c / CPR, ch = c % CPR;                                                 \
-            const int qc = min(qcb + (row >> GSHIFT), L - 1);                                      \
-            const int hd = min(row & (Gp - 1), G - 1);                                             \
-            const int64_t off = ((int64_t)(s0 + qc) * Hq + kvh * G + hd) * D + ch * 8;             \
-            qst[SET][i] = *reinterpret_cast<const u32x4 *>(q + off);                               \
-            dost[SET][i] = *reinterpret_cast<const u32x4 *>(dout + off);                           \
-        }                                                                                          \
-        aux_st[SET] = aux_base[(int64_t)aux_stride * min(qcb + aux_q, L - 1)];                     \
-    }
-#define DKV_STORE(SET, BUF, BLK)                                                                    \
-    {                                                                                              \
-        const int qcb = q0 + (BLK) * QB;                                                           \
-        const u32x4 z4 = {0u, 0u, 0u, 0u};                                                         \
-        _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                        \
-            const int c = i * 256 + tid;                                                           \
-            const int row = c / CPR, ch = c % CPR;                                                 \
-            /* rows past the segment and padded heads are zeroed: they add nothing to dK, dV */     \
-            const bool live = qcb + (row >> GSHIFT) < L && (row & (Gp - 1)) < G;                   \
-            *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(row, ch)]) = live ? qst[SET][i] : z4;  \
-            *reinterpret_cast<u32x4 *>(&lds[BUF][1][tile_off<D>(row, ch)]) = live ? dost[SET][i] : z4; \
-        }                                                                                          \
-        if (tid < 32) lse_s[BUF][tid] = __uint_as_float(aux_st[SET]) * LOG2E_F;                    \
-        else if (tid < 64) dlt_s[BUF][tid - 32] = __uint_as_float(aux_st[SET]);                    \
-        else if (HAS_IDX && tid < 64 + 4 * QB)                                                     \
-            mask_s[BUF][(tid - 64) / QB][(tid - 64) % QB] = (aux_mask_ok && qcb + aux_q < L) ? aux_st[SET] : 0u; \
-    }
-#define DKV_COMPUTE(BLK, BUF)                                                                       \
-    {                                                                                              \
-        const int qcb = q0 + (BLK) * QB;                                                           \
-        const unsigned char *qt = lds[BUF][0], *dot = lds[BUF][1];                                 \
-        f32x16 sacc = zero16(), pacc = zero16();                                                   \
-        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
-            sacc = mfma32(lo.rowop(qt, ks), kB[ks], sacc);                              \
-            pacc = mfma32(lo.rowop(dot, ks), vB[ks], pacc);                             \
-        }                                                                                          \
-        float pv[16], dsv[16];                                                                     \
-        const bool diag = causal && qcb < kc + 32;      /* wave-uniform: block touches the diagonal */ \
-        _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {                                         \
-            const f32x4 l4 = *reinterpret_cast<const f32x4 *>(&lse_s[BUF][8 * g4 + 4 * h]);        \
-            const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&dlt_s[BUF][8 * g4 + 4 * h]);        \
-            uint32_t keep = 0u;                                                                    \
-            _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                        \
-                const int vi = 4 * g4 + e, row = 8 * g4 + 4 * h + e;                               \
-                if (e == 0 || GSHIFT < 2) {              /* rows of one query share the mask bit */  \
-                    const int qi = row >> GSHIFT;                                                  \
-                    uint32_t mw = HAS_IDX ? mask_s[BUF][wv][qi] : 0xffffffffu;                     \
-                    if (diag) mw &= causal_bits(qcb + qi - kc);                                    \
-                    keep = bit_mask(mw, j);                                                        \
-                }                                                                                  \
-                const float p = fast_exp2(keep_or_neginf(fmaf(sacc[vi], scale_log2, -l4[e]), keep)); \
-                pv[vi] = p;                                                                        \
-                dsv[vi] = p * (pacc[vi] - d4[e]);                                                  \
-            }                                                                                      \
-        }                                                                                          \
-        const bf16x8 pB0 = pack8(pv), pB1 = pack8(pv + 8), dB0 = pack8(dsv), dB1 = pack8(dsv + 8); \
-        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
-            mfma32_acc(dvacc[dt], lo.trop(dot, 0, dt), pB0);                        \
-            mfma32_acc(dvacc[dt], lo.trop(dot, 1, dt), pB1);                   \
-            mfma32_acc(dkacc[dt], lo.trop(qt, 0, dt), dB0);                         \
-            mfma32_acc(dkacc[dt], lo.trop(qt, 1, dt), dB1);                    \
-        }                                                                                          \
-    }
-    TILE_PIPELINE(nblocks, DKV_LOAD, DKV_STORE, DKV_COMPUTE)
-#undef DKV_LOAD
-#undef DKV_STORE
-#undef DKV_COMPUTE
-
-    if (key_ok) {
-        bf16_t *pk = dk + krow * D + 4 * h, *pv_ = dv + krow * D + 4 * h;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                const u32x2 wk = {pack2bf(dkacc[dt][4 * g4] * scale, dkacc[dt][4 * g4 + 1] * scale),
-                                  pack2bf(dkacc[dt][4 * g4 + 2] * scale, dkacc[dt][4 * g4 + 3] * scale)};
-                const u32x2 wvv = {pack2bf(dvacc[dt][4 * g4], dvacc[dt][4 * g4 + 1]),
-                                   pack2bf(dvacc[dt][4 * g4 + 2], dvacc[dt][4 * g4 + 3])};
-                *reinterpret_cast<u32x2 *>(pk + dt * 32 + 8 * g4) = wk;
-                *reinterpret_cast<u32x2 *>(pv_ + dt * 32 + 8 * g4) = wvv;
-            }
-    }
-}
-
-// ==================================================================================================
-// dK, dV for head_dim <= 128, producer/consumer form.  A workgroup owns a 128-key tile (4 groups of 32
-// keys) of one segment and kv head and walks the later queries in blocks of 32 (query, head) rows,
-// from the end of the segment down to the key tile: workgroups that run side by side then read the
-// same q / dO rows at about the same time and share them in L2.
+// dK, dV, producer/consumer form, key-stationary ("scatter by key": every key row is reduced by exactly
+// one wave, in a fixed query order, so the result needs no atomics and is bit-reproducible).  A
+// workgroup owns a 128-key tile (4 groups of 32 keys) of one segment and kv head and walks the later
+// queries in blocks of 32 (query, head) rows, from the end of the segment down to the key tile:
+// workgroups that run side by side then read the same q / dO rows at about the same time and share
+// them in L2.
 //   waves 0-3 (producers, one per key group): S = Q K^T and dP = dO V^T against the group's K / V rows
 //     held in registers, then P and dS = P * (dP - delta) in bf16, written to LDS in MFMA B layout.
 //     The two GEMMs of block b+1 are issued between the softmax arithmetic of block b: a SIMD overlaps
 //     matrix and vector instructions of one instruction stream far better than those of two waves.
 //   waves 4-7 (consumers, one per key group): dV^T += dO^T P and dK^T += Q^T dS for block b-1,
 //     A operands read transposed from the staged q / dO block, B operands read back from LDS.  They
-//     also do all the staging (global -> registers one block ahead -> LDS), so the producers' stream
+//     also do all the staging (global -> registers two blocks ahead -> LDS), so the producers' stream
 //     holds nothing but the GEMMs and the softmax.
 // Nothing is computed twice (32 MFMAs per 32x32 block pair), each wave stays under 256 registers.
 // LDS (dynamic, ~115 KiB): q/dO blocks in a ring of four (b+2 being staged, b+1 read row-wise by the
 // producers, b-1 read transposed by the consumers), P/dS in a ring of two, row statistics and
 // selection words in a ring of four.  One barrier per block.
+// head_dim 256: the K and V rows of a producer fill 128 registers and a consumer's accumulators would
+// fill 256, so the kernel is launched once per half of head_dim (`dhalf`: the consumers accumulate and
+// write that half, the producers repeat S and dP), the q/dO ring has three slots (~145 KiB) and the
+// producers run GEMMs and softmax of a block in turn.
 // ==================================================================================================
 template <int D, bool HAS_IDX, int GSHIFT>
 __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
-    float scale, int causal, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    float scale, int causal, int dhalf, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>();
+    // head_dim 256: a consumer's accumulators cover one half of head_dim per launch (`dhalf`), the
+    // q/dO ring holds three blocks instead of four and the producers run GEMMs and softmax of one block
+    // in turn (the ring has no room for the block a pipelined producer would read ahead)
+    constexpr bool PIPE = D <= 128;
+    constexpr int NQD = PIPE ? 4 : 3, LEAD = PIPE ? 2 : 1;
+    constexpr int DTC = DT > 4 ? 4 : DT;
+    const int dt0 = dhalf * DTC;
     constexpr int NCHUNK = 32 * CPR;                     // 16-byte chunks per staged operand
     constexpr int CPT = NCHUNK / 256;                    // chunks per consumer thread and operand
     constexpr int Gp = 1 << GSHIFT, QB = 32 >> GSHIFT;
@@ -588,9 +443,10 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     constexpr int AUX_SLOT = (32 + 32 + 4 * 32) * 4;     // lse | delta | selection words [key group][query]
     static_assert(CPT >= 1 && NCHUNK % 256 == 0, "every consumer thread stages whole chunks");
     extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
-    unsigned char *const qd_ring = dyn_lds;                          // 4 slots
-    unsigned char *const pd_ring = dyn_lds + 4 * QD_SLOT;            // 2 slots
-    unsigned char *const aux_ring = pd_ring + 2 * PD_SLOT;           // 4 slots
+    unsigned char *const qd_ring = dyn_lds;                          // NQD slots
+    unsigned char *const pd_ring = dyn_lds + NQD * QD_SLOT;          // 2 slots
+    unsigned char *const aux_ring = pd_ring + 2 * PD_SLOT;           // NQD slots
+    auto qslot = [](int b) { return PIPE ? (b & 3) : (b % 3); };
 
     const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5, j = lane & 31;
     LaneOffsets<D> lo;
@@ -682,8 +538,8 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
             aux_st = *reinterpret_cast<const uint32_t *>(ap);
         };
         auto lstore = [&](int b, const u32x4 (&qst)[CPT], const u32x4 (&dost)[CPT], uint32_t aux_st) {   // step b -> ring slot b % 4
-            unsigned char *slot = qd_ring + (b & 3) * QD_SLOT;
-            float *lse_s = reinterpret_cast<float *>(aux_ring + (b & 3) * AUX_SLOT);
+            unsigned char *slot = qd_ring + qslot(b) * QD_SLOT;
+            float *lse_s = reinterpret_cast<float *>(aux_ring + qslot(b) * AUX_SLOT);
             float *dlt_s = lse_s + 32;
             uint32_t *mask_s = reinterpret_cast<uint32_t *>(dlt_s + 32);
             // rows past the segment (last block only) and padded heads are zeroed: they add nothing to dK, dV
@@ -706,27 +562,34 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
                 mask_s[((ctid - 64) / QB) * 32 + (ctid - 64) % QB] =
                     (aux_mask_ok && !(b > last || (b == 0 && aux_over > 0))) ? aux_st : 0u;
         };
-        gload(0, qst0, dost0, aux_st0);
-        gload(1, qst1, dost1, aux_st1);
-        lstore(0, qst0, dost0, aux_st0);
-        lstore(1, qst1, dost1, aux_st1);
-        gload(2, qst0, dost0, aux_st0);
-        gload(3, qst1, dost1, aux_st1);
-        __syncthreads();                                 // steps 0 and 1 staged
+        if (PIPE) {
+            gload(0, qst0, dost0, aux_st0);
+            gload(1, qst1, dost1, aux_st1);
+            lstore(0, qst0, dost0, aux_st0);
+            lstore(1, qst1, dost1, aux_st1);
+            gload(2, qst0, dost0, aux_st0);
+            gload(3, qst1, dost1, aux_st1);
+        } else {                                         // head_dim 256: one register set (four chunks per operand and thread)
+            gload(0, qst0, dost0, aux_st0);
+            lstore(0, qst0, dost0, aux_st0);
+            gload(1, qst0, dost0, aux_st0);
+        }
+        __syncthreads();                                 // the first LEAD steps staged
 
-        f32x16 dkacc[DT], dvacc[DT];
+        f32x16 dkacc[DTC], dvacc[DTC];
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) { dkacc[dt] = zero16(); dvacc[dt] = zero16(); }
-        // one consumer step: stage step B+2 from the given register set, refill it with step B+4, then the MFMAs of step B-1
+        for (int dt = 0; dt < DTC; ++dt) { dkacc[dt] = zero16(); dvacc[dt] = zero16(); }
+        // one consumer step: stage step B+LEAD from the register set that holds it, refill the set (two sets:
+        // with step B+LEAD+2, one set: with step B+LEAD+1), then the MFMAs of step B-1
 #define DKV_CONSUMER_STEP(B, QS, DS, AS)                                                            \
     {                                                                                              \
-        lstore((B) + 2, QS, DS, AS);    /* slot (B+2)%4 was last read (as step B-2) before the previous barrier */ \
-        gload((B) + 4, QS, DS, AS);                                                                \
+        lstore((B) + LEAD, QS, DS, AS); /* its slot was last read (as step B+LEAD-NQD) before the previous barrier */ \
+        gload((B) + LEAD + (PIPE ? 2 : 1), QS, DS, AS);                                            \
         if ((B) >= 1) consume((B) - 1);                                                            \
         __syncthreads();                                                                           \
     }
         auto consume = [&](int b) {
-            const unsigned char *qt = qd_ring + (b & 3) * QD_SLOT;
+            const unsigned char *qt = qd_ring + qslot(b) * QD_SLOT + dt0 * 64;
             lds_u8 *pt[4];                  // lane addresses in the q block; the dO block sits TILE_B behind
 #pragma unroll
             for (int vv = 0; vv < 4; ++vv) {
@@ -737,25 +600,29 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
             const bf16x8 pB0 = *reinterpret_cast<const bf16x8 *>(pd), pB1 = *reinterpret_cast<const bf16x8 *>(pd + 1024);
             const bf16x8 dB0 = *reinterpret_cast<const bf16x8 *>(pd + 2048), dB1 = *reinterpret_cast<const bf16x8 *>(pd + 3072);
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
+            for (int dt = 0; dt < DTC; ++dt) {
                 dvacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 0, dt, TILE_B), pB0, dvacc[dt]);
                 dkacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 0, dt, 0), dB0, dkacc[dt]);
                 dvacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 1, dt, TILE_B), pB1, dvacc[dt]);
                 dkacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 1, dt, 0), dB1, dkacc[dt]);
             }
-            sched_reads_ahead<4 * DT, 3, 2, 4>();
+            sched_reads_ahead<4 * DTC, 3, 2, 4>();
         };
         int b = 0;
-        for (; b + 1 <= nblocks; b += 2) {
-            DKV_CONSUMER_STEP(b, qst0, dost0, aux_st0)
-            DKV_CONSUMER_STEP(b + 1, qst1, dost1, aux_st1)
+        if (PIPE) {                                      // step b + 2 sits in set b % 2
+            for (; b + 1 <= nblocks; b += 2) {
+                DKV_CONSUMER_STEP(b, qst0, dost0, aux_st0)
+                DKV_CONSUMER_STEP(b + 1, qst1, dost1, aux_st1)
+            }
+            if (b <= nblocks) DKV_CONSUMER_STEP(b, qst0, dost0, aux_st0)
+        } else {
+            for (; b <= nblocks; ++b) DKV_CONSUMER_STEP(b, qst0, dost0, aux_st0)
         }
-        if (b <= nblocks) DKV_CONSUMER_STEP(b, qst0, dost0, aux_st0)
 #undef DKV_CONSUMER_STEP
         if (key_ok) {
-            bf16_t *pk = dk + krow * D + 4 * h, *pv_ = dv + krow * D + 4 * h;
+            bf16_t *pk = dk + krow * D + dt0 * 32 + 4 * h, *pv_ = dv + krow * D + dt0 * 32 + 4 * h;
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
+            for (int dt = 0; dt < DTC; ++dt)
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4) {
                     const u32x2 wk = {pack2bf(dkacc[dt][4 * g4] * scale, dkacc[dt][4 * g4 + 1] * scale),
@@ -780,7 +647,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     f32x4 l4[4], d4[4];
     uint32_t mw[16];
     auto read_aux = [&](int b) {
-        const float *lse_s = reinterpret_cast<const float *>(aux_ring + (b & 3) * AUX_SLOT);
+        const float *lse_s = reinterpret_cast<const float *>(aux_ring + qslot(b) * AUX_SLOT);
         const float *dlt_s = lse_s + 32;
         const uint32_t *mask_s = reinterpret_cast<const uint32_t *>(dlt_s + 32) + kg * 32;
 #pragma unroll
@@ -793,7 +660,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
         }
     };
     auto gemms = [&](int b, f32x16 &sacc, f32x16 &pacc) {            // S and dP of block b
-        const unsigned char *qt = qd_ring + (b & 3) * QD_SLOT, *dot = qt + TILE_B;
+        const unsigned char *qt = qd_ring + qslot(b) * QD_SLOT, *dot = qt + TILE_B;
         sacc = zero16();
         pacc = zero16();
 #pragma unroll
@@ -837,7 +704,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     // MFMA's operand and the scale used by the next step's arithmetic pass through.
     auto fused = [&](auto may_diag, int b, const f32x16 &sc, const f32x16 &pc, f32x16 &sn, f32x16 &pn) {
         constexpr int NM = 2 * KS, EPM = 16 / NM;
-        const unsigned char *qt = qd_ring + ((b + 1) & 3) * QD_SLOT, *dot = qt + TILE_B;
+        const unsigned char *qt = qd_ring + qslot(b + 1) * QD_SLOT, *dot = qt + TILE_B;
         float pv[16], dsv[16], sl2 = scale_log2;
         uint32_t keep = 0u;
         bf16x8 a[4];
@@ -870,13 +737,51 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
         __syncthreads();                                                                           \
     }
     f32x16 s_a, p_a, s_b, p_b;
-    __syncthreads();                                     // blocks 0 and 1 staged
+    __syncthreads();                                     // the first LEAD steps staged
+    const std::true_type diag_y;
+    const std::false_type diag_n;
+    if (!PIPE) {
+        // GEMMs, then softmax, block by block (the row statistics of a block are staged one step before)
+        for (int b = 0; b <= nblocks; ++b) {
+            if (b < nblocks) {
+                gemms(b, s_a, p_a);
+                // softmax with the row statistics taken from LDS group by group (K and V rows of head_dim 256
+                // leave no registers to hold them across the GEMMs)
+                const float *lse_s = reinterpret_cast<const float *>(aux_ring + qslot(b) * AUX_SLOT);
+                const float *dlt_s = lse_s + 32;
+                const uint32_t *mask_s = reinterpret_cast<const uint32_t *>(dlt_s + 32) + kg * 32;
+                const int qcb = q0 + (nblocks - 1 - b) * QB;
+                const bool diag = causal && qcb < kc + 32;
+                float pv[16], dsv[16];
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const f32x4 l4g = *reinterpret_cast<const f32x4 *>(&lse_s[8 * g4 + 4 * h]);
+                    const f32x4 d4g = *reinterpret_cast<const f32x4 *>(&dlt_s[8 * g4 + 4 * h]);
+                    uint32_t keep = 0u;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int vi = 4 * g4 + e, row = 8 * g4 + 4 * h + e;
+                        if (e == 0 || GSHIFT < 2) {
+                            const int qi = row >> GSHIFT;
+                            uint32_t w = HAS_IDX ? mask_s[qi] : 0xffffffffu;
+                            if (diag) w &= causal_bits(qcb + qi - kc);
+                            keep = bit_mask(w, j);
+                        }
+                        const float p = fast_exp2(keep_or_neginf(fmaf(s_a[vi], scale_log2, -l4g[e]), keep));
+                        pv[vi] = p;
+                        dsv[vi] = p * (p_a[vi] - d4g[e]);
+                    }
+                }
+                store_pd(b, pv, dsv);
+            }
+            __syncthreads();
+        }
+        return;
+    }
     gemms(0, s_a, p_a);
     read_aux(0);
     // The blocks that can touch the causal diagonal come last; the steady loop before them has no mask
     // arithmetic besides the selection bits and is one basic block.
-    const std::true_type diag_y;
-    const std::false_type diag_n;
     const int nb_diag = causal ? (kc + 32 - q0 + QB - 1) / QB : 0;
     const int steady = max(nblocks - nb_diag, 0) & ~1;   // steps [0, steady) see blocks fully past the diagonal
     int b = 0;
@@ -892,7 +797,9 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
 #undef DKV_PRODUCER_STEP
 }
 template <int D>
-constexpr size_t dkvpc_lds_bytes() { return 4 * (2 * tile_bytes<D>()) + 2 * (4 * 4 * 1024) + 4 * ((32 + 32 + 4 * 32) * 4); }
+constexpr size_t dkvpc_lds_bytes() {
+    return (D <= 128 ? 4 : 3) * ((size_t)2 * tile_bytes<D>() + (32 + 32 + 4 * 32) * 4) + 2 * (4 * 4 * 1024);
+}
 
 // ==================================================================================================
 // launchers: instantiate per head_dim, mask kind and (power-of-two padded) group size
@@ -923,21 +830,17 @@ template <int D, bool HAS_IDX, int GS>
 static void launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
                          const float *lse, const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N,
                          int T, int Hq, int Hkv, float scale, int causal, void *dk, void *dv) {
-    if constexpr (D <= 128) {
-        static bool configured = false;                  // LDS above 64 KiB has to be requested once per kernel
-        if (!configured) {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkvpc_lds_bytes<D>());
-            configured = true;
-        }
+    static bool configured = false;                      // LDS above 64 KiB has to be requested once per kernel
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkvpc_lds_bytes<D>());
+        configured = true;
+    }
+    // head_dim 256: one launch per half of head_dim (a consumer wave holds 128 accumulator registers)
+    for (int dhalf = 0; dhalf < (D > 128 ? 2 : 1); ++dhalf)
         hipLaunchKernelGGL((dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>), grid, dim3(512), dkvpc_lds_bytes<D>(), stream,
                            (const bf16_t *)dout, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap,
-                           ldw, cu, N, T, Hq, Hkv, scale, causal, (bf16_t *)dk, (bf16_t *)dv);
-    }
-    else
-        hipLaunchKernelGGL((dsa_tile_dkv_kernel<D, HAS_IDX, GS>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
-                           (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T, Hq,
-                           Hkv, scale, causal, (bf16_t *)dk, (bf16_t *)dv);
+                           ldw, cu, N, T, Hq, Hkv, scale, causal, dhalf, (bf16_t *)dk, (bf16_t *)dv);
 }
 
 #define GS_SWITCH(FN, DD, HI, ...)                                    \
