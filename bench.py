@@ -207,7 +207,11 @@ def main():
                      "algorithmic_flop": dom_flop, "avg_ms": stage_ms[dom]},
         "stage_ms": stage_ms,
         "roofline_whole_op": {"t_roof_ms": t_roof_ms, "sum_ms": roof_total, "frac": roof_total / ms_per_step,
-                              "compute_only_bound_ms": (wk["F1"] + 3.5 * wk["F3"]) / (PEAK_MFMA_BF16_TFLOPS * 1e12) * 1e3},
+                              "compute_only_bound_ms": (wk["F1"] + 3.5 * wk["F3"]) / (PEAK_MFMA_BF16_TFLOPS * 1e12) * 1e3,
+                              "note": "t_roof_ms prices the attention stages by the bytes a row gather of the selected keys "
+                                      "would move (the nominal roofline the target was derived from); the tile kernels "
+                                      "do not gather, so frac > 1 means that bound was left behind - roofline.frac is the "
+                                      "figure of merit of the dominant kernel"},
         "device": torch.cuda.get_device_name(0),
     }
     result["adjacent_kernels"] = prologue_stage(w, dev, it)
