@@ -100,6 +100,29 @@ def prologue_stage(w, dev, iters):
     return res
 
 
+def reference_operator(w, t, iters):
+    """The reference's own operator on the same GPU and batch: torch.nn.attention.varlen.varlen_attn (dense
+    causal, what train/model_attention.py:123-132 calls) against this library's dense path (no indexer)."""
+    from vlm_training_amd import ops
+    try:
+        from torch.nn.attention.varlen import varlen_attn as torch_varlen_attn
+    except Exception as e:
+        return {"error": repr(e)[:200]}
+    cu, msl = t["cu_seqlens"], w.max_seqlen
+
+    def run(fn):
+        q, k, v = (t[x].detach().requires_grad_(True) for x in ("q", "k", "v"))
+        fn(q, k, v).backward(t["dout"])
+
+    try:
+        theirs = timed(lambda: run(lambda q, k, v: torch_varlen_attn(q, k, v, cu, cu, msl, msl, is_causal=True)), iters)
+    except Exception as e:
+        return {"error": repr(e)[:200]}
+    ours = timed(lambda: run(lambda q, k, v: ops.dsa_varlen_attn(q, k, v, cu, msl)), iters)
+    return {"what": "dense causal packed attention fwd+bwd on this workload (the operator the reference calls)",
+            "torch_varlen_attn_ms": theirs, "this_library_dense_ms": ours, "speedup": theirs / ours}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -215,6 +238,7 @@ def main():
         "device": torch.cuda.get_device_name(0),
     }
     result["adjacent_kernels"] = prologue_stage(w, dev, it)
+    result["reference_operator"] = reference_operator(w, t, it)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, torch.get_num_threads())
     print(json.dumps(result))

@@ -447,3 +447,34 @@ def test_headline_configuration_at_full_size_by_invariants():
     again = run(t["v"])
     for x, y in zip((out, idx, n, dq, dk, dv), again):
         assert torch.equal(x, y)
+
+
+# ------------------------------------------------------------------------------------------ the torch routine itself
+def test_dense_path_against_torch_varlen_attn_on_the_gpu():
+    """The routine the reference calls (train/model_attention.py:123-132: torch.nn.attention.varlen.varlen_attn,
+    here in the torch 2.10 ``is_causal`` form) runs on the GPU box; the dense path must agree with it on the
+    packed layout the reference uses, forward and gradients, to the bar of two bf16 kernels."""
+    _log("torch varlen_attn")
+    try:
+        from torch.nn.attention.varlen import varlen_attn as torch_varlen_attn
+    except Exception as e:                               # older / differently built torch
+        pytest.skip(f"torch.nn.attention.varlen not available: {e!r}")
+    for w in (W.scaled(W.C3, (700, 64, 1300, 1), name="vs-torch-gqa4"), W.scaled(W.C5, (333, 512, 90), name="vs-torch-d256")):
+        t = W.make_inputs(w, device=DEV)
+        cu = t["cu_seqlens"]
+        res = []
+        for fn in ("torch", "ours"):
+            q, k, v = (t[x].clone().requires_grad_(True) for x in ("q", "k", "v"))
+            if fn == "torch":
+                try:
+                    out = torch_varlen_attn(q, k, v, cu, cu, w.max_seqlen, w.max_seqlen, is_causal=True)
+                except Exception as e:
+                    pytest.skip(f"torch varlen_attn does not run on this build: {e!r}")
+            else:
+                out = ops.dsa_varlen_attn(q, k, v, cu, w.max_seqlen)
+            out.backward(t["dout"])
+            res.append((out.detach(), q.grad, k.grad, v.grad))
+        torch.cuda.synchronize()
+        for name, a, b in zip(("out", "dq", "dk", "dv"), res[1], res[0]):
+            err, cos = assert_close_bf16(a, b, f"{w.name} {name} vs torch")
+            _log(f"  {w.name} {name}: max-abs {err:.2e} cosine {cos:.6f}")
