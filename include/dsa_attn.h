@@ -135,6 +135,18 @@ int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k, const voi
                        int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen, int causal,
                        void *dq, void *dk, void *dv, void *ws, size_t ws_bytes, int parts, void *stream);
 
+/*
+ * Dense causal / non-causal packed attention, the operator the reference itself calls
+ * (torch.nn.attention.varlen.varlen_attn: train/model_attention.py:123-132, models/qwen3_vl/model.py:41-46,
+ * models/qwen3_5/model.py:93-98).  Same as dsa_attn_fwd / dsa_attn_bwd with idx == n == NULL and K == 0;
+ * no workspace is needed forward, dsa_attn_bwd_workspace_bytes(T, Hq, max_seqlen, 0) bytes backward.
+ */
+int dsa_dense_fwd(const void *q, const void *k, const void *v, const int32_t *cu_seqlens, int T, int N, int Hq, int Hkv,
+                  int D, float softmax_scale, int dtype, int max_seqlen, int causal, void *out, float *lse, void *stream);
+int dsa_dense_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out, const float *lse,
+                  const int32_t *cu_seqlens, int T, int N, int Hq, int Hkv, int D, float softmax_scale, int dtype,
+                  int max_seqlen, int causal, void *dq, void *dk, void *dv, void *ws, size_t ws_bytes, void *stream);
+
 /* ---------------------------------------------------------------------------------------------------
  * Pre-attention prologue and post-attention gate (the element-wise work either side of the operator).
  *

@@ -478,3 +478,30 @@ def test_dense_path_against_torch_varlen_attn_on_the_gpu():
         for name, a, b in zip(("out", "dq", "dk", "dv"), res[1], res[0]):
             err, cos = assert_close_bf16(a, b, f"{w.name} {name} vs torch")
             _log(f"  {w.name} {name}: max-abs {err:.2e} cosine {cos:.6f}")
+
+
+def test_dense_c_abi_entry_points_equal_the_general_ones():
+    """dsa_dense_fwd / dsa_dense_bwd are the general entry points with no selection: same bits."""
+    import ctypes
+    from vlm_training_amd import _lib
+    lib = _lib.load()
+    w = W.scaled(W.C2, (300, 77, 500), name="dense-abi")
+    t = W.make_inputs(w, device=DEV)
+    q, k, v, cu = t["q"], t["k"], t["v"], t["cu_seqlens"]
+    scale = w.D ** -0.5
+    out0, lse0 = ops.attn_fwd(q, k, v, None, None, cu, w.max_seqlen, scale)
+    dq0, dk0, dv0 = ops.attn_bwd(t["dout"], q, k, v, out0, lse0, None, None, cu, w.max_seqlen, scale)
+    out, lse = torch.empty_like(out0), torch.empty_like(lse0)
+    st = torch.cuda.current_stream().cuda_stream
+    p = lambda x: ctypes.c_void_p(x.data_ptr())
+    rc = lib.dsa_dense_fwd(p(q), p(k), p(v), p(cu), w.T, len(w.seg_lens), w.Hq, w.Hkv, w.D, scale, 0, w.max_seqlen, 1,
+                           p(out), p(lse), st)
+    assert rc == 0, lib.dsa_last_error()
+    ws = torch.empty((lib.dsa_attn_bwd_workspace_bytes(w.T, w.Hq, w.max_seqlen, 0),), dtype=torch.uint8, device=DEV)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    rc = lib.dsa_dense_bwd(p(t["dout"]), p(q), p(k), p(v), p(out), p(lse), p(cu), w.T, len(w.seg_lens), w.Hq, w.Hkv, w.D,
+                           scale, 0, w.max_seqlen, 1, p(dq), p(dk), p(dv), p(ws), ws.numel(), st)
+    assert rc == 0, lib.dsa_last_error()
+    torch.cuda.synchronize()
+    for a, b in ((out, out0), (lse, lse0), (dq, dq0), (dk, dk0), (dv, dv0)):
+        assert torch.equal(a, b)

@@ -274,6 +274,21 @@ extern "C" int dsa_attn_bwd(const void *dout, const void *q, const void *k, cons
                               causal, dq, dk, dv, ws, ws_bytes, DSA_BWD_ALL, stream);
 }
 
+extern "C" int dsa_dense_fwd(const void *q, const void *k, const void *v, const int32_t *cu, int T, int N, int Hq, int Hkv,
+                             int D, float softmax_scale, int dtype, int max_seqlen, int causal, void *out, float *lse,
+                             void *stream) {
+    return dsa_attn_fwd(q, k, v, nullptr, nullptr, cu, T, N, Hq, Hkv, D, 0, softmax_scale, dtype, max_seqlen, causal, out, lse,
+                        nullptr, 0, stream);
+}
+
+extern "C" int dsa_dense_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out, const float *lse,
+                             const int32_t *cu, int T, int N, int Hq, int Hkv, int D, float softmax_scale, int dtype,
+                             int max_seqlen, int causal, void *dq, void *dk, void *dv, void *ws, size_t ws_bytes,
+                             void *stream) {
+    return dsa_attn_bwd(dout, q, k, v, out, lse, nullptr, nullptr, cu, T, N, Hq, Hkv, D, 0, softmax_scale, dtype, max_seqlen,
+                        causal, dq, dk, dv, ws, ws_bytes, stream);
+}
+
 // ---------------------------------------------------------------------------------------------------
 // prologue / gate
 // ---------------------------------------------------------------------------------------------------

@@ -60,6 +60,9 @@ def _hf_indexer_to_packed(x):
 
 def varlen_attention_forward(query, key, value, attention_mask, **dsa):
     """(1,Hq,T,D),(1,Hkv,T,D),(1,Hkv,T,D), cu_seqlens -> ((1,T,Hq,D), None)."""
+    # tensor-parallel runs hand over DTensors sharded by head: the kernels see the local shard
+    # (train/model_attention.py:104-106)
+    query, key, value = (x.to_local() if hasattr(x, "to_local") else x for x in (query, key, value))
     # batch, head, seq_len, dim -> batch, seq_len, head, dim -> (T, head, dim)
     query = query.transpose(1, 2).contiguous()
     key = key.transpose(1, 2).contiguous()
