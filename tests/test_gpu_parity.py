@@ -216,13 +216,15 @@ def test_non_causal_packed_attention_for_the_vision_towers():
     g = torch.Generator().manual_seed(21)
     cu = [0, 64, 64, 320, 401, 977]
     T = cu[-1]
-    for Hq, Hkv, D in ((16, 16, 64), (4, 2, 128), (2, 1, 256)):
+    # 16 x 72 is the 1152-wide vision tower of the 8B models (head_dim between the kernels' sizes), 16 x 64 the 1024-wide one
+    for Hq, Hkv, D in ((16, 16, 64), (16, 16, 72), (4, 2, 128), (2, 1, 256)):
         q = (torch.randn(T, Hq, D, generator=g) * 0.6).bfloat16()
         k = (torch.randn(T, Hkv, D, generator=g) * 0.6).bfloat16()
         v = (torch.randn(T, Hkv, D, generator=g) * 0.6).bfloat16()
         do = torch.randn(T, Hq, D, generator=g).bfloat16()
         qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
         out = M.dispatch_varlen_attention(qd, kd, vd, torch.tensor(cu, dtype=torch.int32, device=DEV), 576, causal=False)
+        assert out.shape == (T, Hq, D)
         out.backward(do.to(DEV))
         qr, kr, vr = (x.float().requires_grad_(True) for x in (q, k, v))
         ref = R.dense_varlen_causal(qr, kr, vr, cu, causal=False)
@@ -324,8 +326,12 @@ def test_argument_errors_cross_the_boundary_as_exceptions():
     with pytest.raises(ValueError):
         ops.dsa_varlen_attn(q, k, k, cu, 8)
     q = torch.zeros(8, 4, 96, dtype=torch.bfloat16, device=DEV)
+    assert ops.dsa_varlen_attn(q, k, k, cu, 8).shape == q.shape        # padded to head_dim 128 and cut back
     with pytest.raises(RuntimeError):
-        ops.dsa_varlen_attn(q, k, k, cu, 8)            # head_dim 96 is not covered by the kernels
+        ops.attn_fwd(q, k, k, None, None, cu, 8, 0.1)  # the C ABI itself covers head_dim 64 / 128 / 256 only
+    big = torch.zeros(8, 2, 320, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError):
+        ops.dsa_varlen_attn(big, big, big, cu, 8)
     with pytest.raises(RuntimeError):
         ops.dsa_varlen_attn(q.cpu(), k.cpu(), k.cpu(), cu.cpu(), 8)
 

@@ -107,7 +107,7 @@ __global__ __launch_bounds__(64) void dsa_attn_fwd_kernel(
             mloc = fmaxf(mloc, s2[e]);
         }
         mloc = fmaxf(mloc, wave_xor_f(mloc, 16));
-        mloc = fmaxf(mloc, wave_xor_f(mloc, 32));
+        mloc = half_max_f(mloc);
         const float mnew = fmaxf(mrun, mloc);             // finite: key j0 is always valid
         const float alpha = exp2f(mrun - mnew);
         float psum = 0.f;
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(64) void dsa_attn_fwd_kernel(
     }
     float l = lsum;
     l += wave_xor_f(l, 16);
-    l += wave_xor_f(l, 32);
+    l = half_sum_f(l);
     const float inv = 1.f / l;
     if (m < G) {
         bf16_t *op = out + ((int64_t)t * Hq + kvh * G + m) * D + 4 * g;

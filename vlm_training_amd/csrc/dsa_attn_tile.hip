@@ -240,7 +240,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
             s2[vi] = keep_or_neginf(sacc[vi], bit_mask(word, 8 * (vi >> 2) + (vi & 3)));           \
             mloc = fmaxf(mloc, s2[vi]);                                                            \
         }                                                                                          \
-        mloc = fmaxf(mloc, wave_xor_f(mloc, 32)) * scale_log2;                                     \
+        mloc = half_max_f(mloc) * scale_log2;                                     \
         /* the reference maximum only moves when a row's maximum grows by more than 2^8 (rare      \
            after the first tiles); until then P stays below 2^8, exact in fp32 and safe in bf16 */ \
         if (__builtin_amdgcn_ballot_w64(mloc > mrun + 8.f)) {                                      \
@@ -270,7 +270,7 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
 #undef FWD_STORE
 #undef FWD_COMPUTE
 
-    float l = lsum + wave_xor_f(lsum, 32);
+    float l = half_sum_f(lsum);
     if (row_ok) {
         const float inv = 1.f / l;
         bf16_t *op = out + ((int64_t)t * Hq + hq) * D + 4 * h;

@@ -54,3 +54,13 @@ __device__ __forceinline__ int find_segment(const int32_t *__restrict__ cu, int 
 }
 
 __device__ __forceinline__ float wave_xor_f(float v, int m) { return __shfl_xor(v, m, 64); }
+// maximum / sum over the two lanes 32 apart, on every lane: v_permlane32_swap exchanges the wave's halves in
+// the vector ALU (no LDS round trip, so LDS reads in flight are not waited for)
+__device__ __forceinline__ float half_max_f(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_sum_f(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}

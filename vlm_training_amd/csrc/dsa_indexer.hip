@@ -121,7 +121,7 @@ __global__ __launch_bounds__(IDX_WAVES * 64, 2) void dsa_indexer_scores_kernel(
                 for (int ht = 0; ht < HT; ++ht)
 #pragma unroll
                     for (int v = 0; v < 16; ++v) sum += wreg[ht][v] * __int_as_float(max(__float_as_int(acc[ht][v]), 0));
-                sum += wave_xor_f(sum, 32);
+                sum = half_sum_f(sum);
                 const int s = kb + (lane & 31);
                 if (lane < 32 && s >= s0 && s <= t) orow[s - s0] = sum * scale;
             };

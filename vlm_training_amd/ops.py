@@ -42,6 +42,9 @@ def _check_cu(cu_seqlens: torch.Tensor, T: int):
     return cu_seqlens.contiguous()
 
 
+_KERNEL_HEAD_DIMS = (64, 128, 256)                   # head_dim instantiations of the tile and gather kernels
+
+
 def _check_qkv(q, k, v):
     if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
         raise ValueError("q, k, v must be (T, H, D)")
@@ -269,7 +272,8 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, in
     every causal key of the token's own segment is attended (the reference's behaviour).  With
     ``indexer_q (T,Hi,Di)``, ``indexer_k (T,Di)``, ``indexer_w (T,Hi)`` and ``top_k`` each query keeps
     the top_k keys of its causal window under (indexer score descending, key index ascending).
-    Gradients flow to q, k, v only.  ``causal=False`` (dense only) attends every key of the own segment, the
+    Gradients flow to q, k, v only.  A head_dim between the kernels' 64 / 128 / 256 is zero-padded to the
+    next one and the output cut back (the scale stays that of the true head_dim).  ``causal=False`` (dense only) attends every key of the own segment, the
     vision towers' form of the call (models/qwen3_vl/model.py:423-428).
     """
     _require_cuda(q, k, v, cu_seqlens)
@@ -290,6 +294,14 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, in
             idx, n = index_topk(indexer_q, indexer_k, indexer_w, cu, int(max_seqlen), int(top_k), index_scale)
     elif return_indices:
         raise ValueError("return_indices needs the indexer inputs")
+    d_kernel = next((d for d in _KERNEL_HEAD_DIMS if d >= D), None)
+    if d_kernel is None:
+        raise ValueError(f"head_dim {D} is beyond the kernels' largest ({_KERNEL_HEAD_DIMS[-1]})")
+    if d_kernel != D:
+        # e.g. the 72-wide heads of the 1152/16 vision towers: zero columns change neither q.k nor the used part of p.v
+        q, k, v = (torch.nn.functional.pad(x, (0, d_kernel - D)) for x in (q, k, v))
     out = _DsaVarlenAttn.apply(q.contiguous(), k.contiguous(), v.contiguous(), cu, int(max_seqlen), idx, n, scale,
                                bool(causal))
+    if d_kernel != D:
+        out = out[..., :D]
     return (out, idx, n) if return_indices else out
