@@ -112,18 +112,25 @@ __device__ __forceinline__ f32x16 zero16() {
 
 // slot -> (segment, block) for blocks of `blk` columns handed out segment by segment; within a segment
 // the blocks are numbered from the end when `reverse` (heaviest causal blocks first).  Returns false
-// for spare slots.
+// for spare slots.  The segment bounds are fetched 64 segments at a time, one per lane (one memory
+// round trip instead of one per segment), and walked with lane reads.
 __device__ __forceinline__ bool locate_block(const int32_t *cu, int N, int slot, int blk, bool reverse, int &s0, int &L,
                                              int &b) {
-    for (int seg = 0; seg < N; ++seg) {
-        s0 = cu[seg];
-        L = cu[seg + 1] - s0;
-        const int nb = (L + blk - 1) / blk;
-        if (slot < nb) {
-            b = reverse ? nb - 1 - slot : slot;
-            return true;
+    const int lane = threadIdx.x & 63;
+    for (int base = 0; base < N; base += 64) {
+        const int seg = min(base + lane, N - 1);
+        const int lo = cu[seg], len = cu[seg + 1] - lo;
+        const int cnt = min(64, N - base);
+        for (int w = 0; w < cnt; ++w) {
+            L = __builtin_amdgcn_readlane(len, w);
+            const int nb = (L + blk - 1) / blk;
+            if (slot < nb) {
+                s0 = __builtin_amdgcn_readlane(lo, w);
+                b = reverse ? nb - 1 - slot : slot;
+                return true;
+            }
+            slot -= nb;
         }
-        slot -= nb;
     }
     return false;
 }
@@ -139,11 +146,11 @@ __device__ __forceinline__ bool locate_block(const int32_t *cu, int N, int slot,
 // ==================================================================================================
 // Every global load of the pipeline is issued unconditionally (indices past the end are clamped to
 // the last tile) and nothing is computed from a loaded value before the matching STORE, so the
-// compiler can wait with exact vmcnt counts and a load has two tile-times to land.
+// compiler can wait with exact vmcnt counts and a load has two tile-times to land.  The kernel issues
+// LOAD(0, 0) itself, before the loads of its stationary rows.
 #define TILE_PIPELINE(NT, LOAD, STORE, COMPUTE)                                                     \
     {                                                                                              \
         const int nt_last = (NT) - 1;                                                              \
-        LOAD(0, 0);                                                                                \
         STORE(0, 0, 0);                                                                            \
         LOAD(0, min(1, nt_last));                                                                  \
         LOAD(1, min(2, nt_last));                                                                  \
@@ -165,14 +172,14 @@ __device__ __forceinline__ bool locate_block(const int32_t *cu, int N, int slot,
         if (it < (NT)) COMPUTE(it, 0);                                                             \
     }
 
-template <int D, bool HAS_IDX, int GSHIFT>
-__global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
+template <int D, bool HAS_IDX, int GSHIFT, int NW>
+__global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_tile_fwd_kernel(
     const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
     float scale_log2, int pos_split, int causal, bf16_t *__restrict__ out, float *__restrict__ lse) {
-    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / 256;
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / (NW * 64);
     constexpr int NBUF = (D > 128) ? 1 : 2;           // double buffering where 64 KiB of static LDS allow it
-    constexpr int Gp = 1 << GSHIFT, QBW = 128 >> GSHIFT;
+    constexpr int NT = NW * 64, Gp = 1 << GSHIFT, QBW = (NW * 32) >> GSHIFT;
     static_assert(LOADS >= 1, "tile must give every thread a chunk");
     __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];   // [buffer][K|V]
 
@@ -190,6 +197,16 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
     const int qcol = qc0 + (r >> GSHIFT), head = r & (Gp - 1);
     const bool row_ok = qcol < L && head < G;
     const int t = s0 + min(qcol, L - 1), hq = kvh * G + min(head, G - 1);
+    u32x4 kst[2][LOADS], vst[2][LOADS];
+#define FWD_LOAD(SET, TILE)                                                                         \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+        const int c = i * NT + tid;                                                               \
+        const int row = c / CPR, ch = c % CPR;                                                     \
+        const int64_t off = ((int64_t)(s0 + min((TILE) * 32 + row, L - 1)) * Hkv + kvh) * D + ch * 8; \
+        kst[SET][i] = *reinterpret_cast<const u32x4 *>(k + off);                                   \
+        vst[SET][i] = *reinterpret_cast<const u32x4 *>(v + off);                                   \
+    }
+    FWD_LOAD(0, 0)                                      // ahead of the q rows: staging waits for this tile only
     bf16x8 qB[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
@@ -198,24 +215,15 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
     const int klim = causal ? qcol : L - 1;             // last key column this row may attend (dense mode)
     const uint32_t *wrow = bitmap + (int64_t)t * ldw;
 
-    u32x4 kst[2][LOADS], vst[2][LOADS];
     f32x16 oacc[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) oacc[dt] = zero16();
     float mrun = -INFINITY, lsum = 0.f;
     uint32_t word_next = HAS_IDX ? wrow[0] : 0u;        // unconditional loads; rows that are not live are masked at use
 
-#define FWD_LOAD(SET, TILE)                                                                         \
-    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
-        const int c = i * 256 + tid;                                                               \
-        const int row = c / CPR, ch = c % CPR;                                                     \
-        const int64_t off = ((int64_t)(s0 + min((TILE) * 32 + row, L - 1)) * Hkv + kvh) * D + ch * 8; \
-        kst[SET][i] = *reinterpret_cast<const u32x4 *>(k + off);                                   \
-        vst[SET][i] = *reinterpret_cast<const u32x4 *>(v + off);                                   \
-    }
 #define FWD_STORE(SET, BUF, TILE)                                                                        \
     _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
-        const int c = i * 256 + tid;                                                               \
+        const int c = i * NT + tid;                                                               \
         const int row = c / CPR, ch = c % CPR;                                                     \
         *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(row, ch)]) = kst[SET][i];              \
         *reinterpret_cast<u32x4 *>(&lds[BUF][1][tile_off<D>(row, ch)]) = vst[SET][i];              \
@@ -292,15 +300,15 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_fwd_kernel(
 //   dS^T = P^T * (dP^T - delta)  on the C layout
 //   dQ^T[d,row] += K^T[d,key] dS^T[key,row]   (A = K tile transposed, B = dS^T from the C layout)
 // ==================================================================================================
-template <int D, bool HAS_IDX, int GSHIFT>
-__global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
+template <int D, bool HAS_IDX, int GSHIFT, int NW>
+__global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_tile_dq_kernel(
     const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
     float scale, int pos_split, int causal, bf16_t *__restrict__ dq) {
-    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / 256;
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / (NW * 64);
     constexpr int NBUF = (D > 128) ? 1 : 2;
-    constexpr int Gp = 1 << GSHIFT, QBW = 128 >> GSHIFT;
+    constexpr int NT = NW * 64, Gp = 1 << GSHIFT, QBW = (NW * 32) >> GSHIFT;
     __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
@@ -318,6 +326,16 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
     const bool row_ok = qcol < L && head < G;
     const int t = s0 + min(qcol, L - 1), hq = kvh * G + min(head, G - 1);
     const float scale_log2 = scale * LOG2E_F;
+    u32x4 kst[2][LOADS], vst[2][LOADS];
+#define DQ_LOAD(SET, TILE)                                                                          \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+        const int c = i * NT + tid;                                                               \
+        const int row = c / CPR, ch = c % CPR;                                                     \
+        const int64_t off = ((int64_t)(s0 + min((TILE) * 32 + row, L - 1)) * Hkv + kvh) * D + ch * 8; \
+        kst[SET][i] = *reinterpret_cast<const u32x4 *>(k + off);                                   \
+        vst[SET][i] = *reinterpret_cast<const u32x4 *>(v + off);                                   \
+    }
+    DQ_LOAD(0, 0)                                       // ahead of the q / dO rows: staging waits for this tile only
     bf16x8 qB[KS], doB[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -331,23 +349,14 @@ __global__ __launch_bounds__(256, (D <= 128) ? 2 : 1) void dsa_tile_dq_kernel(
     const int klim = causal ? qcol : L - 1;             // last key column this row may attend (dense mode)
     const uint32_t *wrow = bitmap + (int64_t)t * ldw;
 
-    u32x4 kst[2][LOADS], vst[2][LOADS];
     f32x16 acc[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
     uint32_t word_next = HAS_IDX ? wrow[0] : 0u;        // unconditional loads; rows that are not live are masked at use
 
-#define DQ_LOAD(SET, TILE)                                                                          \
-    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
-        const int c = i * 256 + tid;                                                               \
-        const int row = c / CPR, ch = c % CPR;                                                     \
-        const int64_t off = ((int64_t)(s0 + min((TILE) * 32 + row, L - 1)) * Hkv + kvh) * D + ch * 8; \
-        kst[SET][i] = *reinterpret_cast<const u32x4 *>(k + off);                                   \
-        vst[SET][i] = *reinterpret_cast<const u32x4 *>(v + off);                                   \
-    }
 #define DQ_STORE(SET, BUF, TILE)                                                                         \
     _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
-        const int c = i * 256 + tid;                                                               \
+        const int c = i * NT + tid;                                                               \
         const int row = c / CPR, ch = c % CPR;                                                     \
         *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(row, ch)]) = kst[SET][i];              \
         *reinterpret_cast<u32x4 *>(&lds[BUF][1][tile_off<D>(row, ch)]) = vst[SET][i];              \
@@ -811,18 +820,24 @@ static inline int group_shift(int Hq, int Hkv) {
     return gshift;
 }
 
+// waves per workgroup of the query-stationary kernels: all of them share the staged K / V tiles
+#ifndef DSA_TILE_WAVES_128
+#define DSA_TILE_WAVES_128 8
+#endif
+template <int D> constexpr int tile_waves() { return D == 128 ? DSA_TILE_WAVES_128 : 4; }
+static inline int tile_waves_of(int D) { return D == 128 ? DSA_TILE_WAVES_128 : 4; }
 template <int D, bool HAS_IDX, int GS>
 static void launch_fwd_i(dim3 grid, hipStream_t stream, const void *q, const void *k, const void *v,
                          const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T, int Hq, int Hkv, float sl2,
                          int pos_split, int causal, void *out, float *lse) {
-    hipLaunchKernelGGL((dsa_tile_fwd_kernel<D, HAS_IDX, GS>), grid, dim3(256), 0, stream, (const bf16_t *)q,
+    hipLaunchKernelGGL((dsa_tile_fwd_kernel<D, HAS_IDX, GS, tile_waves<D>()>), grid, dim3(64 * tile_waves<D>()), 0, stream, (const bf16_t *)q,
                        (const bf16_t *)k, (const bf16_t *)v, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, pos_split, causal, (bf16_t *)out, lse);
 }
 template <int D, bool HAS_IDX, int GS>
 static void launch_dq_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
                         const float *lse, const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N,
                         int T, int Hq, int Hkv, float scale, int pos_split, int causal, void *dq) {
-    hipLaunchKernelGGL((dsa_tile_dq_kernel<D, HAS_IDX, GS>), grid, dim3(256), 0, stream, (const bf16_t *)dout,
+    hipLaunchKernelGGL((dsa_tile_dq_kernel<D, HAS_IDX, GS, tile_waves<D>()>), grid, dim3(64 * tile_waves<D>()), 0, stream, (const bf16_t *)dout,
                        (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv,
                        scale, pos_split, causal, (bf16_t *)dq);
 }
@@ -863,7 +878,7 @@ extern "C" hipError_t dsa_launch_tile_fwd(const void *q, const void *k, const vo
                                           const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale,
                                           int pos_split, int causal, void *out, float *lse, hipStream_t stream) {
     const int gs = group_shift(Hq, Hkv);
-    const dim3 grid((unsigned)(((int64_t)T / (128 >> gs) + N + 1) * Hkv));
+    const dim3 grid((unsigned)(((int64_t)T / ((32 * tile_waves_of(D)) >> gs) + N + 1) * Hkv));
     TILE_SWITCH(launch_fwd_i, grid, stream, q, k, v, bitmap, ldw, cu, N, T, Hq, Hkv, scale * LOG2E_F, pos_split, causal, out, lse)
     return hipGetLastError();
 }
@@ -872,7 +887,7 @@ extern "C" hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const 
                                          const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale,
                                          int pos_split, int causal, void *dq, hipStream_t stream) {
     const int gs = group_shift(Hq, Hkv);
-    const dim3 grid((unsigned)(((int64_t)T / (128 >> gs) + N + 1) * Hkv));
+    const dim3 grid((unsigned)(((int64_t)T / ((32 * tile_waves_of(D)) >> gs) + N + 1) * Hkv));
     TILE_SWITCH(launch_dq_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, pos_split, causal, dq)
     return hipGetLastError();
 }
