@@ -110,6 +110,22 @@ __device__ __forceinline__ f32x16 zero16() {
     return z;
 }
 
+// Write one 32-column d-tile of a C-layout accumulator as bf16 (lane = row j; a lane holds the four
+// columns 8*g4 + 4*h + {0..3} of every group g4, so a 16-byte chunk of the row is split over the two
+// lanes 32 apart).  The halves of the wave exchange 8-byte pieces - lane (j,0) takes chunk 2m whole,
+// lane (j,1) chunk 2m+1 - and every lane stores 16 bytes.  Both lanes of a row must be active.
+__device__ __forceinline__ void store_c_tile(bf16_t *row_dt, const f32x16 &acc, float mul, int h) {
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+        const uint32_t a0 = pack2bf(acc[8 * m] * mul, acc[8 * m + 1] * mul), a1 = pack2bf(acc[8 * m + 2] * mul, acc[8 * m + 3] * mul);
+        const uint32_t b0 = pack2bf(acc[8 * m + 4] * mul, acc[8 * m + 5] * mul), b1 = pack2bf(acc[8 * m + 6] * mul, acc[8 * m + 7] * mul);
+        const auto r0 = __builtin_amdgcn_permlane32_swap(a0, b0, false, false);   // upper lanes of a <-> lower lanes of b
+        const auto r1 = __builtin_amdgcn_permlane32_swap(a1, b1, false, false);
+        const u32x4 w = {r0[0], r1[0], r0[1], r1[1]};
+        *reinterpret_cast<u32x4 *>(row_dt + 8 * (2 * m + h)) = w;
+    }
+}
+
 // slot -> (segment, block) for blocks of `blk` columns handed out segment by segment; within a segment
 // the blocks are numbered from the end when `reverse` (heaviest causal blocks first).  Returns false
 // for spare slots.  The segment bounds are fetched 64 segments at a time, one per lane (one memory
@@ -281,15 +297,9 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     float l = half_sum_f(lsum);
     if (row_ok) {
         const float inv = 1.f / l;
-        bf16_t *op = out + ((int64_t)t * Hq + hq) * D + 4 * h;
+        bf16_t *op = out + ((int64_t)t * Hq + hq) * D;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                const u32x2 w2 = {pack2bf(oacc[dt][4 * g4] * inv, oacc[dt][4 * g4 + 1] * inv),
-                                  pack2bf(oacc[dt][4 * g4 + 2] * inv, oacc[dt][4 * g4 + 3] * inv)};
-                *reinterpret_cast<u32x2 *>(op + dt * 32 + 8 * g4) = w2;
-            }
+        for (int dt = 0; dt < DT; ++dt) store_c_tile(op + dt * 32, oacc[dt], inv, h);
         if (h == 0) lse[(int64_t)hq * T + t] = (mrun + log2f(l)) * LN2_F;
     }
 }
@@ -394,15 +404,9 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
 #undef DQ_COMPUTE
 
     if (row_ok) {
-        bf16_t *op = dq + ((int64_t)t * Hq + hq) * D + 4 * h;
+        bf16_t *op = dq + ((int64_t)t * Hq + hq) * D;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                const u32x2 w2 = {pack2bf(acc[dt][4 * g4] * scale, acc[dt][4 * g4 + 1] * scale),
-                                  pack2bf(acc[dt][4 * g4 + 2] * scale, acc[dt][4 * g4 + 3] * scale)};
-                *reinterpret_cast<u32x2 *>(op + dt * 32 + 8 * g4) = w2;
-            }
+        for (int dt = 0; dt < DT; ++dt) store_c_tile(op + dt * 32, acc[dt], scale, h);
     }
 }
 
@@ -629,18 +633,12 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
         }
 #undef DKV_CONSUMER_STEP
         if (key_ok) {
-            bf16_t *pk = dk + krow * D + dt0 * 32 + 4 * h, *pv_ = dv + krow * D + dt0 * 32 + 4 * h;
+            bf16_t *pk = dk + krow * D + dt0 * 32, *pv_ = dv + krow * D + dt0 * 32;
 #pragma unroll
-            for (int dt = 0; dt < DTC; ++dt)
-#pragma unroll
-                for (int g4 = 0; g4 < 4; ++g4) {
-                    const u32x2 wk = {pack2bf(dkacc[dt][4 * g4] * scale, dkacc[dt][4 * g4 + 1] * scale),
-                                      pack2bf(dkacc[dt][4 * g4 + 2] * scale, dkacc[dt][4 * g4 + 3] * scale)};
-                    const u32x2 wvv = {pack2bf(dvacc[dt][4 * g4], dvacc[dt][4 * g4 + 1]),
-                                       pack2bf(dvacc[dt][4 * g4 + 2], dvacc[dt][4 * g4 + 3])};
-                    *reinterpret_cast<u32x2 *>(pk + dt * 32 + 8 * g4) = wk;
-                    *reinterpret_cast<u32x2 *>(pv_ + dt * 32 + 8 * g4) = wvv;
-                }
+            for (int dt = 0; dt < DTC; ++dt) {
+                store_c_tile(pk + dt * 32, dkacc[dt], scale, h);
+                store_c_tile(pv_ + dt * 32, dvacc[dt], 1.f, h);
+            }
         }
         return;
     }
