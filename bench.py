@@ -123,6 +123,35 @@ def reference_operator(w, t, iters):
             "torch_varlen_attn_ms": theirs, "this_library_dense_ms": ours, "speedup": theirs / ours}
 
 
+def vision_tower_operator(dev, iters):
+    """The vision towers' form of the call (models/qwen3_vl/model.py:423-428): non-causal packed attention over the
+    patches of each image, 16 heads of 72 (hidden 1152) or 64 (hidden 1024), six images of 768-4096 patches."""
+    from vlm_training_amd import dispatch_varlen_attention
+    try:
+        from torch.nn.attention.varlen import varlen_attn as torch_varlen_attn
+    except Exception:
+        torch_varlen_attn = None
+    lens = [4096, 4096, 2304, 1024, 4096, 768]
+    T, H = sum(lens), 16
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=dev)
+    g = torch.Generator(device=dev).manual_seed(5)
+    res = {"what": f"non-causal packed attention fwd+bwd, {H} heads, images of {lens} patches"}
+    for D in (72, 64):
+        q, k, v = (torch.randn(T, H, D, device=dev, generator=g).mul_(0.5).bfloat16().requires_grad_(True) for _ in range(3))
+        do = torch.randn(T, H, D, device=dev, generator=g).bfloat16()
+        pairs = sum(n * n for n in lens)
+        ms = timed(lambda: dispatch_varlen_attention(q, k, v, cu, max(lens), causal=False).backward(do), iters)
+        e = {"ms": ms, "TFLOP/s": 14.0 * H * D * pairs / ms / 1e9}          # 4 (forward) + 10 (backward) flop per pair, head and dim
+        if torch_varlen_attn is not None:
+            try:
+                e["torch_varlen_attn_ms"] = timed(
+                    lambda: torch_varlen_attn(q, k, v, cu, cu, max(lens), max(lens), is_causal=False).backward(do), iters)
+            except Exception as ex:
+                e["torch_varlen_attn_error"] = repr(ex)[:200]
+        res[f"head_dim_{D}"] = e
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -239,6 +268,7 @@ def main():
     }
     result["adjacent_kernels"] = prologue_stage(w, dev, it)
     result["reference_operator"] = reference_operator(w, t, it)
+    result["vision_tower_operator"] = vision_tower_operator(dev, it)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, torch.get_num_threads())
     print(json.dumps(result))

@@ -22,13 +22,13 @@ __device__ __forceinline__ uint32_t score_key(float x) {
 
 template <bool CACHED>
 __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
-    const float *__restrict__ scores, int64_t ld, int row_begin, const int32_t *__restrict__ cu, int N, int K,
+    const float *__restrict__ scores, int64_t ld, int row_begin, const int32_t *__restrict__ cu, int N, int K, int lds_keys,
     int32_t *__restrict__ idx_out, int32_t *__restrict__ n_out) {
     __shared__ uint32_t hist[256];
     __shared__ uint32_t wave_tot[4];
     __shared__ uint32_t sel_digit, sel_remaining;
     __shared__ uint32_t cnt_gt[4], cnt_eq[4];
-    __shared__ uint32_t keys_lds[CACHED ? TOPK_LDS_CAP : 1];
+    extern __shared__ __attribute__((aligned(16))) uint32_t keys_lds[];   // CACHED: the launch's longest row; the fewer bytes, the more rows per CU
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int t = row_begin + blockIdx.x;
@@ -43,10 +43,31 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
         return;
     }
     const float *row = scores + (int64_t)(t - row_begin) * ld;
-    if (CACHED) {
-        for (int i = tid; i < nvalid; i += TOPK_THREADS) keys_lds[i] = score_key(row[i]);
+    const bool cached = CACHED && nvalid <= lds_keys;    // a row beyond the stated longest one is read from memory each pass
+    if (cached) {
+        // 16-byte loads, four per thread in flight: one load per loop iteration would pay the memory latency
+        // nvalid / 256 times over
+        const float4 *row4 = reinterpret_cast<const float4 *>(row);
+        const int n4 = (reinterpret_cast<uintptr_t>(row) & 15) ? 0 : nvalid >> 2;   // a caller's own rows may not be aligned
+        for (int base = 0; base < n4; base += 4 * TOPK_THREADS) {
+            float4 x[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i4 = base + u * TOPK_THREADS + tid;
+                x[u] = row4[min(i4, n4 - 1)];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i4 = base + u * TOPK_THREADS + tid;
+                if (i4 < n4) {
+                    const uint4 kk = {score_key(x[u].x), score_key(x[u].y), score_key(x[u].z), score_key(x[u].w)};
+                    *reinterpret_cast<uint4 *>(&keys_lds[4 * i4]) = kk;
+                }
+            }
+        }
+        for (int i = (n4 << 2) + tid; i < nvalid; i += TOPK_THREADS) keys_lds[i] = score_key(row[i]);
     }
-    auto key_at = [&](int i) -> uint32_t { return CACHED ? keys_lds[i] : score_key(row[i]); };
+    auto key_at = [&](int i) -> uint32_t { return cached ? keys_lds[i] : score_key(row[i]); };
 
     uint32_t prefix = 0u, pmask = 0u, remaining = (uint32_t)K;
     for (int pass = 0; pass < 4; ++pass) {
@@ -129,10 +150,10 @@ extern "C" hipError_t dsa_launch_topk(const float *scores, int64_t ld, int row_b
     const int rows = row_end - row_begin;
     if (rows <= 0) return hipSuccess;
     if (max_row <= TOPK_LDS_CAP)
-        hipLaunchKernelGGL(dsa_topk_rows_kernel<true>, dim3(rows), dim3(TOPK_THREADS), 0, stream, scores, ld,
-                           row_begin, cu, N, K, idx, n);
+        hipLaunchKernelGGL(dsa_topk_rows_kernel<true>, dim3(rows), dim3(TOPK_THREADS), (size_t)((max_row + 3) & ~3) * 4, stream,
+                           scores, ld, row_begin, cu, N, K, (max_row + 3) & ~3, idx, n);
     else
-        hipLaunchKernelGGL(dsa_topk_rows_kernel<false>, dim3(rows), dim3(TOPK_THREADS), 0, stream, scores, ld,
-                           row_begin, cu, N, K, idx, n);
+        hipLaunchKernelGGL(dsa_topk_rows_kernel<false>, dim3(rows), dim3(TOPK_THREADS), 16, stream, scores, ld,
+                           row_begin, cu, N, K, 0, idx, n);
     return hipGetLastError();
 }
