@@ -140,12 +140,17 @@ def vision_tower_operator(dev, iters):
         q, k, v = (torch.randn(T, H, D, device=dev, generator=g).mul_(0.5).bfloat16().requires_grad_(True) for _ in range(3))
         do = torch.randn(T, H, D, device=dev, generator=g).bfloat16()
         pairs = sum(n * n for n in lens)
-        ms = timed(lambda: dispatch_varlen_attention(q, k, v, cu, max(lens), causal=False).backward(do), iters)
+
+        def run(fn):
+            q.grad = k.grad = v.grad = None              # no accumulation kernels inside the timed region
+            fn(q, k, v).backward(do)
+
+        ms = timed(lambda: run(lambda a, b, c: dispatch_varlen_attention(a, b, c, cu, max(lens), causal=False)), iters)
         e = {"ms": ms, "TFLOP/s": 14.0 * H * D * pairs / ms / 1e9}          # 4 (forward) + 10 (backward) flop per pair, head and dim
         if torch_varlen_attn is not None:
             try:
-                e["torch_varlen_attn_ms"] = timed(
-                    lambda: torch_varlen_attn(q, k, v, cu, cu, max(lens), max(lens), is_causal=False).backward(do), iters)
+                e["torch_varlen_attn_ms"] = timed(lambda: run(lambda a, b, c: torch_varlen_attn(
+                    a, b, c, cu, cu, max(lens), max(lens), is_causal=False)), iters)
             except Exception as ex:
                 e["torch_varlen_attn_error"] = repr(ex)[:200]
         res[f"head_dim_{D}"] = e

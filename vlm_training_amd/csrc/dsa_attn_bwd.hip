@@ -173,7 +173,22 @@ __global__ __launch_bounds__(256) void dsa_bitmap_kernel(const int32_t *__restri
     __syncthreads();
     const int nt = nsel[t];
     const int32_t *irow = idx + (int64_t)t * K;
-    for (int j = tid; j < nt; j += 256) {
+    // 16-byte loads, all of a thread's in flight (one load per loop iteration would pay the memory latency nt/256 times)
+    const int n4 = (reinterpret_cast<uintptr_t>(irow) & 15) ? 0 : nt >> 2;
+    const int4 *irow4 = reinterpret_cast<const int4 *>(irow);
+    for (int base = 0; base < n4; base += 4 * 256) {
+        int4 c4[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) c4[u] = irow4[min(base + u * 256 + tid, n4 - 1)];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (base + u * 256 + tid < n4) {
+                const int cs[4] = {c4[u].x - s0, c4[u].y - s0, c4[u].z - s0, c4[u].w - s0};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) atomicOr(&words[cs[e] >> 5], 1u << (cs[e] & 31));
+            }
+    }
+    for (int j = (n4 << 2) + tid; j < nt; j += 256) {
         const int c = irow[j] - s0;
         atomicOr(&words[c >> 5], 1u << (c & 31));
     }
