@@ -74,9 +74,14 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
         const int shift = 24 - 8 * pass;
         hist[tid] = 0u;
         __syncthreads();
-        for (int i = tid; i < nvalid; i += TOPK_THREADS) {
-            uint32_t key = key_at(i);
-            if ((key & pmask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+        // eight keys per thread in flight (rows that are not cached come from memory on every sweep)
+        for (int base = tid; base < nvalid; base += 8 * TOPK_THREADS) {
+            uint32_t kk[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) kk[u] = key_at(min(base + u * TOPK_THREADS, nvalid - 1));
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (base + u * TOPK_THREADS < nvalid && (kk[u] & pmask) == prefix) atomicAdd(&hist[(kk[u] >> shift) & 255u], 1u);
         }
         __syncthreads();
         // inclusive suffix sum over the 256 digits (digit 255 first)
@@ -106,10 +111,16 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
     const int per = (((nvalid + 3) >> 2) + 63) & ~63;
     const int c_begin = min(wv * per, nvalid), c_end = min(c_begin + per, nvalid);
     uint32_t g = 0, e = 0;
-    for (int i = c_begin + lane; i < c_end; i += 64) {
-        uint32_t key = key_at(i);
-        g += key > tau;
-        e += key == tau;
+    for (int base = c_begin + lane; base < c_end; base += 8 * 64) {
+        uint32_t kk[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) kk[u] = key_at(min(base + u * 64, nvalid - 1));
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (base + u * 64 < c_end) {
+                g += kk[u] > tau;
+                e += kk[u] == tau;
+            }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -125,21 +136,23 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
         eq_seen += cnt_eq[w2];
     }
     const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-    for (int i0 = c_begin; i0 < c_end; i0 += 64) {
-        const int i = i0 + lane;
-        bool is_gt = false, is_eq = false;
-        if (i < c_end) {
-            uint32_t key = key_at(i);
-            is_gt = key > tau;
-            is_eq = key == tau;
+    for (int base = c_begin; base < c_end; base += 4 * 64) {
+        uint32_t kk[4];                                 // four chunks of 64 columns fetched, then ranked in index order
+#pragma unroll
+        for (int u = 0; u < 4; ++u) kk[u] = key_at(min(base + u * 64 + lane, nvalid - 1));
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int i = base + u * 64 + lane;
+            if (base + u * 64 >= c_end) break;          // wave-uniform
+            const bool is_gt = i < c_end && kk[u] > tau, is_eq = i < c_end && kk[u] == tau;
+            const uint64_t b_eq = __ballot(is_eq);
+            const uint32_t eq_rank = eq_seen + (uint32_t)__popcll(b_eq & lt_mask);
+            const bool take = is_gt || (is_eq && eq_rank < need_eq);
+            const uint64_t b_take = __ballot(take);
+            if (take) orow[out_pos + (uint32_t)__popcll(b_take & lt_mask)] = s0 + i;
+            out_pos += (uint32_t)__popcll(b_take);
+            eq_seen += (uint32_t)__popcll(b_eq);
         }
-        const uint64_t b_eq = __ballot(is_eq);
-        const uint32_t eq_rank = eq_seen + (uint32_t)__popcll(b_eq & lt_mask);
-        const bool take = is_gt || (is_eq && eq_rank < need_eq);
-        const uint64_t b_take = __ballot(take);
-        if (take) orow[out_pos + (uint32_t)__popcll(b_take & lt_mask)] = s0 + i;
-        out_pos += (uint32_t)__popcll(b_take);
-        eq_seen += (uint32_t)__popcll(b_eq);
     }
     if (tid == 0) n_out[t] = K;
 }
