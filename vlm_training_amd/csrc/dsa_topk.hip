@@ -2,8 +2,9 @@
 // ascending).  One 256-thread workgroup per query row.
 //
 //   1. rows with pos+1 <= K are the whole causal window: write the range, done;
-//   2. MSB-first radix select (4 passes x 8 bits) over order-preserving uint32 keys finds the K-th
-//      largest key tau and how many keys equal to tau are still wanted (need_eq);
+//   2. MSB-first radix select (3 passes of 11, 11 and 10 bits) over order-preserving uint32 keys finds the
+//      K-th largest key tau and how many keys equal to tau are still wanted (need_eq); the first histogram
+//      is filled while the row is read;
 //   3. an index-ordered compaction keeps key > tau, plus the first need_eq keys == tau.  The row is
 //      split into four contiguous quarters (one per wave); per-quarter counts give every wave its
 //      output offset, so the result comes out ascending and deterministic without sorting.
@@ -13,6 +14,7 @@
 
 #define TOPK_THREADS 256
 #define TOPK_LDS_CAP 8192
+#define TOPK_BINS 2048                                  // 11-bit digits (the last pass uses 1024 of them)
 
 __device__ __forceinline__ uint32_t score_key(float x) {
     uint32_t u = __float_as_uint(x);
@@ -24,7 +26,7 @@ template <bool CACHED>
 __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
     const float *__restrict__ scores, int64_t ld, int row_begin, const int32_t *__restrict__ cu, int N, int K, int lds_keys,
     int32_t *__restrict__ idx_out, int32_t *__restrict__ n_out) {
-    __shared__ uint32_t hist[256];
+    __shared__ uint32_t hist[TOPK_BINS];
     __shared__ uint32_t wave_tot[4];
     __shared__ uint32_t sel_digit, sel_remaining;
     __shared__ uint32_t cnt_gt[4], cnt_eq[4];
@@ -44,6 +46,8 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
     }
     const float *row = scores + (int64_t)(t - row_begin) * ld;
     const bool cached = CACHED && nvalid <= lds_keys;    // a row beyond the stated longest one is read from memory each pass
+    for (int i = tid; i < TOPK_BINS; i += TOPK_THREADS) hist[i] = 0u;
+    __syncthreads();
     if (cached) {
         // 16-byte loads, four per thread in flight: one load per loop iteration would pay the memory latency
         // nvalid / 256 times over
@@ -62,30 +66,50 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
                 if (i4 < n4) {
                     const uint4 kk = {score_key(x[u].x), score_key(x[u].y), score_key(x[u].z), score_key(x[u].w)};
                     *reinterpret_cast<uint4 *>(&keys_lds[4 * i4]) = kk;
+                    atomicAdd(&hist[kk.x >> 21], 1u);    // first digit: the top 11 bits
+                    atomicAdd(&hist[kk.y >> 21], 1u);
+                    atomicAdd(&hist[kk.z >> 21], 1u);
+                    atomicAdd(&hist[kk.w >> 21], 1u);
                 }
             }
         }
-        for (int i = (n4 << 2) + tid; i < nvalid; i += TOPK_THREADS) keys_lds[i] = score_key(row[i]);
+        for (int i = (n4 << 2) + tid; i < nvalid; i += TOPK_THREADS) {
+            const uint32_t key = score_key(row[i]);
+            keys_lds[i] = key;
+            atomicAdd(&hist[key >> 21], 1u);
+        }
     }
     auto key_at = [&](int i) -> uint32_t { return cached ? keys_lds[i] : score_key(row[i]); };
 
     uint32_t prefix = 0u, pmask = 0u, remaining = (uint32_t)K;
-    for (int pass = 0; pass < 4; ++pass) {
-        const int shift = 24 - 8 * pass;
-        hist[tid] = 0u;
-        __syncthreads();
-        // eight keys per thread in flight (rows that are not cached come from memory on every sweep)
-        for (int base = tid; base < nvalid; base += 8 * TOPK_THREADS) {
-            uint32_t kk[8];
+    for (int pass = 0; pass < 3; ++pass) {
+        const int shift = pass == 0 ? 21 : (pass == 1 ? 10 : 0);
+        const uint32_t dmask = pass == 2 ? 1023u : 2047u;
+        const int per = pass == 2 ? 4 : 8;              // consecutive digits per thread
+        if (pass > 0 || !cached) {
+            if (pass > 0) {
+                for (int i = tid; i < TOPK_BINS; i += TOPK_THREADS) hist[i] = 0u;
+                __syncthreads();
+            }
+            // eight keys per thread in flight (rows that are not cached come from memory on every sweep)
+            for (int base = tid; base < nvalid; base += 8 * TOPK_THREADS) {
+                uint32_t kk[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) kk[u] = key_at(min(base + u * TOPK_THREADS, nvalid - 1));
+                for (int u = 0; u < 8; ++u) kk[u] = key_at(min(base + u * TOPK_THREADS, nvalid - 1));
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (base + u * TOPK_THREADS < nvalid && (kk[u] & pmask) == prefix) atomicAdd(&hist[(kk[u] >> shift) & 255u], 1u);
+                for (int u = 0; u < 8; ++u)
+                    if (base + u * TOPK_THREADS < nvalid && (kk[u] & pmask) == prefix) atomicAdd(&hist[(kk[u] >> shift) & dmask], 1u);
+            }
         }
         __syncthreads();
-        // inclusive suffix sum over the 256 digits (digit 255 first)
-        uint32_t h = hist[tid], v = h;
+        // thread tid owns the digits [per*tid, per*tid + per); inclusive suffix sum over threads (largest digits first)
+        uint32_t own[8], h = 0u;
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            own[b] = b < per ? hist[per * tid + b] : 0u;
+            h += own[b];
+        }
+        uint32_t v = h;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
             uint32_t u = __shfl_down(v, off, 64);
@@ -94,14 +118,22 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
         if (lane == 0) wave_tot[wv] = v;
         __syncthreads();
         for (int w2 = wv + 1; w2 < 4; ++w2) v += wave_tot[w2];
-        const uint32_t excl = v - h;                    // keys with a larger digit
-        if (excl < remaining && remaining <= v) {       // exactly one digit satisfies this
-            sel_digit = (uint32_t)tid;
-            sel_remaining = remaining - excl;
+        uint32_t above = v - h;                         // keys with a digit beyond this thread's
+        if (above < remaining && remaining <= v) {      // exactly one thread satisfies this; walk its digits from the top
+#pragma unroll
+            for (int b = 7; b >= 0; --b) {
+                if (b < per && above < remaining) {
+                    if (remaining <= above + own[b]) {
+                        sel_digit = (uint32_t)(per * tid + b);
+                        sel_remaining = remaining - above;
+                    }
+                    above += own[b];
+                }
+            }
         }
         __syncthreads();
         prefix |= sel_digit << shift;
-        pmask |= 255u << shift;
+        pmask |= dmask << shift;
         remaining = sel_remaining;
         __syncthreads();
     }
