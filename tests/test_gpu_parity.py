@@ -239,6 +239,26 @@ def test_non_causal_packed_attention_for_the_vision_towers():
                             indexer_w=torch.zeros(T, 2, device=DEV), top_k=8)
 
 
+def test_call_from_a_compiled_block():
+    """The reference compiles every decoder block (train/infra.py:236-248); the operator must then run as an
+    opaque call inside the compiled function (the reference wraps its own in @torch.compiler.disable,
+    models/qwen3_5/model.py:90-91)."""
+    _log("compiled caller")
+    import vlm_training_amd as M
+    g = torch.Generator().manual_seed(33)
+    cu = torch.tensor([0, 100, 356], dtype=torch.int32, device=DEV)
+    q = (torch.randn(356, 4, 128, generator=g) * 0.5).bfloat16().to(DEV)
+    k = (torch.randn(356, 2, 128, generator=g) * 0.5).bfloat16().to(DEV)
+    v = (torch.randn(356, 2, 128, generator=g) * 0.5).bfloat16().to(DEV)
+
+    def block(q, k, v):
+        return M.dispatch_varlen_attention(q * 1.0, k, v, cu, 256) + 1.0
+
+    want = block(q, k, v)
+    got = torch.compile(block, backend="eager")(q, k, v)
+    assert torch.equal(got, want)
+
+
 def test_topk_at_least_longest_segment_is_dense():
     _log("K >= L")
     w = W.scaled(W.C2, (300, 120, 77), top_k=512, name="C2-dense")

@@ -260,6 +260,7 @@ class _DsaVarlenAttn(torch.autograd.Function):
         return dq, dk, dv, None, None, None, None, None, None
 
 
+@torch.compiler.disable                                  # a compiled caller (the reference compiles per block) breaks the graph here
 def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, indexer_q=None, indexer_k=None, indexer_w=None,
                     top_k: Optional[int] = None, index_scale: Optional[float] = None,
                     softmax_scale: Optional[float] = None, return_indices: bool = False, causal: bool = True):

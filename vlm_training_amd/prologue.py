@@ -85,6 +85,7 @@ class _QkNormRope(torch.autograd.Function):
         return dq, dk, dqw.to(qw_dtype), dkw.to(kw_dtype), None, None, None, None
 
 
+@torch.compiler.disable
 def qk_norm_rope(q, k, q_weight, k_weight, cos, sin, eps: float = 1e-6, offset: bool = False):
     """q (T, Hq, D), k (T, Hkv, D) bf16 views -> rope(rms_norm(q)), rope(rms_norm(k)) as contiguous (T, H, D).
 
@@ -121,6 +122,7 @@ class _SigmoidGate(torch.autograd.Function):
         return dx, dgate
 
 
+@torch.compiler.disable
 def sigmoid_gate(x, gate):
     """``x * torch.sigmoid(gate)`` for x (T, H, D) contiguous and gate a (T, H, D) view (strided allowed)."""
     return _SigmoidGate.apply(x, gate)
