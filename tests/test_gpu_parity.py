@@ -336,7 +336,7 @@ def test_reference_named_entry_points():
     assert_close_bf16(a, ref, "dispatch_varlen_attention")
 
 
-def test_argument_errors_cross_the_boundary_as_exceptions():
+def test_argument_errors_cross_the_boundary_as_exceptions(monkeypatch):
     q = torch.zeros(8, 4, 64, dtype=torch.bfloat16, device=DEV)
     k = torch.zeros(8, 3, 64, dtype=torch.bfloat16, device=DEV)
     cu = torch.tensor([0, 8], dtype=torch.int32, device=DEV)
@@ -354,6 +354,12 @@ def test_argument_errors_cross_the_boundary_as_exceptions():
         ops.dsa_varlen_attn(big, big, big, cu, 8)
     with pytest.raises(RuntimeError):
         ops.dsa_varlen_attn(q.cpu(), k.cpu(), k.cpu(), cu.cpu(), 8)
+    monkeypatch.setenv("DSA_DEBUG_NAN", "1")
+    qi = torch.zeros(8, 2, 32, dtype=torch.bfloat16, device=DEV)
+    qi[3, 1, 5] = float("nan")
+    with pytest.raises(ValueError):
+        ops.index_topk(qi, torch.zeros(8, 32, dtype=torch.bfloat16, device=DEV),
+                       torch.zeros(8, 2, dtype=torch.bfloat16, device=DEV), cu, 8, 2)
 
 
 # ------------------------------------------------------------------------------------------ golden fixtures

@@ -8,6 +8,8 @@ torch is used for device memory and streams only; all arithmetic runs in the HIP
 """
 from __future__ import annotations
 
+import os
+
 from typing import Optional, Tuple
 
 import torch
@@ -115,6 +117,11 @@ def index_topk(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen: int, top_k: int,
     ws_bytes = lib.dsa_index_topk_workspace_bytes(T, max_seqlen, top_k) if max_seqlen > top_k else 0
     ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q_idx.device)
     qi, ki, wi = _as_bf16(q_idx), _as_bf16(k_idx), _as_bf16(w_idx)     # keep the casts alive over the launch
+    if os.environ.get("DSA_DEBUG_NAN"):
+        # the device ranks NaN above +inf without a word; with this switch (one device-to-host copy) it is an error,
+        # as it is in the CPU restatement of the selection
+        if not (torch.isfinite(qi.float()).all() and torch.isfinite(ki.float()).all() and torch.isfinite(wi.float()).all()):
+            raise ValueError("non-finite indexer inputs: their scores have no defined rank")
     rc = lib.dsa_index_topk(_ptr(qi), _ptr(ki), _ptr(wi), _ptr(cu), T,
                             cu.numel() - 1, Hi, Di, top_k, scale, _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(idx), _ptr(n),
                             _ptr(ws), ws_bytes, _stream(q_idx.device))
