@@ -92,6 +92,19 @@ int dsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx
 size_t dsa_attn_fwd_workspace_bytes(int T, int max_seqlen, int has_idx);
 
 /*
+ * Attention mass of the selected keys: mass[t*K + j] = 1/Hq * sum over query heads of the softmax
+ * probability that D3 gave key idx[t*K + j] (lse is D3's output), 0 for j >= n[t].  Every head's softmax
+ * over sel(t) sums to one, so a row sums to one: it is the target distribution of the KL loss that
+ * trains a DSA indexer (the selection itself passes no gradient).  No reference counterpart - the
+ * reference holds no indexer; it would be called beside the attention call of a layer in its training
+ * step (train/train_qwen.py:534-548).  fp32 out, deterministic.  ws: dsa_attn_mass_workspace_bytes().
+ */
+int dsa_attn_mass(const void *q, const void *k, const float *lse, const int32_t *idx, const int32_t *n,
+                  const int32_t *cu_seqlens, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
+                  int dtype, int max_seqlen, float *mass, void *ws, size_t ws_bytes, void *stream);
+size_t dsa_attn_mass_workspace_bytes(int T, int Hkv, int K, int max_seqlen);
+
+/*
  * Tuning knob (process-wide, no reference counterpart): query rows whose position in their segment is
  * below top_k * crossover run on the dense MFMA tile kernels with the selection as a bitmap mask, the
  * rest on the gather kernels.  Default 16; 0 = gather only; INT_MAX/top_k or more = tiles only.

@@ -24,6 +24,8 @@ Pinning status (what independent check fixes each function; see tests/test_oracl
   adversarial tie patterns (all equal, +-0.0, duplicates straddling the K-th place).
 * ``sparse_attention``       - pure-Python loop over selected keys; with K >= longest segment it
   must equal ``dense_varlen_causal``; gradients by ``torch.autograd.gradcheck`` in fp64.
+* ``attention_mass``         - pure-Python loop on a tiny case; rows sum to one; with one kv head the
+  mass-weighted sum of the selected value rows equals the head mean of ``sparse_attention``'s output.
 
 The reference holds no golden vector for this path (its tests compare whole-model logits with
 HuggingFace weights that are not in the tree), so the torch==2.11 ``varlen_attn`` boundary itself
@@ -230,6 +232,38 @@ def sparse_attention(q, k, v, idx, n, cu_seqlens, softmax_scale: Optional[float]
     if return_lse:
         return out, (torch.cat(lses, dim=1) if lses else qf.new_zeros(Hq, 0))
     return out
+
+
+def attention_mass(q, k, idx, n, cu_seqlens, softmax_scale: Optional[float] = None, chunk: int = 256):
+    """Target distribution of the indexer's training loss: the attention probability of every selected key,
+    averaged over the query heads,
+
+        mass[t,j] = 1/Hq * sum_h softmax_{s in sel(t)}(q[t,h].k[s,h//G] * scale) at s = idx[t,j]   (0 where idx = -1).
+
+    Every head's softmax over sel(t) sums to one, so a row sums to one: the head sum needs no further
+    normalisation.  Written as a gather over ``idx`` (not as the masked dense product ``sparse_attention``
+    uses), so that the two restatements check each other: with one kv head,
+    ``sum_j mass[t,j] v[idx[t,j]]`` is the head mean of the attention output.
+    """
+    T, Hq, D = q.shape
+    Hkv = k.shape[1]
+    G = Hq // Hkv
+    scale = softmax_scale if softmax_scale is not None else D ** -0.5
+    cdt = torch.float64 if q.dtype == torch.float64 else torch.float32
+    qf, kf = q.to(cdt), k.to(cdt)
+    K = idx.shape[1]
+    mass = torch.zeros(T, K, dtype=cdt)
+    for c0 in range(0, T, chunk):
+        c1 = min(T, c0 + chunk)
+        ok = idx[c0:c1] >= 0                                                    # (R,K)
+        rows = kf[idx[c0:c1].clamp(min=0).long()]                               # (R,K,Hkv,D)
+        rows = rows.repeat_interleave(G, dim=2)                                 # (R,K,Hq,D): head h reads kv head h//G
+        logits = torch.einsum("rhd,rkhd->rhk", qf[c0:c1], rows) * scale
+        logits = logits.masked_fill(~ok[:, None, :], float("-inf"))
+        p = torch.softmax(logits, dim=-1)
+        p = torch.where(ok[:, None, :], p, torch.zeros((), dtype=cdt))          # rows without any key stay zero
+        mass[c0:c1] = p.mean(dim=1)
+    return mass
 
 
 def dsa_varlen_attn_ref(q, k, v, cu_seqlens, q_idx, k_idx, w, top_k: int,

@@ -537,3 +537,30 @@ def test_dense_c_abi_entry_points_equal_the_general_ones():
     torch.cuda.synchronize()
     for a, b in ((out, out0), (lse, lse0), (dq, dq0), (dk, dk0), (dv, dv0)):
         assert torch.equal(a, b)
+
+
+# ------------------------------------------------------------------------------------------ indexer training target
+@pytest.mark.parametrize("Hq,Hkv,D,K,segs", [(8, 2, 128, 64, (300, 1, 77, 513)), (32, 8, 128, 256, (1024, 700)),
+                                              (6, 2, 64, 16, (130, 64, 5)), (16, 2, 256, 128, (600, 257)),
+                                              (16, 1, 128, 32, (200, 90)), (5, 1, 128, 8, (97,)), (3, 3, 64, 100, (50, 400))])
+def test_attention_mass_matches_the_oracle(Hq, Hkv, D, K, segs):
+    """Target of the indexer's KL loss: head mean of the probabilities the forward gave the selected keys.
+    Tolerance: |err| <= 2e-3 absolute on probabilities in [0,1] (bf16 inputs, fp32 exponentials against the
+    forward's own lse) and rows summing to one within 2e-3."""
+    _log(f"mass {Hq}/{Hkv}/{D} K={K}")
+    w = W.Workload("mass", torch.bfloat16, segs, Hq, Hkv, D, 4, 32, K, 0.5, 77)
+    t = W.make_inputs(w, device="cpu")
+    d = {k_: (v_.to(DEV) if torch.is_tensor(v_) else v_) for k_, v_ in t.items()}
+    scale = D ** -0.5
+    idx, n = ops.index_topk(d["q_idx"], d["k_idx"], d["w_idx"], d["cu_seqlens"], w.max_seqlen, K)
+    out, lse = ops.attn_fwd(d["q"], d["k"], d["v"], idx, n, d["cu_seqlens"], w.max_seqlen, scale)
+    mass = ops.attn_mass(d["q"], d["k"], lse, idx, n, d["cu_seqlens"], w.max_seqlen, scale)
+    assert mass.shape == (w.T, K) and mass.dtype == torch.float32
+    want = R.attention_mass(t["q"].float(), t["k"].float(), idx.cpu(), n.cpu(), list(w.cu), scale)
+    err = (mass.cpu() - want).abs().max().item()
+    assert err <= 2e-3, err
+    assert (mass.sum(1).cpu() - 1.0).abs().max().item() <= 2e-3
+    pad = torch.arange(K, device=DEV)[None, :] >= n[:, None]
+    assert float(mass[pad].abs().sum()) == 0.0
+    again = ops.attn_mass(d["q"], d["k"], lse, idx, n, d["cu_seqlens"], w.max_seqlen, scale)
+    assert torch.equal(mass, again)                       # fixed summation order: bit-identical from run to run

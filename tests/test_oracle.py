@@ -353,3 +353,35 @@ def test_pack_lengths_follows_the_reference_collate_convention():
     w = W.random_packed_workload(W.C2, 8192, seed=3)
     assert w.T == 8192 and w.cu[-1] == 8192 and min(w.seg_lens) >= 1
     assert W.random_packed_workload(W.C2, 8192, seed=3).seg_lens == w.seg_lens
+
+
+# ---------------------------------------------------------------- indexer training target (attention mass)
+def test_attention_mass_against_a_python_loop_and_the_attention_output():
+    cu = [0, 7, 7, 19]
+    T, Hq, Hkv, D, K = 19, 4, 2, 8, 5
+    q, k, v = rnd(T, Hq, D, seed=41), rnd(T, Hkv, D, seed=42), rnd(T, Hkv, D, seed=43)
+    qi, ki, w = rnd(T, 2, 4, seed=44), rnd(T, 4, seed=45), rnd(T, 2, seed=46)
+    idx, n = R.dsa_select(qi, ki, w, cu, K)
+    mass = R.attention_mass(q, k, idx, n, cu)
+    assert mass.shape == (T, K)
+    # pure-Python restatement
+    G, scale = Hq // Hkv, 1.0 / math.sqrt(D)
+    for t in range(T):
+        sel = [int(s) for s in idx[t, : int(n[t])]]
+        want = [0.0] * len(sel)
+        for h in range(Hq):
+            logits = [float(torch.dot(q[t, h].double(), k[s, h // G].double())) * scale for s in sel]
+            m = max(logits)
+            e = [math.exp(x - m) for x in logits]
+            z = sum(e)
+            for j in range(len(sel)):
+                want[j] += e[j] / z / Hq
+        assert torch.allclose(mass[t, : len(sel)].double(), torch.tensor(want, dtype=torch.float64), atol=1e-6)
+        assert float(mass[t, len(sel):].abs().sum()) == 0.0
+        assert abs(float(mass[t].sum()) - 1.0) < 1e-5      # every head's softmax over sel(t) sums to one
+    # one kv head: the mass-weighted sum of the selected value rows is the head mean of the attention output
+    k1, v1 = rnd(T, 1, D, seed=47), rnd(T, 1, D, seed=48)
+    out = R.sparse_attention(q, k1, v1, idx, n, cu)                      # (T,Hq,D), the pinned D3 restatement
+    m1 = R.attention_mass(q, k1, idx, n, cu)
+    rows = v1[idx.clamp(min=0).long(), 0]                                # (T,K,D)
+    assert torch.allclose((m1[..., None] * rows).sum(1), out.mean(1), atol=1e-5)

@@ -22,6 +22,9 @@ hipError_t dsa_launch_gather_dq(const void *dout, const void *q, const void *k, 
                                 const float *delta, const int32_t *idx, const int32_t *n, const int32_t *cu, int N,
                                 int T, int Hq, int Hkv, int D, int K, float scale, int pos_min, void *dq,
                                 hipStream_t stream);
+hipError_t dsa_launch_tile_mass(const void *q, const void *k, const float *lse, const uint32_t *bitmap, int ldw,
+                                const int32_t *n, const int32_t *cu, int N, int T, int Hq, int Hkv, int D, int K,
+                                float scale, float *partial, float *mass, hipStream_t stream);
 hipError_t dsa_launch_tile_fwd(const void *q, const void *k, const void *v, const uint32_t *bitmap, int ldw,
                                const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale, int pos_split,
                                int causal, void *out, float *lse, hipStream_t stream);
@@ -207,6 +210,33 @@ extern "C" int dsa_attn_fwd(const void *q, const void *k, const void *v, const i
         e = dsa_launch_attn_fwd(q, k, v, idx, n, cu, N, T, Hq, Hkv, D, K, softmax_scale, split, out, lse, st);
         if (e != hipSuccess) return hip_fail(e, "gather forward launch");
     }
+    return DSA_OK;
+}
+
+// ---- attention mass of the selected keys (training target of the indexer) ---------------------------
+extern "C" size_t dsa_attn_mass_workspace_bytes(int T, int Hkv, int K, int max_seqlen) {
+    if (T <= 0 || Hkv <= 0 || K <= 0) return 0;
+    return align_up((size_t)T * bitmap_ldw(max_seqlen) * 4, 256) + align_up((size_t)Hkv * T * K * 4, 256);
+}
+
+extern "C" int dsa_attn_mass(const void *q, const void *k, const float *lse, const int32_t *idx, const int32_t *n,
+                             const int32_t *cu, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
+                             int dtype, int max_seqlen, float *mass, void *ws, size_t ws_bytes, void *stream) {
+    if (int rc = check_attn(T, N, cu, Hq, Hkv, D, K, dtype, idx, n)) return rc;
+    if (!q || !k || !lse || !idx || !n || !mass) return fail(DSA_ERR_ARG, "null tensor pointer");
+    if (max_seqlen < 1 || max_seqlen > (T > 0 ? T : 1)) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
+    if (T == 0) return DSA_OK;
+    const size_t need = dsa_attn_mass_workspace_bytes(T, Hkv, K, max_seqlen);
+    if (!ws || ws_bytes < need) return fail(DSA_ERR_WORKSPACE, "mass workspace: have %zu bytes, need %zu", ws_bytes, need);
+    const int ldw = bitmap_ldw(max_seqlen);
+    if ((size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);
+    hipStream_t st = (hipStream_t)stream;
+    uint32_t *bitmap = (uint32_t *)ws;
+    float *partial = (float *)((char *)ws + align_up((size_t)T * ldw * 4, 256));
+    hipError_t e = dsa_launch_bitmap(idx, n, cu, N, T, K, ldw, bitmap, st);
+    if (e != hipSuccess) return hip_fail(e, "bitmap launch");
+    e = dsa_launch_tile_mass(q, k, lse, bitmap, ldw, n, cu, N, T, Hq, Hkv, D, K, softmax_scale, partial, mass, st);
+    if (e != hipSuccess) return hip_fail(e, "attention mass launch");
     return DSA_OK;
 }
 

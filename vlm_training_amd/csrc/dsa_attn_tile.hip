@@ -305,6 +305,119 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
 }
 
 // ==================================================================================================
+// attention mass: the indexer's training target.  Same walk and S^T = K Q^T as the forward, with the
+// saved log-sum-exp instead of the online softmax and no V: P = exp(S*scale - lse) on the selected
+// keys, summed over the heads of a query that share the kv head (lanes of one query are adjacent:
+// DPP adds), and written to the slot the key has in the query's ascending selection list
+// (slot = selected keys of earlier tiles + selected keys below it in the tile's word).  One partial
+// (T,K) table per kv head; dsa_mass_reduce_kernel adds them in a fixed order.
+// ==================================================================================================
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, false));
+}
+// sum over the aligned group of 2^GSHIFT adjacent lanes, on every lane of the group
+template <int GSHIFT>
+__device__ __forceinline__ float group_sum(float x) {
+    if (GSHIFT >= 1) x += dpp_f<0xB1>(x);               // quad_perm [1,0,3,2]
+    if (GSHIFT >= 2) x += dpp_f<0x4E>(x);               // quad_perm [2,3,0,1]
+    if (GSHIFT >= 3) x += dpp_f<0x141>(x);              // row_half_mirror: the other quad's total
+    if (GSHIFT >= 4) x += dpp_f<0x140>(x);              // row_mirror: the other half row's total
+    return x;
+}
+template <int D, int GSHIFT, int NW>
+__global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_tile_mass_kernel(
+    const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const float *__restrict__ lse,
+    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
+    float scale_log2, int K, float *__restrict__ partial) {
+    constexpr int KS = D / 16, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / (NW * 64);
+    constexpr int NBUF = 2, NT = NW * 64, Gp = 1 << GSHIFT, QBW = (NW * 32) >> GSHIFT;
+    static_assert(LOADS >= 1, "tile must give every thread a chunk");
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][TILE_B];
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
+    LaneOffsets<D> lo;
+    lo.init(lane);
+    const int G = Hq / Hkv;
+    const int kvh = blockIdx.x % Hkv;
+    int s0, L, blk;
+    if (!locate_block(cu, N, blockIdx.x / Hkv, QBW, true, s0, L, blk)) return;
+    const int qc0 = blk * QBW;
+
+    const int r = wv * 32 + j;
+    const int qcol = qc0 + (r >> GSHIFT), head = r & (Gp - 1);
+    const bool row_ok = qcol < L && head < G;
+    const int t = s0 + min(qcol, L - 1), hq = kvh * G + min(head, G - 1);
+    u32x4 kst[2][LOADS];
+#define MASS_LOAD(SET, TILE)                                                                        \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+        const int c = i * NT + tid;                                                                \
+        const int row = c / CPR, ch = c % CPR;                                                     \
+        kst[SET][i] = *reinterpret_cast<const u32x4 *>(                                            \
+            k + ((int64_t)(s0 + min((TILE) * 32 + row, L - 1)) * Hkv + kvh) * D + ch * 8);         \
+    }
+    MASS_LOAD(0, 0)
+    bf16x8 qB[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+        qB[ks] = row_ok ? load_bf16x8(q + ((int64_t)t * Hq + hq) * D + 16 * ks + 8 * h) : zero_bf16x8();
+    const float lse2 = lse[(int64_t)hq * T + t] * LOG2E_F;
+    const int ntiles = min(qc0 + QBW - 1, L - 1) / 32 + 1;
+    const uint32_t *wrow = bitmap + (int64_t)t * ldw;
+    uint32_t word_next = wrow[0];
+    int seen = 0;                                        // selected keys of this row in the tiles already walked
+    float *prow = partial + ((int64_t)kvh * T + t) * K;
+
+#define MASS_STORE(SET, BUF, TILE)                                                                  \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+        const int c = i * NT + tid;                                                                \
+        const int row = c / CPR, ch = c % CPR;                                                     \
+        *reinterpret_cast<u32x4 *>(&lds[BUF][tile_off<D>(row, ch)]) = kst[SET][i];                 \
+    }
+#define MASS_COMPUTE(TILE, BUF)                                                                     \
+    {                                                                                              \
+        const unsigned char *kt = lds[BUF];                                                        \
+        const uint32_t word_full = row_ok ? word_next : 0u;                                        \
+        word_next = wrow[min((TILE) + 1, ntiles - 1)];                                             \
+        const uint32_t word = word_full >> (4 * h);      /* element vi then sits at bit 8*(vi/4) + vi%4 */ \
+        f32x16 sacc = zero16();                                                                    \
+        {                                                                                          \
+            bf16x8 ka[KS];                                                                         \
+            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) ka[ks] = lo.rowop(kt, ks);           \
+            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) sacc = mfma32(ka[ks], qB[ks], sacc); \
+            sched_reads_ahead<KS, 4, 1>();                                                         \
+        }                                                                                          \
+        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
+            const int kb = 8 * (vi >> 2) + (vi & 3);                                               \
+            float p = fast_exp2(keep_or_neginf(fmaf(sacc[vi], scale_log2, -lse2), bit_mask(word, kb))); \
+            p = group_sum<GSHIFT>(p);                                                              \
+            const int bit = kb + 4 * h;                  /* the key's column in the tile */         \
+            if (head == 0 && ((word_full >> bit) & 1u))                                            \
+                prow[seen + __popc(word_full & ((1u << bit) - 1u))] = p;                           \
+        }                                                                                          \
+        seen += __popc(word_full);                                                                 \
+    }
+    TILE_PIPELINE(ntiles, MASS_LOAD, MASS_STORE, MASS_COMPUTE)
+#undef MASS_LOAD
+#undef MASS_STORE
+#undef MASS_COMPUTE
+}
+
+// mass[t,j] = inv_hq * sum over kv heads of partial[kvh][t][j] for j < n[t], else 0
+__global__ __launch_bounds__(256) void dsa_mass_reduce_kernel(const float *__restrict__ partial,
+                                                               const int32_t *__restrict__ nsel, int T, int K, int Hkv,
+                                                               float inv_hq, float *__restrict__ mass) {
+    const int64_t total = (int64_t)T * K;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int t = (int)(i / K), jj = (int)(i % K);
+        float acc = 0.f;
+        if (jj < nsel[t])
+            for (int kvh = 0; kvh < Hkv; ++kvh) acc += partial[(int64_t)kvh * total + i];
+        mass[i] = acc * inv_hq;
+    }
+}
+
+// ==================================================================================================
 // dQ: query-stationary, same walk as the forward.
 //   S^T = K Q^T, dP^T = V dO^T  (A = K / V tiles row-wise, B = Q^T / dO^T in registers)
 //   dS^T = P^T * (dP^T - delta)  on the C layout
@@ -878,6 +991,27 @@ extern "C" hipError_t dsa_launch_tile_fwd(const void *q, const void *k, const vo
     const int gs = group_shift(Hq, Hkv);
     const dim3 grid((unsigned)(((int64_t)T / ((32 * tile_waves_of(D)) >> gs) + N + 1) * Hkv));
     TILE_SWITCH(launch_fwd_i, grid, stream, q, k, v, bitmap, ldw, cu, N, T, Hq, Hkv, scale * LOG2E_F, pos_split, causal, out, lse)
+    return hipGetLastError();
+}
+template <int D, bool HAS_IDX, int GS>
+static void launch_mass_i(dim3 grid, hipStream_t stream, const void *q, const void *k, const float *lse,
+                          const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T, int Hq, int Hkv, float sl2,
+                          int K, float *partial) {
+    hipLaunchKernelGGL((dsa_tile_mass_kernel<D, GS, tile_waves<D>()>), grid, dim3(64 * tile_waves<D>()), 0, stream,
+                       (const bf16_t *)q, (const bf16_t *)k, lse, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, K, partial);
+}
+// attention mass of the selected keys: partial (Hkv,T,K) tables, then their sum scaled by 1/Hq into mass (T,K)
+extern "C" hipError_t dsa_launch_tile_mass(const void *q, const void *k, const float *lse, const uint32_t *bitmap,
+                                           int ldw, const int32_t *n, const int32_t *cu, int N, int T, int Hq, int Hkv,
+                                           int D, int K, float scale, float *partial, float *mass, hipStream_t stream) {
+    const int gs = group_shift(Hq, Hkv);
+    const dim3 grid((unsigned)(((int64_t)T / ((32 * tile_waves_of(D)) >> gs) + N + 1) * Hkv));
+    TILE_SWITCH(launch_mass_i, grid, stream, q, k, lse, bitmap, ldw, cu, N, T, Hq, Hkv, scale * LOG2E_F, K, partial)
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const int64_t total = (int64_t)T * K;
+    const unsigned blocks = (unsigned)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
+    hipLaunchKernelGGL(dsa_mass_reduce_kernel, dim3(blocks), dim3(256), 0, stream, partial, n, T, K, Hkv, 1.f / (float)Hq, mass);
     return hipGetLastError();
 }
 extern "C" hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const void *k, const void *v,

@@ -159,6 +159,30 @@ def attn_fwd(q, k, v, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float,
     return out, lse
 
 
+def attn_mass(q, k, lse, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: Optional[float] = None) -> torch.Tensor:
+    """Head-averaged attention probability of every selected key, (T, K) fp32, rows summing to one: the target
+    of the KL loss that trains the indexer.  ``lse`` (Hq, T) is the forward's second output for the same
+    q, k, idx.  Nothing here is differentiable (the target is detached in DSA's objective)."""
+    _require_cuda(q, k, lse, idx, n, cu_seqlens)
+    T, Hq, D = q.shape
+    Hkv, K = k.shape[1], idx.shape[1]
+    cu = _check_cu(cu_seqlens, T)
+    if lse.shape != (Hq, T) or lse.dtype != torch.float32 or idx.shape[0] != T or n.shape != (T,):
+        raise ValueError("lse must be (Hq,T) fp32, idx (T,K) int32, n (T,) int32")
+    scale = float(softmax_scale) if softmax_scale is not None else D ** -0.5
+    max_seqlen = T if max_seqlen is None else int(max_seqlen)
+    lib = _lib.load()
+    qb, kb = _as_bf16(q), _as_bf16(k)
+    mass = torch.empty((T, K), dtype=torch.float32, device=q.device)
+    ws_bytes = lib.dsa_attn_mass_workspace_bytes(T, Hkv, K, max_seqlen)
+    ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q.device)
+    rc = lib.dsa_attn_mass(_ptr(qb), _ptr(kb), _ptr(lse.contiguous()), _ptr(idx), _ptr(n), _ptr(cu), T, cu.numel() - 1, Hq,
+                           Hkv, D, K, scale, _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(mass), _ptr(ws), ws_bytes,
+                           _stream(q.device))
+    _lib.check(rc, "dsa_attn_mass")
+    return mass
+
+
 def attn_bwd(dout, q, k, v, out, lse, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float,
              parts: int = 15, buffers=None, causal: bool = True):
     """Stage D4.  ``parts``/``buffers`` exist for per-kernel timing: ``buffers=(dq, dk, dv, ws)`` reuses
