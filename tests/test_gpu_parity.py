@@ -542,7 +542,8 @@ def test_dense_c_abi_entry_points_equal_the_general_ones():
 # ------------------------------------------------------------------------------------------ indexer training target
 @pytest.mark.parametrize("Hq,Hkv,D,K,segs", [(8, 2, 128, 64, (300, 1, 77, 513)), (32, 8, 128, 256, (1024, 700)),
                                               (6, 2, 64, 16, (130, 64, 5)), (16, 2, 256, 128, (600, 257)),
-                                              (16, 1, 128, 32, (200, 90)), (5, 1, 128, 8, (97,)), (3, 3, 64, 100, (50, 400))])
+                                              (16, 1, 128, 32, (200, 90)), (5, 1, 128, 8, (97,)), (3, 3, 64, 100, (50, 400)),
+                                              (2, 1, 64, 5, (40, 3)), (12, 4, 128, 2048, (2500,))])
 def test_attention_mass_matches_the_oracle(Hq, Hkv, D, K, segs):
     """Target of the indexer's KL loss: head mean of the probabilities the forward gave the selected keys.
     Tolerance: |err| <= 2e-3 absolute on probabilities in [0,1] (bf16 inputs, fp32 exponentials against the

@@ -377,9 +377,10 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
 #define MASS_COMPUTE(TILE, BUF)                                                                     \
     {                                                                                              \
         const unsigned char *kt = lds[BUF];                                                        \
-        const uint32_t word_full = row_ok ? word_next : 0u;                                        \
+        /* padding lanes of a query (head >= G) compute nothing but take their share of the stores */ \
+        const uint32_t word_full = qcol < L ? word_next : 0u;                                      \
         word_next = wrow[min((TILE) + 1, ntiles - 1)];                                             \
-        const uint32_t word = word_full >> (4 * h);      /* element vi then sits at bit 8*(vi/4) + vi%4 */ \
+        const uint32_t word = (row_ok ? word_full : 0u) >> (4 * h); /* element vi then sits at bit 8*(vi/4) + vi%4 */ \
         f32x16 sacc = zero16();                                                                    \
         {                                                                                          \
             bf16x8 ka[KS];                                                                         \
@@ -387,13 +388,19 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
             _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) sacc = mfma32(ka[ks], qB[ks], sacc); \
             sched_reads_ahead<KS, 4, 1>();                                                         \
         }                                                                                          \
+        float p[16];                                                                               \
         _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
             const int kb = 8 * (vi >> 2) + (vi & 3);                                               \
-            float p = fast_exp2(keep_or_neginf(fmaf(sacc[vi], scale_log2, -lse2), bit_mask(word, kb))); \
-            p = group_sum<GSHIFT>(p);                                                              \
-            const int bit = kb + 4 * h;                  /* the key's column in the tile */         \
-            if (head == 0 && ((word_full >> bit) & 1u))                                            \
-                prow[seen + __popc(word_full & ((1u << bit) - 1u))] = p;                           \
+            p[vi] = fast_exp2(keep_or_neginf(fmaf(sacc[vi], scale_log2, -lse2), bit_mask(word, kb))); \
+        }                                                                                          \
+        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) p[vi] = group_sum<GSHIFT>(p[vi]);        \
+        /* the lanes of a query share the stores: lane `head` writes the elements vi = u*Gp + head */ \
+        _Pragma("unroll") for (int u = 0; u < 16 / Gp; ++u) {                                      \
+            float val = p[u * Gp];                                                                 \
+            _Pragma("unroll") for (int g = 1; g < Gp; ++g) val = head == g ? p[u * Gp + g] : val;  \
+            const int vi = u * Gp + head;                                                          \
+            const int bit = 8 * (vi >> 2) + (vi & 3) + 4 * h;    /* the key's column in the tile */ \
+            if ((word_full >> bit) & 1u) prow[seen + __popc(word_full & ((1u << bit) - 1u))] = val; \
         }                                                                                          \
         seen += __popc(word_full);                                                                 \
     }
@@ -403,17 +410,35 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
 #undef MASS_COMPUTE
 }
 
-// mass[t,j] = inv_hq * sum over kv heads of partial[kvh][t][j] for j < n[t], else 0
+// mass[t,j] = inv_hq * sum over kv heads of partial[kvh][t][j] for j < n[t], else 0.  One workgroup per query row
+// and blockIdx.y-th part of it, four columns per thread (16-byte accesses when K is a multiple of four).
 __global__ __launch_bounds__(256) void dsa_mass_reduce_kernel(const float *__restrict__ partial,
                                                                const int32_t *__restrict__ nsel, int T, int K, int Hkv,
                                                                float inv_hq, float *__restrict__ mass) {
-    const int64_t total = (int64_t)T * K;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-        const int t = (int)(i / K), jj = (int)(i % K);
-        float acc = 0.f;
-        if (jj < nsel[t])
-            for (int kvh = 0; kvh < Hkv; ++kvh) acc += partial[(int64_t)kvh * total + i];
-        mass[i] = acc * inv_hq;
+    const int t = blockIdx.x, nt = nsel[t];
+    const int64_t row = (int64_t)t * K, plane = (int64_t)T * K;
+    if ((K & 3) == 0) {
+        for (int j4 = blockIdx.y * 256 + threadIdx.x; j4 < (K >> 2); j4 += gridDim.y * 256) {
+            float4 acc = {0.f, 0.f, 0.f, 0.f};
+            if (4 * j4 < nt)
+                for (int kvh = 0; kvh < Hkv; ++kvh) {
+                    const float4 x = *reinterpret_cast<const float4 *>(partial + kvh * plane + row + 4 * j4);
+                    acc.x += x.x; acc.y += x.y; acc.z += x.z; acc.w += x.w;
+                }
+            // slots at and beyond n[t] were never written
+            acc.x = 4 * j4 < nt ? acc.x * inv_hq : 0.f;
+            acc.y = 4 * j4 + 1 < nt ? acc.y * inv_hq : 0.f;
+            acc.z = 4 * j4 + 2 < nt ? acc.z * inv_hq : 0.f;
+            acc.w = 4 * j4 + 3 < nt ? acc.w * inv_hq : 0.f;
+            *reinterpret_cast<float4 *>(mass + row + 4 * j4) = acc;
+        }
+    } else {
+        for (int jj = blockIdx.y * 256 + threadIdx.x; jj < K; jj += gridDim.y * 256) {
+            float acc = 0.f;
+            if (jj < nt)
+                for (int kvh = 0; kvh < Hkv; ++kvh) acc += partial[kvh * plane + row + jj];
+            mass[row + jj] = acc * inv_hq;
+        }
     }
 }
 
@@ -1009,9 +1034,9 @@ extern "C" hipError_t dsa_launch_tile_mass(const void *q, const void *k, const f
     TILE_SWITCH(launch_mass_i, grid, stream, q, k, lse, bitmap, ldw, cu, N, T, Hq, Hkv, scale * LOG2E_F, K, partial)
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const int64_t total = (int64_t)T * K;
-    const unsigned blocks = (unsigned)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
-    hipLaunchKernelGGL(dsa_mass_reduce_kernel, dim3(blocks), dim3(256), 0, stream, partial, n, T, K, Hkv, 1.f / (float)Hq, mass);
+    const unsigned parts = (unsigned)((K / 4 + 255) / 256 > 0 ? (K / 4 + 255) / 256 : 1);
+    hipLaunchKernelGGL(dsa_mass_reduce_kernel, dim3(T, parts < 8 ? parts : 8), dim3(256), 0, stream, partial, n, T, K, Hkv,
+                       1.f / (float)Hq, mass);
     return hipGetLastError();
 }
 extern "C" hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const void *k, const void *v,
