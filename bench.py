@@ -62,11 +62,27 @@ def cpu_baseline(w, threads):
     }
 
 
+def _eager_qk_norm_rope(q, k, qw, kw, cos, sin, eps=1e-6):
+    """The reference layer's own sequence of eager torch ops around the attention call, in bf16
+    (models/qwen3_vl/model.py:256-269: per-head F.rms_norm, transpose to (1,H,T,D), apply_rope = x*cos +
+    rotate_half(x)*sin, transpose back, .contiguous()) - timed beside the fused kernel, nothing else."""
+    import torch.nn.functional as F
+
+    def rope(x):                                         # x (1,H,T,D)
+        half = x.shape[-1] // 2
+        rot = torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+        return x * cos[None, None] + rot * sin[None, None]
+
+    qn = F.rms_norm(q, (q.shape[-1],), qw, eps).unsqueeze(0).transpose(1, 2)
+    kn = F.rms_norm(k, (k.shape[-1],), kw, eps).unsqueeze(0).transpose(1, 2)
+    qo, ko = rope(qn), rope(kn)
+    return (qo.transpose(1, 2).reshape(q.shape).contiguous(), ko.transpose(1, 2).reshape(k.shape).contiguous())
+
+
 def prologue_stage(w, dev, iters):
     """The fused element-wise kernels either side of the operator, at the workload's geometry: HBM-bound,
     so each is reported as algorithmic bytes / time against the 8 TB/s peak, beside the reference's own
     sequence of eager torch ops (F.rms_norm, transposes, apply_rope, contiguous copies) on the same GPU."""
-    from oracle import prologue_ref as P
     from vlm_training_amd import prologue
     T, Hq, Hkv, D = w.T, w.Hq, w.Hkv, w.D
     g = torch.Generator(device="cpu").manual_seed(w.seed)
@@ -90,7 +106,7 @@ def prologue_stage(w, dev, iters):
     with torch.no_grad():
         ms = timed(lambda: prologue.qk_norm_rope(q, k, qw, kw, cos, sin), iters)
         res["qk_norm_rope_fwd"] = entry(ms, T * (2 * rows + 2 * D * e + (Hq + Hkv) * 4))
-        eager = timed(lambda: P.qk_norm_rope(q, k, qw, kw, cos, sin, eager_bf16=True), iters)
+        eager = timed(lambda: _eager_qk_norm_rope(q, k, qw, kw, cos, sin), iters)
         res["qk_norm_rope_fwd"]["eager_torch_ms"] = eager
         ms = timed(lambda: prologue.sigmoid_gate(q, gate), iters)
         res["sigmoid_gate_fwd"] = entry(ms, T * Hq * D * e * 3)
@@ -121,6 +137,20 @@ def reference_operator(w, t, iters):
     ours = timed(lambda: run(lambda q, k, v: ops.dsa_varlen_attn(q, k, v, cu, msl)), iters)
     return {"what": "dense causal packed attention fwd+bwd on this workload (the operator the reference calls)",
             "torch_varlen_attn_ms": theirs, "this_library_dense_ms": ours, "speedup": theirs / ours}
+
+
+def indexer_target_stage(w, t, iters):
+    """Attention mass of the selected keys (the target of the KL loss that trains the indexer): one more pass
+    over the forward's S = QK^T with the saved log-sum-exp.  Matrix work 2*Hq*D flop per selected pair; the
+    per-kv-head partial tables it writes and adds up are 2 * Hkv * 4 bytes per selected pair of HBM traffic."""
+    from vlm_training_amd import ops
+    cu, msl, scale = t["cu_seqlens"], w.max_seqlen, w.D ** -0.5
+    idx, n = ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k)
+    out, lse = ops.attn_fwd(t["q"], t["k"], t["v"], idx, n, cu, msl, scale)
+    ms = timed(lambda: ops.attn_mass(t["q"], t["k"], lse, idx, n, cu, msl, scale), iters)
+    S = w.pair_counts()[1]
+    return {"ms": ms, "selected_pair_TFLOP/s": 2.0 * w.Hq * w.D * S / ms / 1e9,
+            "partial_table_GB/s": 2.0 * w.Hkv * 4 * S / ms / 1e6}
 
 
 def vision_tower_operator(dev, iters):
@@ -274,6 +304,7 @@ def main():
     result["adjacent_kernels"] = prologue_stage(w, dev, it)
     result["reference_operator"] = reference_operator(w, t, it)
     result["vision_tower_operator"] = vision_tower_operator(dev, it)
+    result["indexer_target"] = indexer_target_stage(w, t, it)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, torch.get_num_threads())
     print(json.dumps(result))

@@ -565,3 +565,23 @@ def test_attention_mass_matches_the_oracle(Hq, Hkv, D, K, segs):
     assert float(mass[pad].abs().sum()) == 0.0
     again = ops.attn_mass(d["q"], d["k"], lse, idx, n, d["cu_seqlens"], w.max_seqlen, scale)
     assert torch.equal(mass, again)                       # fixed summation order: bit-identical from run to run
+
+
+def test_operator_returns_the_mass_beside_the_output_and_stays_differentiable():
+    _log("return_mass")
+    w = W.scaled(W.C2, (300, 120, 77), top_k=64, name="C2-mass")
+    t = W.make_inputs(w, device=DEV)
+    q, k, v = (t[x].clone().requires_grad_(True) for x in ("q", "k", "v"))
+    out, idx, n, mass = ops.dsa_varlen_attn(q, k, v, t["cu_seqlens"], w.max_seqlen, indexer_q=t["q_idx"],
+                                            indexer_k=t["k_idx"], indexer_w=t["w_idx"], top_k=64,
+                                            return_indices=True, return_mass=True)
+    assert mass.shape == (w.T, 64) and not mass.requires_grad
+    assert (mass.sum(1) - 1.0).abs().max().item() <= 2e-3
+    want = R.attention_mass(t["q"].float().cpu(), t["k"].float().cpu(), idx.cpu(), n.cpu(), list(w.cu))
+    assert (mass.cpu() - want).abs().max().item() <= 2e-3
+    out.backward(t["dout"])
+    ref = ops.dsa_varlen_attn(t["q"], t["k"], t["v"], t["cu_seqlens"], w.max_seqlen, indexer_q=t["q_idx"],
+                              indexer_k=t["k_idx"], indexer_w=t["w_idx"], top_k=64)
+    assert torch.equal(out, ref) and q.grad is not None and torch.isfinite(q.grad).all()
+    with pytest.raises(ValueError):
+        ops.dsa_varlen_attn(t["q"], t["k"], t["v"], t["cu_seqlens"], w.max_seqlen, return_mass=True)

@@ -230,7 +230,7 @@ class _DsaVarlenAttn(torch.autograd.Function):
     Other dtypes / larger head_dim are rounded to bf16 once."""
 
     @staticmethod
-    def forward(ctx, q, k, v, cu_seqlens, max_seqlen, idx, n, softmax_scale, causal=True):
+    def forward(ctx, q, k, v, cu_seqlens, max_seqlen, idx, n, softmax_scale, causal=True, want_mass=False):
         in_dtype = q.dtype
         D = q.shape[-1]
         split = in_dtype == torch.float32 and 4 * D <= 256
@@ -260,11 +260,18 @@ class _DsaVarlenAttn(torch.autograd.Function):
         ctx.split = split
         ctx.D = D
         if split:
-            return out[..., :D].float() + out[..., D:2 * D].float()
-        return out if in_dtype == torch.bfloat16 else out.to(in_dtype)
+            res = out[..., :D].float() + out[..., D:2 * D].float()
+        else:
+            res = out if in_dtype == torch.bfloat16 else out.to(in_dtype)
+        if not want_mass:
+            return res
+        # from the very operands and log-sum-exp of the forward, so that every row sums to one
+        mass = attn_mass(qb, kb, lse, idx, n, cu_seqlens, int(max_seqlen), softmax_scale)
+        ctx.mark_non_differentiable(mass)
+        return res, mass
 
     @staticmethod
-    def backward(ctx, dout):
+    def backward(ctx, dout, *_):
         saved = ctx.saved_tensors
         qb, kb, vb, out, lse, cu = saved[:6]
         idx, n = (saved[6], saved[7]) if ctx.has_idx else (None, None)
@@ -288,13 +295,14 @@ class _DsaVarlenAttn(torch.autograd.Function):
             dv = dv[..., :D].float() + dv[..., 2 * D:3 * D].float()
         elif ctx.in_dtype != torch.bfloat16:
             dq, dk, dv = dq.to(ctx.in_dtype), dk.to(ctx.in_dtype), dv.to(ctx.in_dtype)
-        return dq, dk, dv, None, None, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None, None, None
 
 
 @torch.compiler.disable                                  # a compiled caller (the reference compiles per block) breaks the graph here
 def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, indexer_q=None, indexer_k=None, indexer_w=None,
                     top_k: Optional[int] = None, index_scale: Optional[float] = None,
-                    softmax_scale: Optional[float] = None, return_indices: bool = False, causal: bool = True):
+                    softmax_scale: Optional[float] = None, return_indices: bool = False, causal: bool = True,
+                    return_mass: bool = False):
     """Packed causal attention over ``cu_seqlens`` segments, optionally sparsified by the DSA indexer.
 
     q (T,Hq,D), k/v (T,Hkv,D) contiguous, cu_seqlens (N+1,) int32 on the device, max_seqlen host int
@@ -304,6 +312,9 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, in
     every causal key of the token's own segment is attended (the reference's behaviour).  With
     ``indexer_q (T,Hi,Di)``, ``indexer_k (T,Di)``, ``indexer_w (T,Hi)`` and ``top_k`` each query keeps
     the top_k keys of its causal window under (indexer score descending, key index ascending).
+    ``return_mass=True`` (with the indexer inputs) also returns the (T, top_k) fp32 table of head-averaged attention
+    probabilities of the selected keys, rows summing to one and aligned with the indices: the detached target of the
+    KL loss that trains the indexer.
     Gradients flow to q, k, v only.  A head_dim between the kernels' 64 / 128 / 256 is zero-padded to the
     next one and the output cut back (the scale stays that of the true head_dim).  ``causal=False`` (dense only) attends every key of the own segment, the
     vision towers' form of the call (models/qwen3_vl/model.py:423-428).
@@ -332,8 +343,14 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, in
     if d_kernel != D:
         # e.g. the 72-wide heads of the 1152/16 vision towers: zero columns change neither q.k nor the used part of p.v
         q, k, v = (torch.nn.functional.pad(x, (0, d_kernel - D)) for x in (q, k, v))
+    if return_mass and not sparse:
+        raise ValueError("return_mass needs the indexer inputs")
     out = _DsaVarlenAttn.apply(q.contiguous(), k.contiguous(), v.contiguous(), cu, int(max_seqlen), idx, n, scale,
-                               bool(causal))
+                               bool(causal), bool(return_mass))
+    mass = None
+    if return_mass:
+        out, mass = out
     if d_kernel != D:
         out = out[..., :D]
-    return (out, idx, n) if return_indices else out
+    res = (out,) + ((idx, n) if return_indices else ()) + ((mass,) if return_mass else ())
+    return res if len(res) > 1 else out
