@@ -77,6 +77,24 @@ int dsa_index_topk(const void *q_idx, const void *k_idx, const void *w_idx, cons
                    int32_t *idx, int32_t *n, void *ws, size_t ws_bytes, void *stream);
 
 /*
+ * dsa_index_topk that also returns the indexer scores of the selected keys: sel_scores[t*K + j] = score of key
+ * idx[t*K + j] (0 for j >= n[t]).  Every row is scored here, also those whose whole causal window is selected.
+ * No reference counterpart (the reference holds no indexer); serves the indexer's training loss below.
+ */
+int dsa_index_topk_scores(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu_seqlens,
+                          int T, int N, int Hi, int Di, int K, float scale, int dtype, int max_seqlen,
+                          int32_t *idx, int32_t *n, float *sel_scores, void *ws, size_t ws_bytes, void *stream);
+
+/*
+ * KL divergence of the indexer's distribution over the selected keys, softmax_j(sel_scores[t,:n[t]]), from a target
+ * distribution (dsa_attn_mass): loss[t] = sum_j mass (log mass - log softmax), and, when dscore != NULL, its
+ * gradient w.r.t. the scores times grad_scale: (softmax - mass) * grad_scale, 0 for j >= n[t].  No reference
+ * counterpart; a DSA layer adds mean(loss) to its objective in the training step (train/train_qwen.py:534-548).
+ */
+int dsa_indexer_kl(const float *sel_scores, const float *mass, const int32_t *n, int T, int K, float grad_scale,
+                   float *loss, float *dscore, void *stream);
+
+/*
  * Stage D3 - attention forward over the selected keys (idx/n), or over every causal key of the own
  * segment when idx == NULL: that case is the drop-in for varlen_attn(..., window_size=(-1,0))
  * (train/model_attention.py:123-132; models/qwen3_vl/model.py:41-46; models/qwen3_5/model.py:93-98).

@@ -24,6 +24,9 @@ Pinning status (what independent check fixes each function; see tests/test_oracl
   adversarial tie patterns (all equal, +-0.0, duplicates straddling the K-th place).
 * ``sparse_attention``       - pure-Python loop over selected keys; with K >= longest segment it
   must equal ``dense_varlen_causal``; gradients by ``torch.autograd.gradcheck`` in fp64.
+* ``selected_scores``        - a gather of the pinned ``indexer_scores_segment``; checked entry by entry in Python.
+* ``indexer_kl``             - ``torch.nn.functional.kl_div`` (library routine) on rows without padding, and
+  ``softmax - mass`` for its gradient.
 * ``attention_mass``         - pure-Python loop on a tiny case; rows sum to one; with one kv head the
   mass-weighted sum of the selected value rows equals the head mean of ``sparse_attention``'s output.
 
@@ -264,6 +267,31 @@ def attention_mass(q, k, idx, n, cu_seqlens, softmax_scale: Optional[float] = No
         p = torch.where(ok[:, None, :], p, torch.zeros((), dtype=cdt))          # rows without any key stay zero
         mass[c0:c1] = p.mean(dim=1)
     return mass
+
+
+def selected_scores(q_idx, k_idx, w, idx, n, cu_seqlens, index_scale: Optional[float] = None):
+    """Indexer scores of the selected keys: sel[t,j] = score(t, idx[t,j]) (0 where idx = -1), fp32."""
+    T, K = idx.shape
+    sel = torch.zeros(T, K, dtype=torch.float32)
+    for a, b in segments(cu_seqlens):
+        if b == a:
+            continue
+        sc = indexer_scores_segment(q_idx[a:b], k_idx[a:b], w[a:b], index_scale)     # (L,L), row t, column s - a
+        loc = (idx[a:b].long() - a).clamp(min=0)
+        sel[a:b] = torch.where(idx[a:b] >= 0, torch.gather(sc.float(), 1, loc), torch.zeros(()))
+    return sel
+
+
+def indexer_kl(sel, mass, n):
+    """loss[t] = KL(mass[t,:n[t]] || softmax(sel[t,:n[t]])) with 0 log 0 = 0, built from differentiable torch ops
+    (``sel`` may require grad: autograd then gives softmax - mass per row)."""
+    T, K = sel.shape
+    ok = torch.arange(K)[None, :] < n[:, None]
+    logq = torch.log_softmax(sel.masked_fill(~ok, float("-inf")), dim=-1)
+    logq = torch.where(ok, logq, torch.zeros((), dtype=sel.dtype))
+    p = torch.where(ok, mass.to(sel.dtype), torch.zeros((), dtype=sel.dtype))
+    terms = torch.where(p > 0, p * (torch.log(p.clamp(min=1e-45)) - logq), torch.zeros((), dtype=sel.dtype))
+    return terms.sum(-1)
 
 
 def dsa_varlen_attn_ref(q, k, v, cu_seqlens, q_idx, k_idx, w, top_k: int,

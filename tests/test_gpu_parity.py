@@ -585,3 +585,39 @@ def test_operator_returns_the_mass_beside_the_output_and_stays_differentiable():
     assert torch.equal(out, ref) and q.grad is not None and torch.isfinite(q.grad).all()
     with pytest.raises(ValueError):
         ops.dsa_varlen_attn(t["q"], t["k"], t["v"], t["cu_seqlens"], w.max_seqlen, return_mass=True)
+
+
+@pytest.mark.parametrize("segs,K", [((300, 1, 77, 513), 64), ((40, 3), 5), ((900,), 1024)])
+def test_selected_scores_and_indexer_kl(segs, K):
+    """Scores of the selected keys (also for rows whose whole window is selected) and the KL loss of the indexer
+    against the attention mass with its gradient.  Scores: same tolerance as the dense score rows (the same kernel
+    wrote them); loss and gradient: 1e-4 absolute against torch's log_softmax / autograd on the same inputs."""
+    _log(f"indexer kl {segs} K={K}")
+    w = W.Workload("kl", torch.bfloat16, segs, 8, 2, 128, 8, 64, K, 0.5, 91)
+    t = W.make_inputs(w, device="cpu")
+    d = {k_: (v_.to(DEV) if torch.is_tensor(v_) else v_) for k_, v_ in t.items()}
+    idx0, n0 = ops.index_topk(d["q_idx"], d["k_idx"], d["w_idx"], d["cu_seqlens"], w.max_seqlen, K)
+    idx, n, sel = ops.index_topk(d["q_idx"], d["k_idx"], d["w_idx"], d["cu_seqlens"], w.max_seqlen, K, return_scores=True)
+    assert torch.equal(idx, idx0) and torch.equal(n, n0)
+    dense = ops.indexer_scores(d["q_idx"], d["k_idx"], d["w_idx"], d["cu_seqlens"], w.max_seqlen)      # (T, ld)
+    cu = list(w.cu)
+    seg_start = torch.zeros(w.T, dtype=torch.long)
+    for a, b in zip(cu[:-1], cu[1:]):
+        seg_start[a:b] = a
+    loc = (idx.cpu().long() - seg_start[:, None]).clamp(min=0)
+    want_sel = torch.where(idx.cpu() >= 0, torch.gather(dense.cpu(), 1, loc), torch.zeros(()))
+    assert torch.equal(sel.cpu(), want_sel)                 # the very values the selection was made from
+    ref_sel = R.selected_scores(t["q_idx"].float(), t["k_idx"].float(), t["w_idx"].float(), idx.cpu(), n.cpu(), cu)
+    assert (sel.cpu() - ref_sel).abs().max().item() <= 2e-2 * max(1.0, ref_sel.abs().max().item())
+    scale = w.D ** -0.5
+    out, lse = ops.attn_fwd(d["q"], d["k"], d["v"], idx, n, d["cu_seqlens"], w.max_seqlen, scale)
+    mass = ops.attn_mass(d["q"], d["k"], lse, idx, n, d["cu_seqlens"], w.max_seqlen, scale)
+    loss, dscore = ops.indexer_kl(sel, mass, n)
+    s = sel.cpu().clone().requires_grad_(True)
+    ref_loss = R.indexer_kl(s, mass.cpu(), n.cpu())
+    (ref_loss.sum() / w.T).backward()
+    assert (loss.cpu() - ref_loss.detach()).abs().max().item() <= 1e-4 * max(1.0, ref_loss.max().item())
+    assert (dscore.cpu() - s.grad).abs().max().item() <= 1e-4 / w.T + 1e-7
+    assert (loss >= -1e-6).all()                            # a KL divergence
+    loss2, none = ops.indexer_kl(sel, mass, n, want_grad=False)
+    assert none is None and torch.equal(loss2, loss)

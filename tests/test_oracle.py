@@ -385,3 +385,31 @@ def test_attention_mass_against_a_python_loop_and_the_attention_output():
     m1 = R.attention_mass(q, k1, idx, n, cu)
     rows = v1[idx.clamp(min=0).long(), 0]                                # (T,K,D)
     assert torch.allclose((m1[..., None] * rows).sum(1), out.mean(1), atol=1e-5)
+
+
+def test_selected_scores_and_indexer_kl_against_library_routines():
+    import torch.nn.functional as F
+    cu = [0, 9, 20]
+    T, K = 20, 6
+    qi, ki, w = rnd(T, 3, 8, seed=51), rnd(T, 8, seed=52), rnd(T, 3, seed=53)
+    idx, n = R.dsa_select(qi, ki, w, cu, K)
+    sel = R.selected_scores(qi, ki, w, idx, n, cu)
+    for a, b in zip(cu[:-1], cu[1:]):
+        sc = R.indexer_scores_segment(qi[a:b], ki[a:b], w[a:b])
+        for t in range(a, b):
+            for j in range(K):
+                want = float(sc[t - a, int(idx[t, j]) - a]) if j < int(n[t]) else 0.0
+                assert abs(float(sel[t, j]) - want) < 1e-6
+    mass = torch.rand(T, K, generator=torch.Generator().manual_seed(54))
+    mass = torch.where(torch.arange(K)[None] < n[:, None], mass, torch.zeros(()))
+    mass[3, 0] = 0.0                                        # a zero target entry contributes nothing
+    mass = mass / mass.sum(-1, keepdim=True)
+    s = sel.clone().requires_grad_(True)
+    loss = R.indexer_kl(s, mass, n)
+    loss.sum().backward()
+    for t in range(T):
+        m = int(n[t])
+        want = F.kl_div(torch.log_softmax(sel[t, :m], -1), mass[t, :m], reduction="sum")
+        assert abs(float(loss[t]) - float(want)) < 1e-5
+        assert torch.allclose(s.grad[t, :m], torch.softmax(sel[t, :m], -1) - mass[t, :m], atol=1e-6)
+        assert float(s.grad[t, m:].abs().sum()) == 0.0

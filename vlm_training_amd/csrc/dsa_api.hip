@@ -9,6 +9,10 @@
 extern "C" {
 hipError_t dsa_launch_topk(const float *scores, int64_t ld, int row_begin, int row_end, const int32_t *cu, int N,
                            int K, int max_row, int32_t *idx, int32_t *n, hipStream_t stream);
+hipError_t dsa_launch_gather_scores(const float *scores, int64_t ld, int row_begin, int row_end, const int32_t *cu, int N,
+                                    int K, const int32_t *idx, const int32_t *n, float *sel, hipStream_t stream);
+hipError_t dsa_launch_indexer_kl(const float *sel, const float *mass, const int32_t *n, int T, int K, float grad_scale,
+                                 float *loss, float *dscore, hipStream_t stream);
 hipError_t dsa_launch_indexer(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu, int N,
                               int T, int Hi, int Di, float scale, int row_begin, int row_end, int skip_dense_k,
                               float *scores, int64_t ld, hipStream_t stream);
@@ -115,9 +119,11 @@ extern "C" size_t dsa_index_topk_workspace_bytes(int T, int max_seqlen, int K) {
     return align_up(rows, 4) * row_bytes;
 }
 
-extern "C" int dsa_index_topk(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu, int T, int N,
-                              int Hi, int Di, int K, float scale, int dtype, int max_seqlen, int32_t *idx, int32_t *n,
-                              void *ws, size_t ws_bytes, void *stream) {
+// sel_scores != NULL: every row is scored (also those whose whole causal window is selected) and the scores of
+// the selected keys are kept
+static int index_topk_impl(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu, int T, int N,
+                           int Hi, int Di, int K, float scale, int dtype, int max_seqlen, int32_t *idx, int32_t *n,
+                           float *sel_scores, void *ws, size_t ws_bytes, void *stream) {
     if (int rc = check_packed(T, N, cu)) return rc;
     if (K < 1) return fail(DSA_ERR_ARG, "top_k=%d must be >= 1", K);
     if (max_seqlen < 1 || max_seqlen > T) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
@@ -126,19 +132,47 @@ extern "C" int dsa_index_topk(const void *q_idx, const void *k_idx, const void *
     const int64_t ld = score_ld(max_seqlen);
     int64_t rows = ws ? (int64_t)(ws_bytes / ((size_t)ld * 4)) : 0;
     rows &= ~(int64_t)3;
-    if (max_seqlen <= K) rows = T;   // every row is dense: no score is read or written
+    if (max_seqlen <= K && !sel_scores) rows = T;   // every row is dense: no score is read or written
     else if (rows < 4) return fail(DSA_ERR_WORKSPACE, "workspace of %zu bytes holds no score chunk (row = %lld bytes)", ws_bytes, (long long)ld * 4);
     if (rows > T) rows = T;
     for (int64_t r0 = 0; r0 < T; r0 += rows) {
         const int r1 = (int)((r0 + rows < T) ? r0 + rows : T);
-        if (max_seqlen > K) {
-            int rc = dsa_indexer_scores(q_idx, k_idx, w_idx, cu, T, N, Hi, Di, scale, dtype, (int)r0, r1, K, (float *)ws, ld, stream);
+        if (max_seqlen > K || sel_scores) {
+            int rc = dsa_indexer_scores(q_idx, k_idx, w_idx, cu, T, N, Hi, Di, scale, dtype, (int)r0, r1, sel_scores ? 0 : K,
+                                        (float *)ws, ld, stream);
             if (rc) return rc;
         }
         hipError_t e = dsa_launch_topk((const float *)ws, ld, (int)r0, r1, cu, N, K, max_seqlen, idx, n, (hipStream_t)stream);
         if (e != hipSuccess) return hip_fail(e, "top-k launch");
+        if (sel_scores) {
+            e = dsa_launch_gather_scores((const float *)ws, ld, (int)r0, r1, cu, N, K, idx, n, sel_scores, (hipStream_t)stream);
+            if (e != hipSuccess) return hip_fail(e, "score gather launch");
+        }
     }
     return DSA_OK;
+}
+
+extern "C" int dsa_index_topk(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu, int T, int N,
+                              int Hi, int Di, int K, float scale, int dtype, int max_seqlen, int32_t *idx, int32_t *n,
+                              void *ws, size_t ws_bytes, void *stream) {
+    return index_topk_impl(q_idx, k_idx, w_idx, cu, T, N, Hi, Di, K, scale, dtype, max_seqlen, idx, n, nullptr, ws, ws_bytes,
+                           stream);
+}
+
+extern "C" int dsa_index_topk_scores(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu, int T,
+                                     int N, int Hi, int Di, int K, float scale, int dtype, int max_seqlen, int32_t *idx,
+                                     int32_t *n, float *sel_scores, void *ws, size_t ws_bytes, void *stream) {
+    if (!sel_scores) return fail(DSA_ERR_ARG, "null output pointer");
+    return index_topk_impl(q_idx, k_idx, w_idx, cu, T, N, Hi, Di, K, scale, dtype, max_seqlen, idx, n, sel_scores, ws,
+                           ws_bytes, stream);
+}
+
+extern "C" int dsa_indexer_kl(const float *sel_scores, const float *mass, const int32_t *n, int T, int K, float grad_scale,
+                              float *loss, float *dscore, void *stream) {
+    if (T < 0 || K < 1) return fail(DSA_ERR_ARG, "T=%d, top_k=%d", T, K);
+    if (T > 0 && (!sel_scores || !mass || !n || !loss)) return fail(DSA_ERR_ARG, "null tensor pointer");
+    hipError_t e = dsa_launch_indexer_kl(sel_scores, mass, n, T, K, grad_scale, loss, dscore, (hipStream_t)stream);
+    return e == hipSuccess ? DSA_OK : hip_fail(e, "indexer KL launch");
 }
 
 static int check_attn(int T, int N, const int32_t *cu, int Hq, int Hkv, int D, int K, int dtype, const int32_t *idx,

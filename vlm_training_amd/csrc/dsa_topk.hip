@@ -202,3 +202,81 @@ extern "C" hipError_t dsa_launch_topk(const float *scores, int64_t ld, int row_b
                            row_begin, cu, N, K, 0, idx, n);
     return hipGetLastError();
 }
+
+// ------------------------------------------------------------------------------------------------
+// Indexer scores of the selected keys, sel[t,j] = score of key idx[t,j] (0 for j >= n[t]), picked out of
+// the chunk's score rows after its top-k; and the KL divergence of the indexer's distribution over the
+// selected keys from a target distribution (the attention mass), with its gradient w.r.t. the scores.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void dsa_gather_scores_kernel(const float *__restrict__ scores, int64_t ld, int row_begin,
+                                                                 const int32_t *__restrict__ cu, int N, int K,
+                                                                 const int32_t *__restrict__ idx,
+                                                                 const int32_t *__restrict__ nsel, float *__restrict__ sel) {
+    const int t = row_begin + blockIdx.x;
+    const int s0 = cu[find_segment(cu, N, t)], nt = nsel[t];
+    const float *row = scores + (int64_t)(t - row_begin) * ld;
+    const int32_t *irow = idx + (int64_t)t * K;
+    float *orow = sel + (int64_t)t * K;
+    for (int j = threadIdx.x; j < K; j += 256) orow[j] = j < nt ? row[irow[j] - s0] : 0.f;
+}
+
+// block-wide reductions over 256 threads (4 waves)
+__device__ __forceinline__ float block_max_256(float v, float *red) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+__device__ __forceinline__ float block_sum_256(float v, float *red) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+// One workgroup per query row.  loss[t] = sum_j p_j (log p_j - log softmax(I)_j) over j < n[t] (terms with p_j = 0
+// are 0), dscore[t,j] = (softmax(I)_j - p_j) * grad_scale, 0 for j >= n[t].
+__global__ __launch_bounds__(256) void dsa_indexer_kl_kernel(const float *__restrict__ sel, const float *__restrict__ mass,
+                                                              const int32_t *__restrict__ nsel, int K, float grad_scale,
+                                                              float *__restrict__ loss, float *__restrict__ dscore) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, nt = nsel[t];
+    const float *irow = sel + (int64_t)t * K, *prow = mass + (int64_t)t * K;
+    float m = -INFINITY;
+    for (int j = threadIdx.x; j < nt; j += 256) m = fmaxf(m, irow[j]);
+    m = block_max_256(m, red);
+    float z = 0.f;
+    for (int j = threadIdx.x; j < nt; j += 256) z += __expf(irow[j] - m);
+    z = block_sum_256(z, red);
+    const float lse = m + __logf(z);
+    float acc = 0.f;
+    for (int j = threadIdx.x; j < K; j += 256) {
+        float g = 0.f;
+        if (j < nt) {
+            const float p = prow[j], logq = irow[j] - lse;
+            if (p > 0.f) acc += p * (__logf(p) - logq);
+            g = (__expf(logq) - p) * grad_scale;
+        }
+        if (dscore) dscore[(int64_t)t * K + j] = g;
+    }
+    acc = block_sum_256(acc, red);
+    if (threadIdx.x == 0) loss[t] = nt > 0 ? acc : 0.f;
+}
+
+extern "C" hipError_t dsa_launch_gather_scores(const float *scores, int64_t ld, int row_begin, int row_end,
+                                               const int32_t *cu, int N, int K, const int32_t *idx, const int32_t *n,
+                                               float *sel, hipStream_t stream) {
+    if (row_end <= row_begin) return hipSuccess;
+    hipLaunchKernelGGL(dsa_gather_scores_kernel, dim3(row_end - row_begin), dim3(256), 0, stream, scores, ld, row_begin, cu, N,
+                       K, idx, n, sel);
+    return hipGetLastError();
+}
+extern "C" hipError_t dsa_launch_indexer_kl(const float *sel, const float *mass, const int32_t *n, int T, int K,
+                                            float grad_scale, float *loss, float *dscore, hipStream_t stream) {
+    if (T <= 0) return hipSuccess;
+    hipLaunchKernelGGL(dsa_indexer_kl_kernel, dim3(T), dim3(256), 0, stream, sel, mass, n, K, grad_scale, loss, dscore);
+    return hipGetLastError();
+}

@@ -99,8 +99,9 @@ def topk_from_scores(scores: torch.Tensor, cu_seqlens, top_k: int) -> Tuple[torc
 
 
 def index_topk(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen: int, top_k: int,
-               index_scale: Optional[float] = None) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Stages D1+D2: selected key rows per query, (idx (T,K) int32 ascending/-1 padded, n (T,) int32)."""
+               index_scale: Optional[float] = None, return_scores: bool = False):
+    """Stages D1+D2: selected key rows per query, (idx (T,K) int32 ascending/-1 padded, n (T,) int32);
+    ``return_scores=True`` adds the (T,K) fp32 indexer scores of the selected keys (0 past n[t])."""
     _require_cuda(q_idx, k_idx, w_idx, cu_seqlens)
     if q_idx.dim() != 3 or k_idx.dim() != 2 or w_idx.dim() != 2:
         raise ValueError("indexer tensors must be q_idx (T,Hi,Di), k_idx (T,Di), w_idx (T,Hi)")
@@ -114,7 +115,7 @@ def index_topk(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen: int, top_k: int,
     lib = _lib.load()
     idx = torch.empty((T, top_k), dtype=torch.int32, device=q_idx.device)
     n = torch.empty((T,), dtype=torch.int32, device=q_idx.device)
-    ws_bytes = lib.dsa_index_topk_workspace_bytes(T, max_seqlen, top_k) if max_seqlen > top_k else 0
+    ws_bytes = lib.dsa_index_topk_workspace_bytes(T, max_seqlen, top_k) if (max_seqlen > top_k or return_scores) else 0
     ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q_idx.device)
     qi, ki, wi = _as_bf16(q_idx), _as_bf16(k_idx), _as_bf16(w_idx)     # keep the casts alive over the launch
     if os.environ.get("DSA_DEBUG_NAN"):
@@ -122,11 +123,34 @@ def index_topk(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen: int, top_k: int,
         # as it is in the CPU restatement of the selection
         if not (torch.isfinite(qi.float()).all() and torch.isfinite(ki.float()).all() and torch.isfinite(wi.float()).all()):
             raise ValueError("non-finite indexer inputs: their scores have no defined rank")
+    if return_scores:
+        sel = torch.empty((T, top_k), dtype=torch.float32, device=q_idx.device)
+        rc = lib.dsa_index_topk_scores(_ptr(qi), _ptr(ki), _ptr(wi), _ptr(cu), T, cu.numel() - 1, Hi, Di, top_k, scale,
+                                       _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(idx), _ptr(n), _ptr(sel), _ptr(ws), ws_bytes,
+                                       _stream(q_idx.device))
+        _lib.check(rc, "dsa_index_topk_scores")
+        return idx, n, sel
     rc = lib.dsa_index_topk(_ptr(qi), _ptr(ki), _ptr(wi), _ptr(cu), T,
                             cu.numel() - 1, Hi, Di, top_k, scale, _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(idx), _ptr(n),
                             _ptr(ws), ws_bytes, _stream(q_idx.device))
     _lib.check(rc, "dsa_index_topk")
     return idx, n
+
+
+def indexer_kl(sel_scores, mass, n, grad_scale: Optional[float] = None, want_grad: bool = True):
+    """KL(mass || softmax(sel_scores)) per query row over its selected keys -> (loss (T,) fp32, dscore (T,K) fp32 or
+    None).  ``dscore`` = d(grad_scale * sum_t loss[t]) / d sel_scores; grad_scale defaults to 1/T (mean loss)."""
+    _require_cuda(sel_scores, mass, n)
+    T, K = sel_scores.shape
+    if mass.shape != (T, K) or n.shape != (T,) or sel_scores.dtype != torch.float32 or mass.dtype != torch.float32:
+        raise ValueError("sel_scores and mass must be (T,K) fp32, n (T,) int32")
+    gs = float(grad_scale) if grad_scale is not None else 1.0 / max(T, 1)
+    loss = torch.empty((T,), dtype=torch.float32, device=mass.device)
+    dscore = torch.empty((T, K), dtype=torch.float32, device=mass.device) if want_grad else None
+    sc, ms = sel_scores.contiguous(), mass.contiguous()
+    rc = _lib.load().dsa_indexer_kl(_ptr(sc), _ptr(ms), _ptr(n), T, K, gs, _ptr(loss), _ptr(dscore), _stream(mass.device))
+    _lib.check(rc, "dsa_indexer_kl")
+    return loss, dscore
 
 
 def set_tile_crossover(crossover: int) -> int:
