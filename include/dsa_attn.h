@@ -95,6 +95,18 @@ int dsa_indexer_kl(const float *sel_scores, const float *mass, const int32_t *n,
                    float *loss, float *dscore, void *stream);
 
 /*
+ * Gradients of the selected indexer scores w.r.t. the indexer's inputs: given dscore[t*K + j] = dLoss/dScore of
+ * key idx[t*K + j] (dsa_indexer_kl), dq_idx (T,Hi,Di) and dk_idx (T,Di) in bf16 and dw (T,Hi) in fp32, for
+ * score = scale * sum_h w[t,h] relu(q_idx[t,h].k_idx[s]).  Deterministic (no atomics).  Hi <= 64, Di 64 or 128.
+ * No reference counterpart (autograd of a DSA layer's indexer in the training step, train/train_qwen.py:534-548).
+ */
+int dsa_indexer_bwd(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *idx, const int32_t *n,
+                    const float *dscore, const int32_t *cu_seqlens, int T, int N, int Hi, int Di, int K, float scale,
+                    int dtype, int max_seqlen, void *dq_idx, void *dk_idx, float *dw, void *ws, size_t ws_bytes,
+                    void *stream);
+size_t dsa_indexer_bwd_workspace_bytes(int T, int max_seqlen);
+
+/*
  * Stage D3 - attention forward over the selected keys (idx/n), or over every causal key of the own
  * segment when idx == NULL: that case is the drop-in for varlen_attn(..., window_size=(-1,0))
  * (train/model_attention.py:123-132; models/qwen3_vl/model.py:41-46; models/qwen3_5/model.py:93-98).

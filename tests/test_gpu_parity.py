@@ -621,3 +621,27 @@ def test_selected_scores_and_indexer_kl(segs, K):
     assert (loss >= -1e-6).all()                            # a KL divergence
     loss2, none = ops.indexer_kl(sel, mass, n, want_grad=False)
     assert none is None and torch.equal(loss2, loss)
+
+
+@pytest.mark.parametrize("Hi,Di,K,segs", [(8, 64, 16, (130, 64, 5)), (64, 128, 64, (300, 1, 77, 513)), (32, 64, 100, (50, 400)),
+                                           (40, 128, 8, (97, 200)), (64, 128, 512, (700,))])
+def test_indexer_backward_matches_autograd_of_the_oracle(Hi, Di, K, segs):
+    """dq_idx, dk_idx, dw for an arbitrary gradient at the selected scores, against torch autograd through the
+    oracle's score formula on the same bf16 inputs.  Tolerance as for the attention gradients (bf16 outputs)."""
+    _log(f"indexer bwd Hi={Hi} Di={Di} K={K}")
+    w = W.Workload("ibwd", torch.bfloat16, segs, 4, 2, 64, Hi, Di, K, 0.5, 123)
+    t = W.make_inputs(w, device="cpu")
+    d = {k_: (v_.to(DEV) if torch.is_tensor(v_) else v_) for k_, v_ in t.items()}
+    idx, n = ops.index_topk(d["q_idx"], d["k_idx"], d["w_idx"], d["cu_seqlens"], w.max_seqlen, K)
+    g = torch.Generator().manual_seed(5)
+    dscore = torch.randn(w.T, K, generator=g)
+    dscore = torch.where(torch.arange(K)[None] < n.cpu()[:, None], dscore, torch.zeros(()))
+    dq, dk, dw = ops.indexer_bwd(d["q_idx"], d["k_idx"], d["w_idx"], idx, n, dscore.to(DEV), d["cu_seqlens"], w.max_seqlen)
+    qi, ki, wi = (t[x].float().requires_grad_(True) for x in ("q_idx", "k_idx", "w_idx"))
+    sel = R.selected_scores(qi, ki, wi, idx.cpu(), n.cpu(), list(w.cu))
+    (sel * dscore).sum().backward()
+    assert_close_bf16(dq, qi.grad, "dq_idx")
+    assert_close_bf16(dk, ki.grad, "dk_idx")
+    assert_close_bf16(dw, wi.grad, "dw")
+    dq2, dk2, dw2 = ops.indexer_bwd(d["q_idx"], d["k_idx"], d["w_idx"], idx, n, dscore.to(DEV), d["cu_seqlens"], w.max_seqlen)
+    assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dw, dw2)

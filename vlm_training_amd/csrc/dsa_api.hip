@@ -26,6 +26,9 @@ hipError_t dsa_launch_gather_dq(const void *dout, const void *q, const void *k, 
                                 const float *delta, const int32_t *idx, const int32_t *n, const int32_t *cu, int N,
                                 int T, int Hq, int Hkv, int D, int K, float scale, int pos_min, void *dq,
                                 hipStream_t stream);
+hipError_t dsa_launch_indexer_bwd(const void *q_idx, const void *k_idx, const void *w_idx, const float *dscore,
+                                  const uint32_t *bitmap, int32_t *prefix, int ldw, const int32_t *cu, int N, int T, int Hi,
+                                  int Di, int K, float cscale, void *dq_idx, void *dk_idx, float *dw, hipStream_t stream);
 hipError_t dsa_launch_tile_mass(const void *q, const void *k, const float *lse, const uint32_t *bitmap, int ldw,
                                 const int32_t *n, const int32_t *cu, int N, int T, int Hq, int Hkv, int D, int K,
                                 float scale, float *partial, float *mass, hipStream_t stream);
@@ -271,6 +274,38 @@ extern "C" int dsa_attn_mass(const void *q, const void *k, const float *lse, con
     if (e != hipSuccess) return hip_fail(e, "bitmap launch");
     e = dsa_launch_tile_mass(q, k, lse, bitmap, ldw, n, cu, N, T, Hq, Hkv, D, K, softmax_scale, partial, mass, st);
     if (e != hipSuccess) return hip_fail(e, "attention mass launch");
+    return DSA_OK;
+}
+
+// ---- indexer backward: gradients of the selected scores w.r.t. the indexer's inputs --------------------
+extern "C" size_t dsa_indexer_bwd_workspace_bytes(int T, int max_seqlen) {
+    if (T <= 0) return 0;
+    return 2 * align_up((size_t)T * bitmap_ldw(max_seqlen) * 4, 256);      // selection bitmap + slot prefix table
+}
+
+extern "C" int dsa_indexer_bwd(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *idx, const int32_t *n,
+                               const float *dscore, const int32_t *cu, int T, int N, int Hi, int Di, int K, float scale,
+                               int dtype, int max_seqlen, void *dq_idx, void *dk_idx, float *dw, void *ws, size_t ws_bytes,
+                               void *stream) {
+    if (int rc = check_packed(T, N, cu)) return rc;
+    if (dtype != DSA_DTYPE_BF16) return fail(DSA_ERR_UNSUPPORTED, "indexer tensors must be bf16 (dtype code %d)", dtype);
+    if (Hi < 1 || Hi > 64) return fail(DSA_ERR_UNSUPPORTED, "Hi=%d: 1..64 indexer heads", Hi);
+    if (!(Di == 64 || Di == 128)) return fail(DSA_ERR_UNSUPPORTED, "Di=%d: the indexer backward covers 64 and 128", Di);
+    if (K < 1) return fail(DSA_ERR_ARG, "top_k=%d must be >= 1", K);
+    if (!q_idx || !k_idx || !w_idx || !idx || !n || !dscore || !dq_idx || !dk_idx || !dw) return fail(DSA_ERR_ARG, "null tensor pointer");
+    if (max_seqlen < 1 || max_seqlen > (T > 0 ? T : 1)) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
+    if (T == 0) return DSA_OK;
+    const size_t need = dsa_indexer_bwd_workspace_bytes(T, max_seqlen);
+    if (!ws || ws_bytes < need) return fail(DSA_ERR_WORKSPACE, "indexer backward workspace: have %zu bytes, need %zu", ws_bytes, need);
+    const int ldw = bitmap_ldw(max_seqlen);
+    if ((size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);
+    hipStream_t st = (hipStream_t)stream;
+    uint32_t *bitmap = (uint32_t *)ws;
+    int32_t *prefix = (int32_t *)((char *)ws + need / 2);
+    hipError_t e = dsa_launch_bitmap(idx, n, cu, N, T, K, ldw, bitmap, st);
+    if (e != hipSuccess) return hip_fail(e, "bitmap launch");
+    e = dsa_launch_indexer_bwd(q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, Di, K, scale, dq_idx, dk_idx, dw, st);
+    if (e != hipSuccess) return hip_fail(e, "indexer backward launch");
     return DSA_OK;
 }
 

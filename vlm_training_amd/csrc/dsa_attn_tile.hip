@@ -443,6 +443,254 @@ __global__ __launch_bounds__(256) void dsa_mass_reduce_kernel(const float *__res
 }
 
 // ==================================================================================================
+// Indexer backward.  The indexer score of a selected pair is  I[t,s] = c * sum_h w[t,h] relu(r[t,h,s]),
+// r = q_idx[t,h,:] . k_idx[s,:]  (multi-query attention with ReLU in place of the softmax: Hi heads, one key
+// head).  Given dscore[t,j] = dLoss/dI at the selected keys (slot j of key s = its rank in the ascending
+// selection list = selected keys of earlier tiles + those below it in the tile's word):
+//     G[t,h,s]   = dscore[t,s] * w[t,h] * (r > 0)
+//     dq_idx[t,h,:] = c * sum_s G[t,h,s] k_idx[s,:]      dw[t,h] = c * sum_s dscore[t,s] relu(r[t,h,s])
+//     dk_idx[s,:]   = c * sum_t sum_h G[t,h,s] q_idx[t,h,:]
+// Query side = the dQ walk (rows = (query, indexer head), padded to 32 or 64 rows per query so that the 32
+// rows of a wave belong to one query): S^T = K Q^T, G^T on the C layout, dQ^T += K^T G^T.  Key side = the
+// key-stationary walk: a wave owns 32 keys (rows in registers) and walks the later queries in blocks of
+// 32 heads of one query: S = Q K^T, G on the C layout, dK^T += Q^T G.  Every output row is reduced by one
+// wave in a fixed order: deterministic, no atomics.
+// ==================================================================================================
+template <int D, int GSHIFT, int NW>
+__global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_tile_idxq_kernel(
+    const bf16_t *__restrict__ q_idx, const bf16_t *__restrict__ k_idx, const bf16_t *__restrict__ w_idx,
+    const float *__restrict__ dscore, const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N,
+    int T, int Hi, int K, float cscale, bf16_t *__restrict__ dq_idx, float *__restrict__ dw) {
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / (NW * 64);
+    constexpr int NBUF = 2, NT = NW * 64, Gp = 1 << GSHIFT, QBW = (NW * 32) >> GSHIFT;
+    static_assert(LOADS >= 1 && GSHIFT >= 5, "a wave's 32 rows are heads of one query");
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][TILE_B];
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
+    LaneOffsets<D> lo;
+    lo.init(lane);
+    int s0, L, blk;
+    if (!locate_block(cu, N, blockIdx.x, QBW, true, s0, L, blk)) return;
+    const int qc0 = blk * QBW;
+    const int r = wv * 32 + j;
+    const int qcol = qc0 + (r >> GSHIFT), head = r & (Gp - 1);
+    const bool row_ok = qcol < L && head < Hi;
+    const int t = s0 + min(qcol, L - 1), hrow = min(head, Hi - 1);
+    u32x4 kst[2][LOADS];
+#define IDXQ_LOAD(SET, TILE)                                                                        \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+        const int c = i * NT + tid;                                                                \
+        const int row = c / CPR, ch = c % CPR;                                                     \
+        kst[SET][i] = *reinterpret_cast<const u32x4 *>(k_idx + (int64_t)(s0 + min((TILE) * 32 + row, L - 1)) * D + ch * 8); \
+    }
+    IDXQ_LOAD(0, 0)
+    bf16x8 qB[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+        qB[ks] = row_ok ? load_bf16x8(q_idx + ((int64_t)t * Hi + hrow) * D + 16 * ks + 8 * h) : zero_bf16x8();
+    const float wrow_v = row_ok ? (float)w_idx[(int64_t)t * Hi + hrow] : 0.f;
+    const int ntiles = min(qc0 + QBW - 1, L - 1) / 32 + 1;
+    const uint32_t *wrow = bitmap + (int64_t)t * ldw;
+    const float *drow = dscore + (int64_t)t * K;
+    uint32_t word_next = wrow[0];
+    int seen = 0;
+    f32x16 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
+    float dwacc = 0.f;
+
+#define IDXQ_STORE(SET, BUF, TILE)                                                                  \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+        const int c = i * NT + tid;                                                                \
+        const int row = c / CPR, ch = c % CPR;                                                     \
+        *reinterpret_cast<u32x4 *>(&lds[BUF][tile_off<D>(row, ch)]) = kst[SET][i];                 \
+    }
+#define IDXQ_COMPUTE(TILE, BUF)                                                                     \
+    {                                                                                              \
+        const unsigned char *kt = lds[BUF];                                                        \
+        const uint32_t word_full = qcol < L ? word_next : 0u;                                      \
+        word_next = wrow[min((TILE) + 1, ntiles - 1)];                                             \
+        /* lane j fetches the gradient of key column j of the tile (both halves of the wave the same) */ \
+        const bool mine = (word_full >> j) & 1u;                                                   \
+        float dl = drow[min(seen + (int)__popc(word_full & ((1u << j) - 1u)), K - 1)];             \
+        dl = mine ? dl : 0.f;                                                                      \
+        seen += __popc(word_full);                                                                 \
+        f32x16 sacc = zero16();                                                                    \
+        {                                                                                          \
+            bf16x8 ka[KS];                                                                         \
+            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) ka[ks] = lo.rowop(kt, ks);           \
+            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) sacc = mfma32(ka[ks], qB[ks], sacc); \
+            sched_reads_ahead<KS, 4, 1>();                                                         \
+        }                                                                                          \
+        float ds[16];                                                                              \
+        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
+            const float dsv = __shfl(dl, 8 * (vi >> 2) + (vi & 3) + 4 * h, 64);   /* element vi is key column 8*(vi/4)+4h+vi%4 */ \
+            const float sv = sacc[vi];                                                             \
+            dwacc = fmaf(dsv, fmaxf(sv, 0.f), dwacc);                                              \
+            ds[vi] = sv > 0.f ? dsv * wrow_v : 0.f;                                                \
+        }                                                                                          \
+        const bf16x8 dB0 = pack8(ds), dB1 = pack8(ds + 8);                                         \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
+            mfma32_acc(acc[dt], lo.trop(kt, 0, dt), dB0);                                          \
+            mfma32_acc(acc[dt], lo.trop(kt, 1, dt), dB1);                                          \
+        }                                                                                          \
+        sched_reads_ahead<2 * DT, 3, 2>();                                                         \
+    }
+    TILE_PIPELINE(ntiles, IDXQ_LOAD, IDXQ_STORE, IDXQ_COMPUTE)
+#undef IDXQ_LOAD
+#undef IDXQ_STORE
+#undef IDXQ_COMPUTE
+
+    const float dwt = half_sum_f(dwacc);
+    if (row_ok) {
+        bf16_t *op = dq_idx + ((int64_t)t * Hi + hrow) * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) store_c_tile(op + dt * 32, acc[dt], cscale, h);
+        if (h == 0) dw[(int64_t)t * Hi + hrow] = dwt * cscale;
+    }
+}
+
+// key side.  Workgroup = 4 waves x 32 keys = one 128-key tile of a segment; block b of its walk = the 32 heads
+// [32*(b % HB), +32) of query c0 + b / HB.
+template <int D, int GSHIFT>
+__global__ __launch_bounds__(256) void dsa_tile_idxk_kernel(
+    const bf16_t *__restrict__ q_idx, const bf16_t *__restrict__ k_idx, const bf16_t *__restrict__ w_idx,
+    const float *__restrict__ dscore, const uint32_t *__restrict__ bitmap, const int32_t *__restrict__ prefix, int ldw,
+    const int32_t *__restrict__ cu, int N, int T, int Hi, int K, float cscale, bf16_t *__restrict__ dk_idx) {
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / 256;
+    constexpr int NBUF = 2, HB = (1 << GSHIFT) / 32;
+    static_assert(GSHIFT >= 5 && LOADS >= 1, "blocks of 32 heads of one query");
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][TILE_B];
+    __shared__ __attribute__((aligned(16))) float w_s[NBUF][32];
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
+    LaneOffsets<D> lo;
+    lo.init(lane);
+    int s0, L, blk;
+    if (!locate_block(cu, N, blockIdx.x, 128, false, s0, L, blk)) return;
+    const int c0 = blk * 128, kc = c0 + wv * 32;
+    const int mykey = kc + j;
+    const bool key_ok = mykey < L;
+    const int64_t krow = (int64_t)s0 + min(mykey, L - 1);
+    const bool kw_ok = kc < L;                           // the word column of this wave's keys exists
+    const int kw = kw_ok ? kc >> 5 : 0;
+    bf16x8 kB[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) kB[ks] = load_bf16x8(k_idx + krow * D + 16 * ks + 8 * h);
+    f32x16 dkacc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) dkacc[dt] = zero16();
+    const int nq = L - c0, nblocks = nq * HB;            // queries c0 .. L-1 can have selected keys of this tile
+
+    // selection words and slot bases of this wave's key column for 64 consecutive queries, one query per lane
+    auto fetch_words = [&](int chunk, uint32_t &wq, int32_t &bq) {
+        const int qc = min(c0 + chunk * 64 + lane, L - 1);
+        const int64_t o = (int64_t)(s0 + qc) * ldw + kw;
+        wq = kw_ok ? bitmap[o] : 0u;
+        bq = prefix[o];
+    };
+    uint32_t wq_cur, wq_nxt;
+    int32_t bq_cur, bq_nxt;
+    fetch_words(0, wq_cur, bq_cur);
+    fetch_words(1, wq_nxt, bq_nxt);
+    int cur_chunk = 0;
+
+    u32x4 qst[2][LOADS];
+    float dl_st[2] = {0.f, 0.f}, dl_buf[NBUF] = {0.f, 0.f};
+    bool sel_st[2] = {false, false};
+    uint32_t w_st[2] = {0u, 0u};
+#define IDXK_LOAD(SET, BLK)                                                                         \
+    {                                                                                              \
+        const int rel = (BLK) / HB, hb = (BLK) % HB, qc = c0 + rel;                                \
+        _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                        \
+            const int c = i * 256 + tid;                                                           \
+            const int row = c / CPR, ch = c % CPR;                                                 \
+            const int hd = min(hb * 32 + row, Hi - 1);                                             \
+            qst[SET][i] = *reinterpret_cast<const u32x4 *>(q_idx + ((int64_t)(s0 + qc) * Hi + hd) * D + ch * 8); \
+        }                                                                                          \
+        w_st[SET] = reinterpret_cast<const unsigned short *>(w_idx)[(int64_t)(s0 + qc) * Hi + min(hb * 32 + (tid & 31), Hi - 1)]; \
+        if ((rel >> 6) != cur_chunk) {                   /* wave-uniform: move on to the next 64 queries */ \
+            wq_cur = wq_nxt;                                                                       \
+            bq_cur = bq_nxt;                                                                       \
+            cur_chunk = rel >> 6;                                                                  \
+            fetch_words(cur_chunk + 1, wq_nxt, bq_nxt);                                            \
+        }                                                                                          \
+        const uint32_t word = __builtin_amdgcn_readlane(wq_cur, rel & 63);                         \
+        const int base = __builtin_amdgcn_readlane(bq_cur, rel & 63);                              \
+        sel_st[SET] = (word >> j) & 1u;                                                            \
+        dl_st[SET] = dscore[(int64_t)(s0 + qc) * K + min(base + (int)__popc(word & ((1u << j) - 1u)), K - 1)]; \
+    }
+#define IDXK_STORE(SET, BUF, BLK)                                                                   \
+    {                                                                                              \
+        const int hb = (BLK) % HB;                                                                 \
+        const u32x4 z4 = {0u, 0u, 0u, 0u};                                                         \
+        _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                        \
+            const int c = i * 256 + tid;                                                           \
+            const int row = c / CPR, ch = c % CPR;                                                 \
+            /* padded heads are zeroed: they add nothing to dK */                                   \
+            *reinterpret_cast<u32x4 *>(&lds[BUF][tile_off<D>(row, ch)]) = hb * 32 + row < Hi ? qst[SET][i] : z4; \
+        }                                                                                          \
+        if (tid < 32) w_s[BUF][tid] = hb * 32 + tid < Hi ? __uint_as_float(w_st[SET] << 16) : 0.f;  \
+        dl_buf[BUF] = sel_st[SET] ? dl_st[SET] : 0.f;                                              \
+    }
+#define IDXK_COMPUTE(BLK, BUF)                                                                      \
+    {                                                                                              \
+        const unsigned char *qt = lds[BUF];                                                        \
+        const float dl = dl_buf[BUF];                    /* gradient of (query of the block, this lane's key) */ \
+        f32x16 sacc = zero16();                                                                    \
+        {                                                                                          \
+            bf16x8 qa[KS];                                                                         \
+            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) qa[ks] = lo.rowop(qt, ks);           \
+            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) sacc = mfma32(qa[ks], kB[ks], sacc); \
+            sched_reads_ahead<KS, 4, 1>();                                                         \
+        }                                                                                          \
+        float gs[16];                                                                              \
+        _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {                                         \
+            const f32x4 w4 = *reinterpret_cast<const f32x4 *>(&w_s[BUF][8 * g4 + 4 * h]);          \
+            _Pragma("unroll") for (int e = 0; e < 4; ++e) gs[4 * g4 + e] = sacc[4 * g4 + e] > 0.f ? dl * w4[e] : 0.f; \
+        }                                                                                          \
+        const bf16x8 gB0 = pack8(gs), gB1 = pack8(gs + 8);                                         \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
+            mfma32_acc(dkacc[dt], lo.trop(qt, 0, dt), gB0);                                        \
+            mfma32_acc(dkacc[dt], lo.trop(qt, 1, dt), gB1);                                        \
+        }                                                                                          \
+        sched_reads_ahead<2 * DT, 3, 2>();                                                         \
+    }
+    IDXK_LOAD(0, 0)
+    TILE_PIPELINE(nblocks, IDXK_LOAD, IDXK_STORE, IDXK_COMPUTE)
+#undef IDXK_LOAD
+#undef IDXK_STORE
+#undef IDXK_COMPUTE
+
+    if (key_ok) {
+        bf16_t *pk = dk_idx + krow * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) store_c_tile(pk + dt * 32, dkacc[dt], cscale, h);
+    }
+}
+
+// prefix[t][w] = selected keys of query t in the words before w (the slot of the first selected key of word w)
+__global__ __launch_bounds__(64) void dsa_bitmap_prefix_kernel(const uint32_t *__restrict__ bitmap, int ldw,
+                                                                int32_t *__restrict__ prefix) {
+    const int lane = threadIdx.x;
+    const uint32_t *row = bitmap + (int64_t)blockIdx.x * ldw;
+    int32_t *orow = prefix + (int64_t)blockIdx.x * ldw;
+    int carry = 0;
+    for (int w0 = 0; w0 < ldw; w0 += 64) {
+        const int w = w0 + lane;
+        const int c = w < ldw ? (int)__popc(row[w]) : 0;
+        int incl = c;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int u = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += u;
+        }
+        if (w < ldw) orow[w] = carry + incl - c;
+        carry += __shfl(incl, 63, 64);
+    }
+}
+
+// ==================================================================================================
 // dQ: query-stationary, same walk as the forward.
 //   S^T = K Q^T, dP^T = V dO^T  (A = K / V tiles row-wise, B = Q^T / dO^T in registers)
 //   dS^T = P^T * (dP^T - delta)  on the C layout
@@ -1037,6 +1285,36 @@ extern "C" hipError_t dsa_launch_tile_mass(const void *q, const void *k, const f
     const unsigned parts = (unsigned)((K / 4 + 255) / 256 > 0 ? (K / 4 + 255) / 256 : 1);
     hipLaunchKernelGGL(dsa_mass_reduce_kernel, dim3(T, parts < 8 ? parts : 8), dim3(256), 0, stream, partial, n, T, K, Hkv,
                        1.f / (float)Hq, mass);
+    return hipGetLastError();
+}
+// indexer backward: prefix table, query side (dq_idx, dw), key side (dk_idx).  D = indexer head_dim (64 or 128),
+// at most 64 indexer heads.
+template <int D, int GS>
+static void launch_idx_bwd_i(hipStream_t stream, const void *q_idx, const void *k_idx, const void *w_idx, const float *dscore,
+                             const uint32_t *bitmap, const int32_t *prefix, int ldw, const int32_t *cu, int N, int T, int Hi,
+                             int K, float cscale, void *dq_idx, void *dk_idx, float *dw) {
+    constexpr int NW = tile_waves<D>();
+    const dim3 gq((unsigned)((int64_t)T / ((32 * NW) >> GS) + N + 1));
+    hipLaunchKernelGGL((dsa_tile_idxq_kernel<D, GS, NW>), gq, dim3(64 * NW), 0, stream, (const bf16_t *)q_idx,
+                       (const bf16_t *)k_idx, (const bf16_t *)w_idx, dscore, bitmap, ldw, cu, N, T, Hi, K, cscale,
+                       (bf16_t *)dq_idx, dw);
+    const dim3 gk((unsigned)((int64_t)T / 128 + N + 1));
+    hipLaunchKernelGGL((dsa_tile_idxk_kernel<D, GS>), gk, dim3(256), 0, stream, (const bf16_t *)q_idx, (const bf16_t *)k_idx,
+                       (const bf16_t *)w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, (bf16_t *)dk_idx);
+}
+extern "C" hipError_t dsa_launch_indexer_bwd(const void *q_idx, const void *k_idx, const void *w_idx, const float *dscore,
+                                             const uint32_t *bitmap, int32_t *prefix, int ldw, const int32_t *cu, int N,
+                                             int T, int Hi, int Di, int K, float cscale, void *dq_idx, void *dk_idx,
+                                             float *dw, hipStream_t stream) {
+    if (Hi < 1 || Hi > 64 || !(Di == 64 || Di == 128)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(dsa_bitmap_prefix_kernel, dim3(T), dim3(64), 0, stream, bitmap, ldw, prefix);
+    if (Di == 128) {
+        if (Hi > 32) launch_idx_bwd_i<128, 6>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw);
+        else launch_idx_bwd_i<128, 5>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw);
+    } else {
+        if (Hi > 32) launch_idx_bwd_i<64, 6>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw);
+        else launch_idx_bwd_i<64, 5>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw);
+    }
     return hipGetLastError();
 }
 extern "C" hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const void *k, const void *v,

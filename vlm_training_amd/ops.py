@@ -153,6 +153,31 @@ def indexer_kl(sel_scores, mass, n, grad_scale: Optional[float] = None, want_gra
     return loss, dscore
 
 
+def indexer_bwd(q_idx, k_idx, w_idx, idx, n, dscore, cu_seqlens, max_seqlen: int, index_scale: Optional[float] = None):
+    """Gradients of the selected indexer scores: (dq_idx (T,Hi,Di) bf16, dk_idx (T,Di) bf16, dw (T,Hi) fp32) for
+    ``dscore`` (T,K) fp32 = dLoss/dScore at the selected keys."""
+    _require_cuda(q_idx, k_idx, w_idx, idx, n, dscore, cu_seqlens)
+    T, Hi, Di = q_idx.shape
+    K = idx.shape[1]
+    cu = _check_cu(cu_seqlens, T)
+    if dscore.shape != (T, K) or dscore.dtype != torch.float32:
+        raise ValueError("dscore must be (T,K) fp32")
+    scale = index_scale if index_scale is not None else (Di ** -0.5) * (Hi ** -0.5)
+    lib = _lib.load()
+    qi, ki, wi = _as_bf16(q_idx), _as_bf16(k_idx), _as_bf16(w_idx)
+    dq = torch.empty_like(qi)
+    dk = torch.empty_like(ki)
+    dw = torch.empty((T, Hi), dtype=torch.float32, device=qi.device)
+    max_seqlen = T if max_seqlen is None else int(max_seqlen)
+    ws_bytes = lib.dsa_indexer_bwd_workspace_bytes(T, max_seqlen)
+    ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=qi.device)
+    rc = lib.dsa_indexer_bwd(_ptr(qi), _ptr(ki), _ptr(wi), _ptr(idx), _ptr(n), _ptr(dscore.contiguous()), _ptr(cu), T,
+                             cu.numel() - 1, Hi, Di, K, scale, _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(dq), _ptr(dk), _ptr(dw),
+                             _ptr(ws), ws_bytes, _stream(qi.device))
+    _lib.check(rc, "dsa_indexer_bwd")
+    return dq, dk, dw
+
+
 def set_tile_crossover(crossover: int) -> int:
     """Rows with pos < top_k * crossover use the MFMA tile kernels, later rows the gather kernels.
     Returns the previous value (tests use it to drive each path on its own)."""
