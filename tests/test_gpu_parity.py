@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from oracle import dsa_ref as R
-from tests.util import assert_close_bf16, oracle_topk_from_gpu_scores
+from tests.util import assert_close_bf16, cosine, oracle_topk_from_gpu_scores
 from vlm_training_amd import ops, workloads as W
 
 pytestmark = pytest.mark.gpu
@@ -645,3 +645,28 @@ def test_indexer_backward_matches_autograd_of_the_oracle(Hi, Di, K, segs):
     assert_close_bf16(dw, wi.grad, "dw")
     dq2, dk2, dw2 = ops.indexer_bwd(d["q_idx"], d["k_idx"], d["w_idx"], idx, n, dscore.to(DEV), d["cu_seqlens"], w.max_seqlen)
     assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dw, dw2)
+
+
+def test_indexer_training_step_end_to_end():
+    """Attention with return_mass, then the indexer's KL loss and its gradients, against the oracle: loss value
+    and d loss / d (q_idx, k_idx, w) through torch autograd of the oracle's formulas."""
+    _log("indexer training step")
+    import vlm_training_amd as M
+    w = W.Workload("itrain", torch.bfloat16, (300, 120, 77, 260), 8, 2, 128, 16, 64, 48, 0.5, 321)
+    t = W.make_inputs(w, device="cpu")
+    d = {k_: (v_.to(DEV) if torch.is_tensor(v_) else v_) for k_, v_ in t.items()}
+    qi, ki, wi = (d[x].clone().requires_grad_(True) for x in ("q_idx", "k_idx", "w_idx"))
+    out, idx, n, mass = M.dsa_varlen_attn(d["q"], d["k"], d["v"], d["cu_seqlens"], w.max_seqlen, indexer_q=qi, indexer_k=ki,
+                                          indexer_w=wi, top_k=w.top_k, return_indices=True, return_mass=True)
+    loss = M.indexer_kl_loss(qi, ki, wi, mass, d["cu_seqlens"], w.max_seqlen, w.top_k)
+    (loss * 3.0).backward()
+    rq, rk, rw = (t[x].float().requires_grad_(True) for x in ("q_idx", "k_idx", "w_idx"))
+    sel = R.selected_scores(rq, rk, rw, idx.cpu(), n.cpu(), list(w.cu))
+    ref = R.indexer_kl(sel, mass.cpu(), n.cpu()).mean()
+    (ref * 3.0).backward()
+    assert abs(loss.item() - ref.item()) <= 1e-3 * max(1.0, abs(ref.item()))
+    for got, want, name in ((qi.grad, rq.grad, "dq_idx"), (ki.grad, rk.grad, "dk_idx"), (wi.grad, rw.grad, "dw")):
+        assert got is not None and got.dtype == torch.bfloat16
+        scale = want.abs().max().item()
+        assert (got.float().cpu() - want).abs().max().item() <= 2e-2 * scale + 1e-6, name
+        assert cosine(got.float().cpu(), want) > 0.9995, name

@@ -178,6 +178,38 @@ def indexer_bwd(q_idx, k_idx, w_idx, idx, n, dscore, cu_seqlens, max_seqlen: int
     return dq, dk, dw
 
 
+class _IndexerKL(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q_idx, k_idx, w_idx, mass, cu_seqlens, max_seqlen, top_k, index_scale):
+        T = q_idx.shape[0]
+        idx, n, sel = index_topk(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen, top_k, index_scale, return_scores=True)
+        loss_rows, dscore = indexer_kl(sel, mass, n, grad_scale=1.0 / max(T, 1))
+        ctx.save_for_backward(q_idx, k_idx, w_idx, idx, n, dscore, cu_seqlens)
+        ctx.max_seqlen, ctx.index_scale = max_seqlen, index_scale
+        return loss_rows.mean()
+
+    @staticmethod
+    def backward(ctx, g):
+        q_idx, k_idx, w_idx, idx, n, dscore, cu = ctx.saved_tensors
+        dq, dk, dw = indexer_bwd(q_idx, k_idx, w_idx, idx, n, dscore, cu, ctx.max_seqlen, ctx.index_scale)
+        g = g.to(torch.float32)
+        return ((dq.float() * g).to(q_idx.dtype), (dk.float() * g).to(k_idx.dtype), (dw * g).to(w_idx.dtype), None, None,
+                None, None, None)
+
+
+@torch.compiler.disable
+def indexer_kl_loss(indexer_q, indexer_k, indexer_w, mass, cu_seqlens, max_seqlen: Optional[int], top_k: int,
+                    index_scale: Optional[float] = None):
+    """Training loss of the DSA indexer: mean over the packed tokens of KL(mass[t] || softmax of the indexer's scores
+    over the keys it selected for t), differentiable w.r.t. indexer_q (T,Hi,Di), indexer_k (T,Di), indexer_w (T,Hi).
+
+    ``mass`` is the detached target ``dsa_varlen_attn(..., return_mass=True)`` returned for the same indexer
+    inputs and top_k (the selection is recomputed here and is the same: it is deterministic)."""
+    T = indexer_q.shape[0]
+    max_seqlen = T if max_seqlen is None else int(max_seqlen)
+    return _IndexerKL.apply(indexer_q, indexer_k, indexer_w, mass, cu_seqlens, max_seqlen, int(top_k), index_scale)
+
+
 def set_tile_crossover(crossover: int) -> int:
     """Rows with pos < top_k * crossover use the MFMA tile kernels, later rows the gather kernels.
     Returns the previous value (tests use it to drive each path on its own)."""
