@@ -140,17 +140,28 @@ def reference_operator(w, t, iters):
 
 
 def indexer_target_stage(w, t, iters):
-    """Attention mass of the selected keys (the target of the KL loss that trains the indexer): one more pass
-    over the forward's S = QK^T with the saved log-sum-exp.  Matrix work 2*Hq*D flop per selected pair; the
-    per-kv-head partial tables it writes and adds up are 2 * Hkv * 4 bytes per selected pair of HBM traffic."""
+    """The indexer's training path beside the operator: attention mass of the selected keys (one more pass over the
+    forward's S = QK^T with the saved log-sum-exp: 2*Hq*D flop per selected pair, 2*Hkv*4 bytes of partial tables),
+    index+top-k that also keeps the selected scores (every row scored), the KL loss with its gradient at the scores,
+    and the indexer backward (query side 4*Hi*Di, key side 4*Hi*Di flop per causal pair of a visited tile)."""
     from vlm_training_amd import ops
     cu, msl, scale = t["cu_seqlens"], w.max_seqlen, w.D ** -0.5
-    idx, n = ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k)
+    idx, n, sel = ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k, return_scores=True)
     out, lse = ops.attn_fwd(t["q"], t["k"], t["v"], idx, n, cu, msl, scale)
     ms = timed(lambda: ops.attn_mass(t["q"], t["k"], lse, idx, n, cu, msl, scale), iters)
-    S = w.pair_counts()[1]
-    return {"ms": ms, "selected_pair_TFLOP/s": 2.0 * w.Hq * w.D * S / ms / 1e9,
-            "partial_table_GB/s": 2.0 * w.Hkv * 4 * S / ms / 1e6}
+    P, S = w.pair_counts()
+    res = {"attn_mass": {"ms": ms, "selected_pair_TFLOP/s": 2.0 * w.Hq * w.D * S / ms / 1e9,
+                         "partial_table_GB/s": 2.0 * w.Hkv * 4 * S / ms / 1e6}}
+    mass = ops.attn_mass(t["q"], t["k"], lse, idx, n, cu, msl, scale)
+    res["index_topk_with_scores_ms"] = timed(
+        lambda: ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k, return_scores=True), iters)
+    res["indexer_kl_ms"] = timed(lambda: ops.indexer_kl(sel, mass, n), iters)
+    loss, dscore = ops.indexer_kl(sel, mass, n)
+    res["mean_kl"] = float(loss.mean())
+    if w.Di in (64, 128) and w.Hi <= 64:
+        ms = timed(lambda: ops.indexer_bwd(t["q_idx"], t["k_idx"], t["w_idx"], idx, n, dscore, cu, msl), iters)
+        res["indexer_bwd"] = {"ms": ms, "causal_pair_TFLOP/s": 8.0 * w.Hi * w.Di * P / ms / 1e9}
+    return res
 
 
 def vision_tower_operator(dev, iters):
@@ -304,7 +315,7 @@ def main():
     result["adjacent_kernels"] = prologue_stage(w, dev, it)
     result["reference_operator"] = reference_operator(w, t, it)
     result["vision_tower_operator"] = vision_tower_operator(dev, it)
-    result["indexer_target"] = indexer_target_stage(w, t, it)
+    result["indexer_training"] = indexer_target_stage(w, t, it)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, torch.get_num_threads())
     print(json.dumps(result))

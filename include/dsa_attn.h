@@ -104,7 +104,7 @@ int dsa_indexer_bwd(const void *q_idx, const void *k_idx, const void *w_idx, con
                     const float *dscore, const int32_t *cu_seqlens, int T, int N, int Hi, int Di, int K, float scale,
                     int dtype, int max_seqlen, void *dq_idx, void *dk_idx, float *dw, void *ws, size_t ws_bytes,
                     void *stream);
-size_t dsa_indexer_bwd_workspace_bytes(int T, int max_seqlen);
+size_t dsa_indexer_bwd_workspace_bytes(int T, int Di, int max_seqlen);
 
 /*
  * Stage D3 - attention forward over the selected keys (idx/n), or over every causal key of the own

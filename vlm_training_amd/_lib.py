@@ -31,7 +31,7 @@ _SIGNATURES = {
     "dsa_indexer_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                 c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                                 c_void_p]),
-    "dsa_indexer_bwd_workspace_bytes": (c_size_t, [c_int, c_int]),
+    "dsa_indexer_bwd_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "dsa_attn_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                              c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "dsa_attn_fwd_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),

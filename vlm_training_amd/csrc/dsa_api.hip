@@ -28,7 +28,9 @@ hipError_t dsa_launch_gather_dq(const void *dout, const void *q, const void *k, 
                                 hipStream_t stream);
 hipError_t dsa_launch_indexer_bwd(const void *q_idx, const void *k_idx, const void *w_idx, const float *dscore,
                                   const uint32_t *bitmap, int32_t *prefix, int ldw, const int32_t *cu, int N, int T, int Hi,
-                                  int Di, int K, float cscale, void *dq_idx, void *dk_idx, float *dw, hipStream_t stream);
+                                  int Di, int K, float cscale, void *dq_idx, void *dk_idx, float *dw, float *partial,
+                                  hipStream_t stream);
+size_t dsa_indexer_bwd_partial_bytes(int T, int Di, int ldw);
 hipError_t dsa_launch_tile_mass(const void *q, const void *k, const float *lse, const uint32_t *bitmap, int ldw,
                                 const int32_t *n, const int32_t *cu, int N, int T, int Hq, int Hkv, int D, int K,
                                 float scale, float *partial, float *mass, hipStream_t stream);
@@ -278,9 +280,10 @@ extern "C" int dsa_attn_mass(const void *q, const void *k, const float *lse, con
 }
 
 // ---- indexer backward: gradients of the selected scores w.r.t. the indexer's inputs --------------------
-extern "C" size_t dsa_indexer_bwd_workspace_bytes(int T, int max_seqlen) {
+extern "C" size_t dsa_indexer_bwd_workspace_bytes(int T, int Di, int max_seqlen) {
     if (T <= 0) return 0;
-    return 2 * align_up((size_t)T * bitmap_ldw(max_seqlen) * 4, 256);      // selection bitmap + slot prefix table
+    const int ldw = bitmap_ldw(max_seqlen);                    // selection bitmap + slot prefix table + partial dk sums
+    return 2 * align_up((size_t)T * ldw * 4, 256) + align_up(dsa_indexer_bwd_partial_bytes(T, Di, ldw), 256);
 }
 
 extern "C" int dsa_indexer_bwd(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *idx, const int32_t *n,
@@ -295,16 +298,19 @@ extern "C" int dsa_indexer_bwd(const void *q_idx, const void *k_idx, const void 
     if (!q_idx || !k_idx || !w_idx || !idx || !n || !dscore || !dq_idx || !dk_idx || !dw) return fail(DSA_ERR_ARG, "null tensor pointer");
     if (max_seqlen < 1 || max_seqlen > (T > 0 ? T : 1)) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
     if (T == 0) return DSA_OK;
-    const size_t need = dsa_indexer_bwd_workspace_bytes(T, max_seqlen);
+    const size_t need = dsa_indexer_bwd_workspace_bytes(T, Di, max_seqlen);
     if (!ws || ws_bytes < need) return fail(DSA_ERR_WORKSPACE, "indexer backward workspace: have %zu bytes, need %zu", ws_bytes, need);
     const int ldw = bitmap_ldw(max_seqlen);
     if ((size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);
     hipStream_t st = (hipStream_t)stream;
+    const size_t bm = align_up((size_t)T * ldw * 4, 256);
     uint32_t *bitmap = (uint32_t *)ws;
-    int32_t *prefix = (int32_t *)((char *)ws + need / 2);
+    int32_t *prefix = (int32_t *)((char *)ws + bm);
+    float *partial = (float *)((char *)ws + 2 * bm);
     hipError_t e = dsa_launch_bitmap(idx, n, cu, N, T, K, ldw, bitmap, st);
     if (e != hipSuccess) return hip_fail(e, "bitmap launch");
-    e = dsa_launch_indexer_bwd(q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, Di, K, scale, dq_idx, dk_idx, dw, st);
+    e = dsa_launch_indexer_bwd(q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, Di, K, scale, dq_idx, dk_idx, dw,
+                               partial, st);
     if (e != hipSuccess) return hip_fail(e, "indexer backward launch");
     return DSA_OK;
 }

@@ -492,8 +492,14 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     const int ntiles = min(qc0 + QBW - 1, L - 1) / 32 + 1;
     const uint32_t *wrow = bitmap + (int64_t)t * ldw;
     const float *drow = dscore + (int64_t)t * K;
-    uint32_t word_next = wrow[0];
+    // selection words run two tiles ahead of the compute and the gradients of a tile's keys one tile ahead: lane j
+    // fetches the gradient of key column j of the next tile (both halves of the wave the same)
+    uint32_t word_cur = qcol < L ? wrow[0] : 0u, word_nx = qcol < L ? wrow[min(1, ntiles - 1)] : 0u;
     int seen = 0;
+    auto fetch_dl = [&](uint32_t word, int before) {
+        return drow[min(before + (int)__popc(word & ((1u << j) - 1u)), K - 1)];
+    };
+    float dl_nx = fetch_dl(word_cur, 0);
     f32x16 acc[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
@@ -508,13 +514,12 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
 #define IDXQ_COMPUTE(TILE, BUF)                                                                     \
     {                                                                                              \
         const unsigned char *kt = lds[BUF];                                                        \
-        const uint32_t word_full = qcol < L ? word_next : 0u;                                      \
-        word_next = wrow[min((TILE) + 1, ntiles - 1)];                                             \
-        /* lane j fetches the gradient of key column j of the tile (both halves of the wave the same) */ \
-        const bool mine = (word_full >> j) & 1u;                                                   \
-        float dl = drow[min(seen + (int)__popc(word_full & ((1u << j) - 1u)), K - 1)];             \
-        dl = mine ? dl : 0.f;                                                                      \
+        const uint32_t word_full = word_cur;                                                       \
+        const float dl = ((word_full >> j) & 1u) ? dl_nx : 0.f;                                    \
         seen += __popc(word_full);                                                                 \
+        word_cur = word_nx;                                                                        \
+        dl_nx = fetch_dl(word_cur, seen);                /* for the next tile */                   \
+        { const uint32_t wl = wrow[min((TILE) + 2, ntiles - 1)]; word_nx = qcol < L ? wl : 0u; }   \
         f32x16 sacc = zero16();                                                                    \
         {                                                                                          \
             bf16x8 ka[KS];                                                                         \
@@ -550,18 +555,20 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     }
 }
 
-// key side.  Workgroup = 4 waves x 32 keys = one 128-key tile of a segment; block b of its walk = the 32 heads
-// [32*(b % HB), +32) of query c0 + b / HB.
+// key side.  Workgroup = 4 waves x 32 keys = one 128-key tile of a segment; step b of its walk = all heads
+// (HB blocks of 32) of query L-1-b: from the end of the segment down to the tile, so that the workgroups of a
+// segment that run side by side read the same index-query rows at about the same time and share them in L2.
 template <int D, int GSHIFT>
 __global__ __launch_bounds__(256) void dsa_tile_idxk_kernel(
     const bf16_t *__restrict__ q_idx, const bf16_t *__restrict__ k_idx, const bf16_t *__restrict__ w_idx,
     const float *__restrict__ dscore, const uint32_t *__restrict__ bitmap, const int32_t *__restrict__ prefix, int ldw,
-    const int32_t *__restrict__ cu, int N, int T, int Hi, int K, float cscale, bf16_t *__restrict__ dk_idx) {
-    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / 256;
-    constexpr int NBUF = 2, HB = (1 << GSHIFT) / 32;
-    static_assert(GSHIFT >= 5 && LOADS >= 1, "blocks of 32 heads of one query");
-    __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][TILE_B];
-    __shared__ __attribute__((aligned(16))) float w_s[NBUF][32];
+    const int32_t *__restrict__ cu, int N, int T, int Hi, int K, float cscale, int chunk_steps,
+    float *__restrict__ partial) {
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>();
+    constexpr int NBUF = 2, HB = (1 << GSHIFT) / 32, LOADS = HB * 32 * CPR / 256;
+    static_assert(GSHIFT >= 5 && LOADS >= 1, "steps of 32*HB heads of one query");
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][HB][TILE_B];
+    __shared__ __attribute__((aligned(16))) float w_s[NBUF][HB * 32];
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
     LaneOffsets<D> lo;
@@ -580,92 +587,122 @@ __global__ __launch_bounds__(256) void dsa_tile_idxk_kernel(
     f32x16 dkacc[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) dkacc[dt] = zero16();
-    const int nq = L - c0, nblocks = nq * HB;            // queries c0 .. L-1 can have selected keys of this tile
+    // queries L-1 down to c0 can have selected keys of this tile; the walk is cut into pieces of chunk_steps queries
+    // (blockIdx.y), each piece leaving a partial sum: a tile at the start of a long segment would otherwise be one
+    // long serial walk
+    const int st0 = blockIdx.y * chunk_steps, nsteps = min(L - c0 - st0, chunk_steps);
+    if (nsteps <= 0) return;
 
-    // selection words and slot bases of this wave's key column for 64 consecutive queries, one query per lane
-    auto fetch_words = [&](int chunk, uint32_t &wq, int32_t &bq) {
-        const int qc = min(c0 + chunk * 64 + lane, L - 1);
-        const int64_t o = (int64_t)(s0 + qc) * ldw + kw;
+    // selection word and slot base of (query of a step, this wave's key column): fetched two LOAD calls before the
+    // LOAD that forms the gradient's address from them (register set s serves the odd steps, set 1 the even ones)
+    const int last_step = nsteps - 1;
+    auto word_of = [&](int step, uint32_t &wq, int32_t &bq) {
+        const int64_t o = (int64_t)(s0 + L - 1 - st0 - min(step, last_step)) * ldw + kw;
         wq = kw_ok ? bitmap[o] : 0u;
         bq = prefix[o];
     };
-    uint32_t wq_cur, wq_nxt;
-    int32_t bq_cur, bq_nxt;
-    fetch_words(0, wq_cur, bq_cur);
-    fetch_words(1, wq_nxt, bq_nxt);
-    int cur_chunk = 0;
+    uint32_t wordp[2], word0;
+    int32_t basep[2], base0;
+    word_of(0, word0, base0);
+    word_of(1, wordp[0], basep[0]);
+    word_of(2, wordp[1], basep[1]);
 
     u32x4 qst[2][LOADS];
     float dl_st[2] = {0.f, 0.f}, dl_buf[NBUF] = {0.f, 0.f};
     bool sel_st[2] = {false, false};
     uint32_t w_st[2] = {0u, 0u};
-#define IDXK_LOAD(SET, BLK)                                                                         \
+#define IDXK_LOAD(SET, STEP)                                                                        \
     {                                                                                              \
-        const int rel = (BLK) / HB, hb = (BLK) % HB, qc = c0 + rel;                                \
+        const int rel = (STEP), qc = L - 1 - st0 - rel;                                            \
         _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                        \
             const int c = i * 256 + tid;                                                           \
-            const int row = c / CPR, ch = c % CPR;                                                 \
-            const int hd = min(hb * 32 + row, Hi - 1);                                             \
-            qst[SET][i] = *reinterpret_cast<const u32x4 *>(q_idx + ((int64_t)(s0 + qc) * Hi + hd) * D + ch * 8); \
+            const int row = c / CPR, ch = c % CPR;       /* row = head, padded to 32*HB */          \
+            qst[SET][i] = *reinterpret_cast<const u32x4 *>(q_idx + ((int64_t)(s0 + qc) * Hi + min(row, Hi - 1)) * D + ch * 8); \
         }                                                                                          \
-        w_st[SET] = reinterpret_cast<const unsigned short *>(w_idx)[(int64_t)(s0 + qc) * Hi + min(hb * 32 + (tid & 31), Hi - 1)]; \
-        if ((rel >> 6) != cur_chunk) {                   /* wave-uniform: move on to the next 64 queries */ \
-            wq_cur = wq_nxt;                                                                       \
-            bq_cur = bq_nxt;                                                                       \
-            cur_chunk = rel >> 6;                                                                  \
-            fetch_words(cur_chunk + 1, wq_nxt, bq_nxt);                                            \
-        }                                                                                          \
-        const uint32_t word = __builtin_amdgcn_readlane(wq_cur, rel & 63);                         \
-        const int base = __builtin_amdgcn_readlane(bq_cur, rel & 63);                              \
+        w_st[SET] = reinterpret_cast<const unsigned short *>(w_idx)[(int64_t)(s0 + qc) * Hi + min(tid & (32 * HB - 1), Hi - 1)]; \
+        const uint32_t word = wordp[SET];                                                          \
+        const int base = basep[SET];                                                               \
+        word_of(rel + 2, wordp[SET], basep[SET]);        /* for this register set's next step */    \
         sel_st[SET] = (word >> j) & 1u;                                                            \
         dl_st[SET] = dscore[(int64_t)(s0 + qc) * K + min(base + (int)__popc(word & ((1u << j) - 1u)), K - 1)]; \
     }
-#define IDXK_STORE(SET, BUF, BLK)                                                                   \
+#define IDXK_STORE(SET, BUF, STEP)                                                                  \
     {                                                                                              \
-        const int hb = (BLK) % HB;                                                                 \
         const u32x4 z4 = {0u, 0u, 0u, 0u};                                                         \
         _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                        \
             const int c = i * 256 + tid;                                                           \
             const int row = c / CPR, ch = c % CPR;                                                 \
             /* padded heads are zeroed: they add nothing to dK */                                   \
-            *reinterpret_cast<u32x4 *>(&lds[BUF][tile_off<D>(row, ch)]) = hb * 32 + row < Hi ? qst[SET][i] : z4; \
+            *reinterpret_cast<u32x4 *>(&lds[BUF][row >> 5][tile_off<D>(row & 31, ch)]) = row < Hi ? qst[SET][i] : z4; \
         }                                                                                          \
-        if (tid < 32) w_s[BUF][tid] = hb * 32 + tid < Hi ? __uint_as_float(w_st[SET] << 16) : 0.f;  \
+        if (tid < 32 * HB) w_s[BUF][tid] = tid < Hi ? __uint_as_float(w_st[SET] << 16) : 0.f;       \
         dl_buf[BUF] = sel_st[SET] ? dl_st[SET] : 0.f;                                              \
     }
-#define IDXK_COMPUTE(BLK, BUF)                                                                      \
+#define IDXK_COMPUTE(STEP, BUF)                                                                     \
     {                                                                                              \
-        const unsigned char *qt = lds[BUF];                                                        \
-        const float dl = dl_buf[BUF];                    /* gradient of (query of the block, this lane's key) */ \
-        f32x16 sacc = zero16();                                                                    \
-        {                                                                                          \
-            bf16x8 qa[KS];                                                                         \
-            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) qa[ks] = lo.rowop(qt, ks);           \
-            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) sacc = mfma32(qa[ks], kB[ks], sacc); \
-            sched_reads_ahead<KS, 4, 1>();                                                         \
+        const float dl = dl_buf[BUF];                    /* gradient of (query of the step, this lane's key) */ \
+        _Pragma("unroll") for (int hb = 0; hb < HB; ++hb) {                                        \
+            const unsigned char *qt = lds[BUF][hb];                                                \
+            f32x16 sacc = zero16();                                                                \
+            {                                                                                      \
+                bf16x8 qa[KS];                                                                     \
+                _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) qa[ks] = lo.rowop(qt, ks);       \
+                _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) sacc = mfma32(qa[ks], kB[ks], sacc); \
+            }                                                                                      \
+            float gs[16];                                                                          \
+            _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {                                     \
+                const f32x4 w4 = *reinterpret_cast<const f32x4 *>(&w_s[BUF][hb * 32 + 8 * g4 + 4 * h]); \
+                _Pragma("unroll") for (int e = 0; e < 4; ++e) gs[4 * g4 + e] = sacc[4 * g4 + e] > 0.f ? dl * w4[e] : 0.f; \
+            }                                                                                      \
+            const bf16x8 gB0 = pack8(gs), gB1 = pack8(gs + 8);                                     \
+            _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                    \
+                mfma32_acc(dkacc[dt], lo.trop(qt, 0, dt), gB0);                                    \
+                mfma32_acc(dkacc[dt], lo.trop(qt, 1, dt), gB1);                                    \
+            }                                                                                      \
         }                                                                                          \
-        float gs[16];                                                                              \
-        _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {                                         \
-            const f32x4 w4 = *reinterpret_cast<const f32x4 *>(&w_s[BUF][8 * g4 + 4 * h]);          \
-            _Pragma("unroll") for (int e = 0; e < 4; ++e) gs[4 * g4 + e] = sacc[4 * g4 + e] > 0.f ? dl * w4[e] : 0.f; \
-        }                                                                                          \
-        const bf16x8 gB0 = pack8(gs), gB1 = pack8(gs + 8);                                         \
-        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
-            mfma32_acc(dkacc[dt], lo.trop(qt, 0, dt), gB0);                                        \
-            mfma32_acc(dkacc[dt], lo.trop(qt, 1, dt), gB1);                                        \
-        }                                                                                          \
-        sched_reads_ahead<2 * DT, 3, 2>();                                                         \
     }
-    IDXK_LOAD(0, 0)
-    TILE_PIPELINE(nblocks, IDXK_LOAD, IDXK_STORE, IDXK_COMPUTE)
+    {                                                    // step 0 into register set 0, with the words fetched above
+        const uint32_t w1 = wordp[0];
+        const int32_t b1 = basep[0];
+        wordp[0] = word0;
+        basep[0] = base0;
+        IDXK_LOAD(0, -2 + 2)                             /* consumes (word0, base0); its own prefetch is overwritten below */
+        wordp[0] = w1;
+        basep[0] = b1;
+    }
+    TILE_PIPELINE(nsteps, IDXK_LOAD, IDXK_STORE, IDXK_COMPUTE)
 #undef IDXK_LOAD
 #undef IDXK_STORE
 #undef IDXK_COMPUTE
 
     if (key_ok) {
-        bf16_t *pk = dk_idx + krow * D;
+        float *pk = partial + ((int64_t)blockIdx.y * T + krow) * D + 4 * h;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) store_c_tile(pk + dt * 32, dkacc[dt], cscale, h);
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const f32x4 o4 = {dkacc[dt][4 * g4] * cscale, dkacc[dt][4 * g4 + 1] * cscale, dkacc[dt][4 * g4 + 2] * cscale,
+                                  dkacc[dt][4 * g4 + 3] * cscale};
+                *reinterpret_cast<f32x4 *>(pk + dt * 32 + 8 * g4) = o4;
+            }
+    }
+}
+
+// dk_idx[s,:] = sum of the partial sums of the pieces of its tile's walk, in piece order
+__global__ __launch_bounds__(256) void dsa_idxk_reduce_kernel(const float *__restrict__ partial,
+                                                               const int32_t *__restrict__ cu, int N, int T, int D,
+                                                               int chunk_steps, bf16_t *__restrict__ dk_idx) {
+    const int s = blockIdx.x * (256 / 32) + (threadIdx.x >> 5), c4 = (threadIdx.x & 31) * 4;   // 32 threads x 4 columns per pass
+    if (s >= T) return;
+    const int seg = find_segment(cu, N, s);
+    const int s0 = cu[seg], L = cu[seg + 1] - s0;
+    const int c0 = ((s - s0) >> 7) << 7;
+    const int pieces = (L - c0 + chunk_steps - 1) / chunk_steps;
+    for (int c = c4; c < D; c += 128) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int pc = 0; pc < pieces; ++pc) acc += *reinterpret_cast<const f32x4 *>(partial + ((int64_t)pc * T + s) * D + c);
+        const u32x2 o = {pack2bf(acc[0], acc[1]), pack2bf(acc[2], acc[3])};
+        *reinterpret_cast<u32x2 *>(dk_idx + (int64_t)s * D + c) = o;
     }
 }
 
@@ -1289,31 +1326,37 @@ extern "C" hipError_t dsa_launch_tile_mass(const void *q, const void *k, const f
 }
 // indexer backward: prefix table, query side (dq_idx, dw), key side (dk_idx).  D = indexer head_dim (64 or 128),
 // at most 64 indexer heads.
+#define IDXK_CHUNK 512                                   // queries per piece of a key tile's walk
 template <int D, int GS>
 static void launch_idx_bwd_i(hipStream_t stream, const void *q_idx, const void *k_idx, const void *w_idx, const float *dscore,
                              const uint32_t *bitmap, const int32_t *prefix, int ldw, const int32_t *cu, int N, int T, int Hi,
-                             int K, float cscale, void *dq_idx, void *dk_idx, float *dw) {
+                             int K, float cscale, void *dq_idx, void *dk_idx, float *dw, float *partial) {
     constexpr int NW = tile_waves<D>();
     const dim3 gq((unsigned)((int64_t)T / ((32 * NW) >> GS) + N + 1));
     hipLaunchKernelGGL((dsa_tile_idxq_kernel<D, GS, NW>), gq, dim3(64 * NW), 0, stream, (const bf16_t *)q_idx,
                        (const bf16_t *)k_idx, (const bf16_t *)w_idx, dscore, bitmap, ldw, cu, N, T, Hi, K, cscale,
                        (bf16_t *)dq_idx, dw);
-    const dim3 gk((unsigned)((int64_t)T / 128 + N + 1));
+    const dim3 gk((unsigned)((int64_t)T / 128 + N + 1), (unsigned)((ldw * 32 + IDXK_CHUNK - 1) / IDXK_CHUNK));
     hipLaunchKernelGGL((dsa_tile_idxk_kernel<D, GS>), gk, dim3(256), 0, stream, (const bf16_t *)q_idx, (const bf16_t *)k_idx,
-                       (const bf16_t *)w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, (bf16_t *)dk_idx);
+                       (const bf16_t *)w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, IDXK_CHUNK, partial);
+    hipLaunchKernelGGL(dsa_idxk_reduce_kernel, dim3((unsigned)((T + 7) / 8)), dim3(256), 0, stream, partial, cu, N, T, D,
+                       IDXK_CHUNK, (bf16_t *)dk_idx);
+}
+extern "C" size_t dsa_indexer_bwd_partial_bytes(int T, int Di, int ldw) {
+    return (size_t)((ldw * 32 + IDXK_CHUNK - 1) / IDXK_CHUNK) * T * Di * 4;
 }
 extern "C" hipError_t dsa_launch_indexer_bwd(const void *q_idx, const void *k_idx, const void *w_idx, const float *dscore,
                                              const uint32_t *bitmap, int32_t *prefix, int ldw, const int32_t *cu, int N,
                                              int T, int Hi, int Di, int K, float cscale, void *dq_idx, void *dk_idx,
-                                             float *dw, hipStream_t stream) {
+                                             float *dw, float *partial, hipStream_t stream) {
     if (Hi < 1 || Hi > 64 || !(Di == 64 || Di == 128)) return hipErrorInvalidValue;
     hipLaunchKernelGGL(dsa_bitmap_prefix_kernel, dim3(T), dim3(64), 0, stream, bitmap, ldw, prefix);
     if (Di == 128) {
-        if (Hi > 32) launch_idx_bwd_i<128, 6>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw);
-        else launch_idx_bwd_i<128, 5>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw);
+        if (Hi > 32) launch_idx_bwd_i<128, 6>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw, partial);
+        else launch_idx_bwd_i<128, 5>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw, partial);
     } else {
-        if (Hi > 32) launch_idx_bwd_i<64, 6>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw);
-        else launch_idx_bwd_i<64, 5>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw);
+        if (Hi > 32) launch_idx_bwd_i<64, 6>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw, partial);
+        else launch_idx_bwd_i<64, 5>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw, partial);
     }
     return hipGetLastError();
 }

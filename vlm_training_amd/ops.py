@@ -169,7 +169,7 @@ def indexer_bwd(q_idx, k_idx, w_idx, idx, n, dscore, cu_seqlens, max_seqlen: int
     dk = torch.empty_like(ki)
     dw = torch.empty((T, Hi), dtype=torch.float32, device=qi.device)
     max_seqlen = T if max_seqlen is None else int(max_seqlen)
-    ws_bytes = lib.dsa_indexer_bwd_workspace_bytes(T, max_seqlen)
+    ws_bytes = lib.dsa_indexer_bwd_workspace_bytes(T, Di, max_seqlen)
     ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=qi.device)
     rc = lib.dsa_indexer_bwd(_ptr(qi), _ptr(ki), _ptr(wi), _ptr(idx), _ptr(n), _ptr(dscore.contiguous()), _ptr(cu), T,
                              cu.numel() - 1, Hi, Di, K, scale, _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(dq), _ptr(dk), _ptr(dw),
