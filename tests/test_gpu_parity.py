@@ -660,6 +660,13 @@ def test_indexer_training_step_end_to_end():
                                           indexer_w=wi, top_k=w.top_k, return_indices=True, return_mass=True)
     loss = M.indexer_kl_loss(qi, ki, wi, mass, d["cu_seqlens"], w.max_seqlen, w.top_k)
     (loss * 3.0).backward()
+    # the same with the selection and its scores handed over by the operator (no second run of the indexer)
+    o2, i2, n2, m2, s2 = M.dsa_varlen_attn(d["q"], d["k"], d["v"], d["cu_seqlens"], w.max_seqlen, indexer_q=qi, indexer_k=ki,
+                                           indexer_w=wi, top_k=w.top_k, return_indices=True, return_mass=True,
+                                           return_scores=True)
+    assert torch.equal(o2, out) and torch.equal(i2, idx) and torch.equal(m2, mass)
+    loss2 = M.indexer_kl_loss(qi, ki, wi, m2, d["cu_seqlens"], w.max_seqlen, w.top_k, selection=(i2, n2, s2))
+    assert torch.equal(loss2, loss)
     rq, rk, rw = (t[x].float().requires_grad_(True) for x in ("q_idx", "k_idx", "w_idx"))
     sel = R.selected_scores(rq, rk, rw, idx.cpu(), n.cpu(), list(w.cu))
     ref = R.indexer_kl(sel, mass.cpu(), n.cpu()).mean()

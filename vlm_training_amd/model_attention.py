@@ -17,7 +17,7 @@ import torch
 
 from .ops import dsa_varlen_attn
 
-_DSA_KEYS = ("indexer_q", "indexer_k", "indexer_w", "top_k", "index_scale", "return_indices", "return_mass")
+_DSA_KEYS = ("indexer_q", "indexer_k", "indexer_w", "top_k", "index_scale", "return_indices", "return_mass", "return_scores")
 
 
 def varlen_attn(query, key, value, cu_seq_q, cu_seq_k, max_q, max_k, is_causal=None, return_aux=None,

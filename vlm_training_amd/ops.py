@@ -180,9 +180,10 @@ def indexer_bwd(q_idx, k_idx, w_idx, idx, n, dscore, cu_seqlens, max_seqlen: int
 
 class _IndexerKL(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q_idx, k_idx, w_idx, mass, cu_seqlens, max_seqlen, top_k, index_scale):
+    def forward(ctx, q_idx, k_idx, w_idx, mass, cu_seqlens, max_seqlen, top_k, index_scale, idx=None, n=None, sel=None):
         T = q_idx.shape[0]
-        idx, n, sel = index_topk(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen, top_k, index_scale, return_scores=True)
+        if sel is None:
+            idx, n, sel = index_topk(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen, top_k, index_scale, return_scores=True)
         loss_rows, dscore = indexer_kl(sel, mass, n, grad_scale=1.0 / max(T, 1))
         ctx.save_for_backward(q_idx, k_idx, w_idx, idx, n, dscore, cu_seqlens)
         ctx.max_seqlen, ctx.index_scale = max_seqlen, index_scale
@@ -194,20 +195,24 @@ class _IndexerKL(torch.autograd.Function):
         dq, dk, dw = indexer_bwd(q_idx, k_idx, w_idx, idx, n, dscore, cu, ctx.max_seqlen, ctx.index_scale)
         g = g.to(torch.float32)
         return ((dq.float() * g).to(q_idx.dtype), (dk.float() * g).to(k_idx.dtype), (dw * g).to(w_idx.dtype), None, None,
-                None, None, None)
+                None, None, None, None, None, None)
 
 
 @torch.compiler.disable
 def indexer_kl_loss(indexer_q, indexer_k, indexer_w, mass, cu_seqlens, max_seqlen: Optional[int], top_k: int,
-                    index_scale: Optional[float] = None):
+                    index_scale: Optional[float] = None, selection=None):
     """Training loss of the DSA indexer: mean over the packed tokens of KL(mass[t] || softmax of the indexer's scores
     over the keys it selected for t), differentiable w.r.t. indexer_q (T,Hi,Di), indexer_k (T,Di), indexer_w (T,Hi).
 
     ``mass`` is the detached target ``dsa_varlen_attn(..., return_mass=True)`` returned for the same indexer
-    inputs and top_k (the selection is recomputed here and is the same: it is deterministic)."""
+    inputs and top_k.  ``selection=(idx, n, scores)`` as returned by ``dsa_varlen_attn(..., return_indices=True,
+    return_scores=True)`` saves a second run of the indexer; without it the selection is recomputed here (it is
+    deterministic, hence the same)."""
     T = indexer_q.shape[0]
     max_seqlen = T if max_seqlen is None else int(max_seqlen)
-    return _IndexerKL.apply(indexer_q, indexer_k, indexer_w, mass, cu_seqlens, max_seqlen, int(top_k), index_scale)
+    idx, n, sel = selection if selection is not None else (None, None, None)
+    return _IndexerKL.apply(indexer_q, indexer_k, indexer_w, mass, cu_seqlens, max_seqlen, int(top_k), index_scale, idx, n,
+                            sel)
 
 
 def set_tile_crossover(crossover: int) -> int:
@@ -383,7 +388,7 @@ class _DsaVarlenAttn(torch.autograd.Function):
 def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, indexer_q=None, indexer_k=None, indexer_w=None,
                     top_k: Optional[int] = None, index_scale: Optional[float] = None,
                     softmax_scale: Optional[float] = None, return_indices: bool = False, causal: bool = True,
-                    return_mass: bool = False):
+                    return_mass: bool = False, return_scores: bool = False):
     """Packed causal attention over ``cu_seqlens`` segments, optionally sparsified by the DSA indexer.
 
     q (T,Hq,D), k/v (T,Hkv,D) contiguous, cu_seqlens (N+1,) int32 on the device, max_seqlen host int
@@ -395,7 +400,9 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, in
     the top_k keys of its causal window under (indexer score descending, key index ascending).
     ``return_mass=True`` (with the indexer inputs) also returns the (T, top_k) fp32 table of head-averaged attention
     probabilities of the selected keys, rows summing to one and aligned with the indices: the detached target of the
-    KL loss that trains the indexer.
+    KL loss that trains the indexer.  ``return_scores=True`` appends the (T, top_k) fp32 indexer scores of the selected
+    keys (every row is then scored, also those whose whole window is selected), which ``indexer_kl_loss`` takes as
+    ``selection=(idx, n, scores)`` instead of running the indexer again.
     Gradients flow to q, k, v only.  A head_dim between the kernels' 64 / 128 / 256 is zero-padded to the
     next one and the output cut back (the scale stays that of the true head_dim).  ``causal=False`` (dense only) attends every key of the own segment, the
     vision towers' form of the call (models/qwen3_vl/model.py:423-428).
@@ -415,9 +422,13 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, in
         if indexer_q.shape[0] != T:
             raise ValueError("indexer tensors must cover the same T packed tokens as q")
         with torch.no_grad():
-            idx, n = index_topk(indexer_q, indexer_k, indexer_w, cu, int(max_seqlen), int(top_k), index_scale)
-    elif return_indices:
-        raise ValueError("return_indices needs the indexer inputs")
+            if return_scores:
+                idx, n, sel_scores = index_topk(indexer_q, indexer_k, indexer_w, cu, int(max_seqlen), int(top_k), index_scale,
+                                                return_scores=True)
+            else:
+                idx, n = index_topk(indexer_q, indexer_k, indexer_w, cu, int(max_seqlen), int(top_k), index_scale)
+    elif return_indices or return_scores:
+        raise ValueError("return_indices / return_scores need the indexer inputs")
     d_kernel = next((d for d in _KERNEL_HEAD_DIMS if d >= D), None)
     if d_kernel is None:
         raise ValueError(f"head_dim {D} is beyond the kernels' largest ({_KERNEL_HEAD_DIMS[-1]})")
@@ -433,5 +444,6 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, in
         out, mass = out
     if d_kernel != D:
         out = out[..., :D]
-    res = (out,) + ((idx, n) if return_indices else ()) + ((mass,) if return_mass else ())
+    res = (out,) + ((idx, n) if return_indices else ()) + ((mass,) if return_mass else ()) + (
+        (sel_scores,) if return_scores else ())
     return res if len(res) > 1 else out
