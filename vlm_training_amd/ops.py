@@ -192,10 +192,10 @@ class _IndexerKL(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g):
         q_idx, k_idx, w_idx, idx, n, dscore, cu = ctx.saved_tensors
-        dq, dk, dw = indexer_bwd(q_idx, k_idx, w_idx, idx, n, dscore, cu, ctx.max_seqlen, ctx.index_scale)
-        g = g.to(torch.float32)
-        return ((dq.float() * g).to(q_idx.dtype), (dk.float() * g).to(k_idx.dtype), (dw * g).to(w_idx.dtype), None, None,
-                None, None, None, None, None, None)
+        # the gradients are linear in dscore: scale the (T,K) table by the incoming gradient, not the three results
+        dq, dk, dw = indexer_bwd(q_idx, k_idx, w_idx, idx, n, dscore * g.to(torch.float32), cu, ctx.max_seqlen,
+                                 ctx.index_scale)
+        return (dq.to(q_idx.dtype), dk.to(k_idx.dtype), dw.to(w_idx.dtype), None, None, None, None, None, None, None, None)
 
 
 @torch.compiler.disable
