@@ -361,7 +361,10 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
         qB[ks] = row_ok ? load_bf16x8(q + ((int64_t)t * Hq + hq) * D + 16 * ks + 8 * h) : zero_bf16x8();
-    const float lse2 = lse[(int64_t)hq * T + t] * LOG2E_F;
+    // padding rows (head >= G, query past the segment) get lse = +inf: their P is exp2(-inf) = 0 in the head sums.
+    // Keys that are not selected need no masking: their sums are never stored.
+    const float lse_row = lse[(int64_t)hq * T + t];
+    const float lse2 = row_ok ? lse_row * LOG2E_F : INFINITY;
     const int ntiles = min(qc0 + QBW - 1, L - 1) / 32 + 1;
     const uint32_t *wrow = bitmap + (int64_t)t * ldw;
     uint32_t word_next = wrow[0];
@@ -380,7 +383,6 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
         /* padding lanes of a query (head >= G) compute nothing but take their share of the stores */ \
         const uint32_t word_full = qcol < L ? word_next : 0u;                                      \
         word_next = wrow[min((TILE) + 1, ntiles - 1)];                                             \
-        const uint32_t word = (row_ok ? word_full : 0u) >> (4 * h); /* element vi then sits at bit 8*(vi/4) + vi%4 */ \
         f32x16 sacc = zero16();                                                                    \
         {                                                                                          \
             bf16x8 ka[KS];                                                                         \
@@ -389,10 +391,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
             sched_reads_ahead<KS, 4, 1>();                                                         \
         }                                                                                          \
         float p[16];                                                                               \
-        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
-            const int kb = 8 * (vi >> 2) + (vi & 3);                                               \
-            p[vi] = fast_exp2(keep_or_neginf(fmaf(sacc[vi], scale_log2, -lse2), bit_mask(word, kb))); \
-        }                                                                                          \
+        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) p[vi] = fast_exp2(fmaf(sacc[vi], scale_log2, -lse2)); \
         _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) p[vi] = group_sum<GSHIFT>(p[vi]);        \
         /* the lanes of a query share the stores: lane `head` writes the elements vi = u*Gp + head */ \
         _Pragma("unroll") for (int u = 0; u < 16 / Gp; ++u) {                                      \
