@@ -624,7 +624,8 @@ def test_selected_scores_and_indexer_kl(segs, K):
 
 
 @pytest.mark.parametrize("Hi,Di,K,segs", [(8, 64, 16, (130, 64, 5)), (64, 128, 64, (300, 1, 77, 513)), (32, 64, 100, (50, 400)),
-                                           (40, 128, 8, (97, 200)), (64, 128, 512, (700,)), (8, 64, 16, (1700, 40, 600))])
+                                           (40, 128, 8, (97, 200)), (64, 128, 512, (700,)), (8, 64, 16, (1700, 40, 600)),
+                                           (4, 32, 128, (256, 512, 384))])
 def test_indexer_backward_matches_autograd_of_the_oracle(Hi, Di, K, segs):
     """dq_idx, dk_idx, dw for an arbitrary gradient at the selected scores, against torch autograd through the
     oracle's score formula on the same bf16 inputs.  Tolerance as for the attention gradients (bf16 outputs)."""

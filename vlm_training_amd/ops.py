@@ -165,6 +165,12 @@ def indexer_bwd(q_idx, k_idx, w_idx, idx, n, dscore, cu_seqlens, max_seqlen: int
     scale = index_scale if index_scale is not None else (Di ** -0.5) * (Hi ** -0.5)
     lib = _lib.load()
     qi, ki, wi = _as_bf16(q_idx), _as_bf16(k_idx), _as_bf16(w_idx)
+    d_kernel = next((d for d in (64, 128) if d >= Di), None)
+    if d_kernel is not None and d_kernel != Di:          # e.g. 32-wide index heads: zero columns change no score
+        pad = d_kernel - Di
+        dq, dk, dw = indexer_bwd(torch.nn.functional.pad(qi, (0, pad)), torch.nn.functional.pad(ki, (0, pad)), wi, idx, n,
+                                 dscore, cu_seqlens, max_seqlen, scale)
+        return dq[..., :Di].contiguous(), dk[..., :Di].contiguous(), dw
     dq = torch.empty_like(qi)
     dk = torch.empty_like(ki)
     dw = torch.empty((T, Hi), dtype=torch.float32, device=qi.device)
