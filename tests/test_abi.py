@@ -71,3 +71,59 @@ def test_workload_tables_match_the_measurement_plan():
     assert t["q"].dtype == torch.bfloat16 and t["cu_seqlens"].tolist() == [0, 2100, 2150]
     t2 = W.make_inputs(W.scaled(W.C3, (2100, 50), top_k=8), device="cpu")
     assert torch.equal(t["q"], t2["q"]) and torch.equal(t["k_idx"], t2["k_idx"])
+
+
+# ------------------------------------------------------------------------------------------------------------
+# the binding and the documentation follow the header
+# ------------------------------------------------------------------------------------------------------------
+def _header_prototypes():
+    """name -> list of parameter type strings, parsed from include/dsa_attn.h."""
+    text = open(os.path.join(ROOT, "include", "dsa_attn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"^\s*#.*$", "", text, flags=re.M)
+    protos = {}
+    for m in re.finditer(r"([A-Za-z_][\w \*]*?)\b(dsa_[a-z_0-9]+)\s*\(([^)]*)\)\s*;", text):
+        params = [p.strip() for p in m.group(3).split(",")]
+        if params == ["void"]:
+            params = []
+        protos[m.group(2)] = (m.group(1).strip(), [re.sub(r"\s*\b\w+$", "", p).strip() if not p.endswith("*") else p for p in params])
+    return protos
+
+
+def _ctype_of(c_type: str):
+    from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
+    t = c_type.replace("const ", "").strip()
+    if t.endswith("*"):
+        return c_char_p if t.startswith("char") else c_void_p
+    return {"int": c_int, "float": c_float, "int64_t": c_int64, "size_t": c_size_t}[t]
+
+
+def test_ctypes_signatures_follow_the_header_prototypes():
+    protos = _header_prototypes()
+    assert sorted(protos) == sorted(_lib.EXPORTS)
+    for name, (ret, params) in protos.items():
+        res, args = _lib._SIGNATURES[name]
+        assert len(args) == len(params), (name, len(args), len(params))
+        assert [_ctype_of(p) for p in params] == list(args), name
+        assert _ctype_of(ret) == res, name
+    assert len(protos["dsa_attn_fwd"][1]) == 21
+
+
+def test_integration_stub_matches_the_header():
+    """The ctypes stub a maintainer would copy out of the integration notes binds dsa_attn_fwd with the header's
+    argument list, and its example call passes one value per argument."""
+    from ctypes import c_float, c_int, c_size_t, c_void_p
+    doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    m = re.search(r"lib\.dsa_attn_fwd\.argtypes = \[([^\]]*)\]", doc)
+    assert m, "stub not found"
+    short = {"P": c_void_p, "I": c_int, "F": c_float, "Z": c_size_t}
+    stub = [short[x.strip()] for x in m.group(1).split(",")]
+    assert stub == list(_lib._SIGNATURES["dsa_attn_fwd"][1])
+    call = re.search(r"rc = lib\.dsa_attn_fwd\((.*?)\)\nif rc", doc, flags=re.S).group(1)
+    call = re.sub(r"#.*", "", call)
+    depth, nargs = 0, 1
+    for ch in call:
+        depth += ch in "([" 
+        depth -= ch in ")]"
+        nargs += ch == "," and depth == 0
+    assert nargs == len(stub) == 21

@@ -186,6 +186,37 @@ def test_sparse_path_odd_head_groups(Hq, Hkv, D):
         ops.set_tile_crossover(old)
 
 
+@pytest.mark.parametrize("D,Hq,Hkv,segs,K,sparse", [
+    (64, 16, 1, (128, 64), 4, True),                       # sixteen heads and a few hundred queries on the same four keys
+    (256, 16, 2, (716, 65, 73, 512, 300), 4, True),        # the head geometry of C5 (group of 8, head_dim 256)
+    (256, 64, 4, (2, 2, 257, 2, 31, 200), 4, True),
+    (128, 48, 3, (64, 257, 64, 1), 4, True),
+    (128, 12, 3, (257, 128, 200, 129), 4, True),
+    (64, 64, 4, (127, 257, 5, 127, 257, 127), 4, True),
+    (128, 64, 4, (31, 2, 200, 1, 2), 4, True),
+    (256, 64, 4, (127, 32, 127, 257, 31, 300), 0, False),  # dense causal, group of 16
+    (128, 16, 1, (2, 2, 300, 1, 100, 1), 0, False),
+])
+def test_large_head_groups_with_few_keys_keep_dv_within_the_bound(D, Hq, Hkv, segs, K, sparse):
+    """dV[s] sums P * dO over every (query, head) that attends s.  With few keys per query the probabilities are
+    large, and with a large head group many rows meet in one key row: the bf16 rounding of P then piles up.  The
+    key-side kernel carries the rounding remainder of P for such blocks; these are the geometries where it matters."""
+    _log(f"few keys D={D} {Hq}/{Hkv} segs={segs} K={K}")
+    w = W.Workload("fewkeys", torch.bfloat16, segs, Hq, Hkv, D, 8, 32, max(K, 1), 0.5, 100 + D + Hq)
+    if sparse:
+        _run_case(w)
+        return
+    t = W.make_inputs(w, device="cpu")
+    qd, kd, vd = (t[x].to(DEV).requires_grad_(True) for x in ("q", "k", "v"))
+    out = ops.dsa_varlen_attn(qd, kd, vd, t["cu_seqlens"].to(DEV), w.max_seqlen)
+    out.backward(t["dout"].to(DEV))
+    qr, kr, vr = (t[x].float().requires_grad_(True) for x in ("q", "k", "v"))
+    ref = R.dense_varlen_causal(qr, kr, vr, t["cu_seqlens"])
+    ref.backward(t["dout"].float())
+    for name, got, want in (("out", out, ref), ("dq", qd.grad, qr.grad), ("dk", kd.grad, kr.grad), ("dv", vd.grad, vr.grad)):
+        assert_close_bf16(got, want, name)
+
+
 def test_dense_path_equals_reference_semantics():
     _log("dense path")
     g = torch.Generator().manual_seed(11)

@@ -66,7 +66,10 @@ def test_qk_norm_rope_forward_and_backward(T, Hq, Hkv, D, R, offset, cs, inter):
     torch.cuda.synchronize()
     assert_close_bf16(oq, want_q, "q_out")
     assert_close_bf16(ok, want_k, "k_out")
-    assert_close_bf16(oq, rq.detach(), "q_out vs fp32")
+    # against an evaluation that never rounds: the reference (and the kernel, and `want_q` above) rounds F.rms_norm's
+    # result to bf16 before the rotation, so the rotated value x*cos + rot(x)*sin carries up to (|cos| + |sin|)/2 <= 0.71
+    # steps of that first rounding plus half a step of the final one - two bf16 steps bound it
+    assert_close_bf16(oq, rq.detach(), "q_out vs fp32", steps=2)
     assert_close_bf16(qd.grad, qf.grad, "dq")
     assert_close_bf16(kd.grad, kf.grad, "dk")
     for name, got, want in (("dqw", qwd.grad, qwf.grad), ("dkw", kwd.grad, kwf.grad)):

@@ -55,11 +55,20 @@ __global__ __launch_bounds__(64) void dsa_bwd_dq_kernel(
     const int G = Hq / Hkv;
     const int s0 = cu[find_segment(cu, N, t)];
     if (t - s0 < pos_min) return;                     // rows before the split belong to the tile kernel
-    const int nt = HAS_IDX ? nsel[t] : (t - s0 + 1);
+    // the count is held to [0, K] and every row id to the batch: a bad list cannot reach outside the tensors
+    const int nt = HAS_IDX ? min(nsel[t], K) : (t - s0 + 1);
     const int32_t *irow = HAS_IDX ? idx + (int64_t)t * K : nullptr;
+    if (nt <= 0) {                                    // nothing selected: dQ = 0
+        if (m < Hq / Hkv) {
+            bf16_t *op = dq + ((int64_t)t * Hq + kvh * (Hq / Hkv) + m) * D + 4 * g;
+#pragma unroll
+            for (int dt = 0; dt < D / 16; ++dt) *reinterpret_cast<u32x2 *>(op + dt * 16) = u32x2{0u, 0u};
+        }
+        return;
+    }
     auto key_of = [&](int j) -> int {
         j = min(j, nt - 1);
-        return HAS_IDX ? irow[j] : s0 + j;
+        return HAS_IDX ? min(max(irow[j], 0), T - 1) : s0 + j;
     };
     const float scale_log2 = scale * LOG2E_F;
     const int hq = kvh * G + min(m, G - 1);
@@ -171,7 +180,10 @@ __global__ __launch_bounds__(256) void dsa_bitmap_kernel(const int32_t *__restri
     const int s0 = cu[find_segment(cu, N, t)];
     for (int i = tid; i < ldw; i += 256) words[i] = 0u;
     __syncthreads();
-    const int nt = nsel[t];
+    // entries outside the row's ldw words (a list that names keys of another segment, or a max_seqlen below the
+    // longest segment) are dropped, the count is held to K: a caller's mistake cannot write outside the row
+    const int nt = min(max(nsel[t], 0), K);
+    const unsigned ncols = (unsigned)ldw * 32u;
     const int32_t *irow = idx + (int64_t)t * K;
     // 16-byte loads, all of a thread's in flight (one load per loop iteration would pay the memory latency nt/256 times)
     const int n4 = (reinterpret_cast<uintptr_t>(irow) & 15) ? 0 : nt >> 2;
@@ -185,12 +197,13 @@ __global__ __launch_bounds__(256) void dsa_bitmap_kernel(const int32_t *__restri
             if (base + u * 256 + tid < n4) {
                 const int cs[4] = {c4[u].x - s0, c4[u].y - s0, c4[u].z - s0, c4[u].w - s0};
 #pragma unroll
-                for (int e = 0; e < 4; ++e) atomicOr(&words[cs[e] >> 5], 1u << (cs[e] & 31));
+                for (int e = 0; e < 4; ++e)
+                    if ((unsigned)cs[e] < ncols) atomicOr(&words[cs[e] >> 5], 1u << (cs[e] & 31));
             }
     }
     for (int j = (n4 << 2) + tid; j < nt; j += 256) {
         const int c = irow[j] - s0;
-        atomicOr(&words[c >> 5], 1u << (c & 31));
+        if ((unsigned)c < ncols) atomicOr(&words[c >> 5], 1u << (c & 31));
     }
     __syncthreads();
     uint32_t *orow = bitmap + (int64_t)t * ldw;

@@ -34,11 +34,22 @@ __global__ __launch_bounds__(64) void dsa_attn_fwd_kernel(
     const int G = Hq / Hkv;
     const int s0 = cu[find_segment(cu, N, t)];
     if (t - s0 < pos_min) return;                             // rows before the split belong to the tile kernel
-    const int nt = HAS_IDX ? nsel[t] : (t - s0 + 1);
+    // a caller's own list is trusted for its order only: the count is held to [0, K] and every row id to the batch, so
+    // that a bad list gives a wrong result, never an access outside the tensors
+    const int nt = HAS_IDX ? min(nsel[t], K) : (t - s0 + 1);
     const int32_t *irow = HAS_IDX ? idx + (int64_t)t * K : nullptr;
+    if (nt <= 0) {                                            // nothing selected: zero output, lse = -inf
+        if (m < G) {
+            bf16_t *op = out + ((int64_t)t * Hq + kvh * G + m) * D + 4 * g;
+#pragma unroll
+            for (int dt = 0; dt < D / 16; ++dt) *reinterpret_cast<u32x2 *>(op + dt * 16) = u32x2{0u, 0u};
+            if (g == 0) lse[(int64_t)(kvh * G + m) * T + t] = -INFINITY;
+        }
+        return;
+    }
     auto key_of = [&](int j) -> int {
         j = min(j, nt - 1);                                   // tail columns re-read a valid row, masked below
-        return HAS_IDX ? irow[j] : s0 + j;
+        return HAS_IDX ? min(max(irow[j], 0), T - 1) : s0 + j;
     };
 
     bf16x8 qB[KS];

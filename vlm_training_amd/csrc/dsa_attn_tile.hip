@@ -206,8 +206,9 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     const int kvh = blockIdx.x % Hkv;
     int s0, L, blk;
     if (!locate_block(cu, N, blockIdx.x / Hkv, QBW, true, s0, L, blk)) return;
+    if (HAS_IDX) L = min(L, ldw * 32);                  // a bitmap row has ldw words whatever the caller's max_seqlen
     const int qc0 = blk * QBW;
-    if (qc0 >= pos_split) return;                       // rows past the split belong to the gather kernel
+    if (qc0 >= pos_split || qc0 >= L) return;                       // rows past the split belong to the gather kernel
 
     const int r = wv * 32 + j;
     const int qcol = qc0 + (r >> GSHIFT), head = r & (Gp - 1);
@@ -342,7 +343,9 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     const int kvh = blockIdx.x % Hkv;
     int s0, L, blk;
     if (!locate_block(cu, N, blockIdx.x / Hkv, QBW, true, s0, L, blk)) return;
+    L = min(L, ldw * 32);                               // a bitmap row has ldw words whatever the caller's max_seqlen
     const int qc0 = blk * QBW;
+    if (qc0 >= L) return;
 
     const int r = wv * 32 + j;
     const int qcol = qc0 + (r >> GSHIFT), head = r & (Gp - 1);
@@ -470,7 +473,9 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     lo.init(lane);
     int s0, L, blk;
     if (!locate_block(cu, N, blockIdx.x, QBW, true, s0, L, blk)) return;
+    L = min(L, ldw * 32);
     const int qc0 = blk * QBW;
+    if (qc0 >= L) return;
     const int r = wv * 32 + j;
     const int qcol = qc0 + (r >> GSHIFT), head = r & (Gp - 1);
     const bool row_ok = qcol < L && head < Hi;
@@ -574,6 +579,8 @@ __global__ __launch_bounds__(256) void dsa_tile_idxk_kernel(
     lo.init(lane);
     int s0, L, blk;
     if (!locate_block(cu, N, blockIdx.x, 128, false, s0, L, blk)) return;
+    L = min(L, ldw * 32);
+    if (blk * 128 >= L) return;
     const int c0 = blk * 128, kc = c0 + wv * 32;
     const int mykey = kc + j;
     const bool key_ok = mykey < L;
@@ -690,12 +697,13 @@ __global__ __launch_bounds__(256) void dsa_tile_idxk_kernel(
 // dk_idx[s,:] = sum of the partial sums of the pieces of its tile's walk, in piece order
 __global__ __launch_bounds__(256) void dsa_idxk_reduce_kernel(const float *__restrict__ partial,
                                                                const int32_t *__restrict__ cu, int N, int T, int D,
-                                                               int chunk_steps, bf16_t *__restrict__ dk_idx) {
+                                                               int chunk_steps, int max_cols, bf16_t *__restrict__ dk_idx) {
     const int s = blockIdx.x * (256 / 32) + (threadIdx.x >> 5), c4 = (threadIdx.x & 31) * 4;   // 32 threads x 4 columns per pass
     if (s >= T) return;
     const int seg = find_segment(cu, N, s);
-    const int s0 = cu[seg], L = cu[seg + 1] - s0;
+    const int s0 = cu[seg], L = min(cu[seg + 1] - s0, max_cols);     // as the walk: no column past the bitmap row
     const int c0 = ((s - s0) >> 7) << 7;
+    if (c0 >= L) return;
     const int pieces = (L - c0 + chunk_steps - 1) / chunk_steps;
     for (int c = c4; c < D; c += 128) {
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -750,8 +758,9 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     const int kvh = blockIdx.x % Hkv;
     int s0, L, blk;
     if (!locate_block(cu, N, blockIdx.x / Hkv, QBW, true, s0, L, blk)) return;
+    if (HAS_IDX) L = min(L, ldw * 32);                  // a bitmap row has ldw words whatever the caller's max_seqlen
     const int qc0 = blk * QBW;
-    if (qc0 >= pos_split) return;
+    if (qc0 >= pos_split || qc0 >= L) return;
 
     const int r = wv * 32 + j;
     const int qcol = qc0 + (r >> GSHIFT), head = r & (Gp - 1);
@@ -848,12 +857,13 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
 //     also do all the staging (global -> registers two blocks ahead -> LDS), so the producers' stream
 //     holds nothing but the GEMMs and the softmax.
 // Nothing is computed twice (32 MFMAs per 32x32 block pair), each wave stays under 256 registers.
-// LDS (dynamic, ~115 KiB): q/dO blocks in a ring of four (b+2 being staged, b+1 read row-wise by the
-// producers, b-1 read transposed by the consumers), P/dS in a ring of two, row statistics and
-// selection words in a ring of four.  One barrier per block.
+// LDS (dynamic, ~131 KiB): q/dO blocks in a ring of four (b+2 being staged, b+1 read row-wise by the
+// producers, b-1 read transposed by the consumers), P/dS (and, for blocks of large probabilities, the
+// bf16 rounding remainder of P) in a ring of two, row statistics and selection words in a ring of four.
+// One barrier per block.
 // head_dim 256: the K and V rows of a producer fill 128 registers and a consumer's accumulators would
 // fill 256, so the kernel is launched once per half of head_dim (`dhalf`: the consumers accumulate and
-// write that half, the producers repeat S and dP), the q/dO ring has three slots (~145 KiB) and the
+// write that half, the producers repeat S and dP), the q/dO ring has three slots (~158 KiB) and the
 // producers run GEMMs and softmax of a block in turn.
 // ==================================================================================================
 template <int D, bool HAS_IDX, int GSHIFT>
@@ -874,13 +884,15 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     constexpr int CPT = NCHUNK / 256;                    // chunks per consumer thread and operand
     constexpr int Gp = 1 << GSHIFT, QB = 32 >> GSHIFT;
     constexpr int QD_SLOT = 2 * TILE_B;                  // q block | dO block
-    constexpr int PD_SLOT = 4 * 4 * 1024;                // 4 key groups x {P lo, P hi, dS lo, dS hi} x 64 lanes x 16 B
+    // 4 key groups x {P (rows 0-15 | 16-31), dS (same), rounding remainder of P (same)} x 64 lanes x 16 B
+    constexpr int PD_GROUP = 6 * 1024, PD_SLOT = 4 * PD_GROUP;
     constexpr int AUX_SLOT = (32 + 32 + 4 * 32) * 4;     // lse | delta | selection words [key group][query]
     static_assert(CPT >= 1 && NCHUNK % 256 == 0, "every consumer thread stages whole chunks");
     extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
     unsigned char *const qd_ring = dyn_lds;                          // NQD slots
     unsigned char *const pd_ring = dyn_lds + NQD * QD_SLOT;          // 2 slots
     unsigned char *const aux_ring = pd_ring + 2 * PD_SLOT;           // NQD slots
+    uint32_t *const split_flag = reinterpret_cast<uint32_t *>(aux_ring + NQD * AUX_SLOT);   // [P/dS slot][key group]
     auto qslot = [](int b) { return PIPE ? (b & 3) : (b % 3); };
 
     const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5, j = lane & 31;
@@ -893,6 +905,8 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     const int kvh = blockIdx.x % Hkv;
     int s0, L, blk;
     if (!locate_block(cu, N, blockIdx.x / Hkv, 128, false, s0, L, blk)) return;
+    if (HAS_IDX) L = min(L, ldw * 32);                  // a bitmap row has ldw words whatever the caller's max_seqlen
+    if (blk * 128 >= L) return;                         // (whole workgroup, before its first barrier)
     const int c0 = blk * 128, kc = c0 + kg * 32;
     const int mykey = kc + j;
     const bool key_ok = mykey < L;
@@ -1031,7 +1045,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
                 pt[vv] = (lds_u8 *)qt + lo.tr[vv];
                 asm volatile("" : "+v"(pt[vv]));         // keep "address + immediate" reads: no re-association
             }
-            const unsigned char *pd = pd_ring + (b & 1) * PD_SLOT + kg * 4096 + lane * 16;
+            const unsigned char *pd = pd_ring + (b & 1) * PD_SLOT + kg * PD_GROUP + lane * 16;
             const bf16x8 pB0 = *reinterpret_cast<const bf16x8 *>(pd), pB1 = *reinterpret_cast<const bf16x8 *>(pd + 1024);
             const bf16x8 dB0 = *reinterpret_cast<const bf16x8 *>(pd + 2048), dB1 = *reinterpret_cast<const bf16x8 *>(pd + 3072);
 #pragma unroll
@@ -1042,6 +1056,15 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
                 dkacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 1, dt, 0), dB1, dkacc[dt]);
             }
             sched_reads_ahead<4 * DTC, 3, 2, 4>();
+            // blocks that hold a large probability also carry what bf16 rounded off P (see store_pd): dV += dO^T P_lo
+            if (__builtin_amdgcn_readfirstlane(split_flag[(b & 1) * 4 + kg])) {
+                const bf16x8 pL0 = *reinterpret_cast<const bf16x8 *>(pd + 4096), pL1 = *reinterpret_cast<const bf16x8 *>(pd + 5120);
+#pragma unroll
+                for (int dt = 0; dt < DTC; ++dt) {
+                    dvacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 0, dt, TILE_B), pL0, dvacc[dt]);
+                    dvacc[dt] = mfma32(LaneOffsets<D>::trop_at(pt, 1, dt, TILE_B), pL1, dvacc[dt]);
+                }
+            }
         };
         int b = 0;
         if (PIPE) {                                      // step b + 2 sits in set b % 2
@@ -1113,12 +1136,37 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
         pv[vi] = p;
         dsv[vi] = p * (pacc[vi] - d4[g4][e]);
     };
+    // P and dS go to the consumers in bf16.  dV[s] = sum over (query, head) of P dO piles the rounding of P (2^-9
+    // relative) onto one key row; where probabilities are large (few keys per query: short rows, small top-k) and many
+    // rows meet in one key, that noise reaches several 1e-2.  A block whose largest P is at least DKV_SPLIT_MIN
+    // therefore also carries P - bf16(P), and the consumers add dO^T times it; blocks of small probabilities (the bulk of
+    // any long row) skip both the arithmetic and the extra MFMAs.
+    constexpr float DKV_SPLIT_MIN = 0.015625f;
     auto store_pd = [&](int b, const float *pv, const float *dsv) {  // -> ring slot b % 2, MFMA B layout
-        unsigned char *pd = pd_ring + (b & 1) * PD_SLOT + kg * 4096 + lane * 16;
-        *reinterpret_cast<bf16x8 *>(pd) = pack8(pv);
-        *reinterpret_cast<bf16x8 *>(pd + 1024) = pack8(pv + 8);
+        unsigned char *pd = pd_ring + (b & 1) * PD_SLOT + kg * PD_GROUP + lane * 16;
+        const bf16x8 p0 = pack8(pv), p1 = pack8(pv + 8);
+        *reinterpret_cast<bf16x8 *>(pd) = p0;
+        *reinterpret_cast<bf16x8 *>(pd + 1024) = p1;
         *reinterpret_cast<bf16x8 *>(pd + 2048) = pack8(dsv);
         *reinterpret_cast<bf16x8 *>(pd + 3072) = pack8(dsv + 8);
+        float pm = pv[0];
+#pragma unroll
+        for (int vi = 1; vi < 16; ++vi) pm = fmaxf(pm, pv[vi]);
+        const bool big = __builtin_amdgcn_ballot_w64(pm >= DKV_SPLIT_MIN) != 0ull;   // wave-uniform
+        if (big) {
+            const u32x4 w0 = __builtin_bit_cast(u32x4, p0), w1 = __builtin_bit_cast(u32x4, p1);
+            float lo[16];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                lo[2 * e] = pv[2 * e] - __uint_as_float(w0[e] << 16);
+                lo[2 * e + 1] = pv[2 * e + 1] - __uint_as_float(w0[e] & 0xffff0000u);
+                lo[8 + 2 * e] = pv[8 + 2 * e] - __uint_as_float(w1[e] << 16);
+                lo[9 + 2 * e] = pv[9 + 2 * e] - __uint_as_float(w1[e] & 0xffff0000u);
+            }
+            *reinterpret_cast<bf16x8 *>(pd + 4096) = pack8(lo);
+            *reinterpret_cast<bf16x8 *>(pd + 5120) = pack8(lo + 8);
+        }
+        if (lane == 0) split_flag[(b & 1) * 4 + kg] = big ? 1u : 0u;
     };
     auto softmax = [&](auto may_diag, int b, const f32x16 &sacc, const f32x16 &pacc) {
         float pv[16], dsv[16];
@@ -1227,7 +1275,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
 }
 template <int D>
 constexpr size_t dkvpc_lds_bytes() {
-    return (D <= 128 ? 4 : 3) * ((size_t)2 * tile_bytes<D>() + (32 + 32 + 4 * 32) * 4) + 2 * (4 * 4 * 1024);
+    return (D <= 128 ? 4 : 3) * ((size_t)2 * tile_bytes<D>() + (32 + 32 + 4 * 32) * 4) + 2 * (4 * 6 * 1024) + 2 * 4 * 4;
 }
 
 // ==================================================================================================
@@ -1247,52 +1295,56 @@ static inline int group_shift(int Hq, int Hkv) {
 template <int D> constexpr int tile_waves() { return D == 128 ? DSA_TILE_WAVES_128 : 4; }
 static inline int tile_waves_of(int D) { return D == 128 ? DSA_TILE_WAVES_128 : 4; }
 template <int D, bool HAS_IDX, int GS>
-static void launch_fwd_i(dim3 grid, hipStream_t stream, const void *q, const void *k, const void *v,
+static hipError_t launch_fwd_i(dim3 grid, hipStream_t stream, const void *q, const void *k, const void *v,
                          const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T, int Hq, int Hkv, float sl2,
                          int pos_split, int causal, void *out, float *lse) {
     hipLaunchKernelGGL((dsa_tile_fwd_kernel<D, HAS_IDX, GS, tile_waves<D>()>), grid, dim3(64 * tile_waves<D>()), 0, stream, (const bf16_t *)q,
                        (const bf16_t *)k, (const bf16_t *)v, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, pos_split, causal, (bf16_t *)out, lse);
+    return hipSuccess;
 }
 template <int D, bool HAS_IDX, int GS>
-static void launch_dq_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
+static hipError_t launch_dq_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
                         const float *lse, const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N,
                         int T, int Hq, int Hkv, float scale, int pos_split, int causal, void *dq) {
     hipLaunchKernelGGL((dsa_tile_dq_kernel<D, HAS_IDX, GS, tile_waves<D>()>), grid, dim3(64 * tile_waves<D>()), 0, stream, (const bf16_t *)dout,
                        (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv,
                        scale, pos_split, causal, (bf16_t *)dq);
+    return hipSuccess;
 }
 template <int D, bool HAS_IDX, int GS>
-static void launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
+static hipError_t launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
                          const float *lse, const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N,
                          int T, int Hq, int Hkv, float scale, int causal, void *dk, void *dv) {
-    static bool configured = false;                      // LDS above 64 KiB has to be requested once per kernel
-    if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkvpc_lds_bytes<D>());
-        configured = true;
-    }
+    // LDS above 64 KiB has to be requested per kernel and device; asked for on every launch (a host-side table
+    // lookup), so that neither a second device nor a second thread can meet a kernel that was never configured
+    const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(&dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkvpc_lds_bytes<D>());
+    if (ea != hipSuccess) return ea;
     // head_dim 256: one launch per half of head_dim (a consumer wave holds 128 accumulator registers)
     for (int dhalf = 0; dhalf < (D > 128 ? 2 : 1); ++dhalf)
         hipLaunchKernelGGL((dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>), grid, dim3(512), dkvpc_lds_bytes<D>(), stream,
                            (const bf16_t *)dout, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap,
                            ldw, cu, N, T, Hq, Hkv, scale, causal, dhalf, (bf16_t *)dk, (bf16_t *)dv);
+    return hipSuccess;
 }
 
 #define GS_SWITCH(FN, DD, HI, ...)                                    \
     switch (gs) {                                                     \
-        case 0: FN<DD, HI, 0>(__VA_ARGS__); break;                    \
-        case 1: FN<DD, HI, 1>(__VA_ARGS__); break;                    \
-        case 2: FN<DD, HI, 2>(__VA_ARGS__); break;                    \
-        case 3: FN<DD, HI, 3>(__VA_ARGS__); break;                    \
-        default: FN<DD, HI, 4>(__VA_ARGS__); break;                   \
+        case 0: launch_status = FN<DD, HI, 0>(__VA_ARGS__); break;    \
+        case 1: launch_status = FN<DD, HI, 1>(__VA_ARGS__); break;    \
+        case 2: launch_status = FN<DD, HI, 2>(__VA_ARGS__); break;    \
+        case 3: launch_status = FN<DD, HI, 3>(__VA_ARGS__); break;    \
+        default: launch_status = FN<DD, HI, 4>(__VA_ARGS__); break;   \
     }
 #define TILE_SWITCH(FN, ...)                                                              \
+    hipError_t launch_status = hipSuccess;                                                \
     switch (D) {                                                                          \
         case 64: if (bitmap) { GS_SWITCH(FN, 64, true, __VA_ARGS__) } else { GS_SWITCH(FN, 64, false, __VA_ARGS__) } break;    \
         case 128: if (bitmap) { GS_SWITCH(FN, 128, true, __VA_ARGS__) } else { GS_SWITCH(FN, 128, false, __VA_ARGS__) } break; \
         case 256: if (bitmap) { GS_SWITCH(FN, 256, true, __VA_ARGS__) } else { GS_SWITCH(FN, 256, false, __VA_ARGS__) } break; \
         default: return hipErrorInvalidValue;                                             \
-    }
+    }                                                                                     \
+    if (launch_status != hipSuccess) return launch_status;
 
 extern "C" hipError_t dsa_launch_tile_fwd(const void *q, const void *k, const void *v, const uint32_t *bitmap, int ldw,
                                           const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale,
@@ -1303,11 +1355,12 @@ extern "C" hipError_t dsa_launch_tile_fwd(const void *q, const void *k, const vo
     return hipGetLastError();
 }
 template <int D, bool HAS_IDX, int GS>
-static void launch_mass_i(dim3 grid, hipStream_t stream, const void *q, const void *k, const float *lse,
+static hipError_t launch_mass_i(dim3 grid, hipStream_t stream, const void *q, const void *k, const float *lse,
                           const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T, int Hq, int Hkv, float sl2,
                           int K, float *partial) {
     hipLaunchKernelGGL((dsa_tile_mass_kernel<D, GS, tile_waves<D>()>), grid, dim3(64 * tile_waves<D>()), 0, stream,
                        (const bf16_t *)q, (const bf16_t *)k, lse, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, K, partial);
+    return hipSuccess;
 }
 // attention mass of the selected keys: partial (Hkv,T,K) tables, then their sum scaled by 1/Hq into mass (T,K)
 extern "C" hipError_t dsa_launch_tile_mass(const void *q, const void *k, const float *lse, const uint32_t *bitmap,
@@ -1339,7 +1392,7 @@ static void launch_idx_bwd_i(hipStream_t stream, const void *q_idx, const void *
     hipLaunchKernelGGL((dsa_tile_idxk_kernel<D, GS>), gk, dim3(256), 0, stream, (const bf16_t *)q_idx, (const bf16_t *)k_idx,
                        (const bf16_t *)w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, IDXK_CHUNK, partial);
     hipLaunchKernelGGL(dsa_idxk_reduce_kernel, dim3((unsigned)((T + 7) / 8)), dim3(256), 0, stream, partial, cu, N, T, D,
-                       IDXK_CHUNK, (bf16_t *)dk_idx);
+                       IDXK_CHUNK, ldw * 32, (bf16_t *)dk_idx);
 }
 extern "C" size_t dsa_indexer_bwd_partial_bytes(int T, int Di, int ldw) {
     return (size_t)((ldw * 32 + IDXK_CHUNK - 1) / IDXK_CHUNK) * T * Di * 4;

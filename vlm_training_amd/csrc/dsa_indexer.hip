@@ -123,7 +123,7 @@ __global__ __launch_bounds__(IDX_WAVES * 64, 2) void dsa_indexer_scores_kernel(
                     for (int v = 0; v < 16; ++v) sum += wreg[ht][v] * __int_as_float(max(__float_as_int(acc[ht][v]), 0));
                 sum = half_sum_f(sum);
                 const int s = kb + (lane & 31);
-                if (lane < 32 && s >= s0 && s <= t) orow[s - s0] = sum * scale;
+                if (lane < 32 && s >= s0 && s <= t && s - s0 < ld) orow[s - s0] = sum * scale;   // ld bounds the row whatever the caller's max_seqlen
             };
             const bool on0 = !(kt > t || kt + 31 < s0), on1 = !(kt + 32 > t || kt + 63 < s0);   // wave-uniform
             if (on0 && on1) {

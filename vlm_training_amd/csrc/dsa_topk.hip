@@ -36,7 +36,9 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
     const int t = row_begin + blockIdx.x;
     const int seg = find_segment(cu, N, t);
     const int s0 = cu[seg];
-    const int nvalid = t - s0 + 1;
+    // a row never reaches past its ld columns: with a max_seqlen below the longest segment (a caller's mistake) the
+    // selection of the long rows is wrong, but nothing outside the score rows is read
+    const int nvalid = (int)min((int64_t)(t - s0 + 1), ld);
     int32_t *orow = idx_out + (int64_t)t * K;
 
     if (nvalid <= K) {
@@ -181,7 +183,10 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
             const uint32_t eq_rank = eq_seen + (uint32_t)__popcll(b_eq & lt_mask);
             const bool take = is_gt || (is_eq && eq_rank < need_eq);
             const uint64_t b_take = __ballot(take);
-            if (take) orow[out_pos + (uint32_t)__popcll(b_take & lt_mask)] = s0 + i;
+            // exactly K keys are taken when every score orders (the radix passes count them); NaN scores can break the
+            // count, hence the bound on the slot
+            const uint32_t slot = out_pos + (uint32_t)__popcll(b_take & lt_mask);
+            if (take && slot < (uint32_t)K) orow[slot] = s0 + i;
             out_pos += (uint32_t)__popcll(b_take);
             eq_seen += (uint32_t)__popcll(b_eq);
         }
