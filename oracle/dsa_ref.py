@@ -269,6 +269,28 @@ def attention_mass(q, k, idx, n, cu_seqlens, softmax_scale: Optional[float] = No
     return mass
 
 
+def sparse_attention_rows(q, k, v, idx, n, rows, softmax_scale: Optional[float] = None):
+    """``sparse_attention`` for the query rows ``rows`` only -> (len(rows), Hq, D).
+
+    Written as a gather (the selected key rows of a query are fetched and attended densely), not as the masked dense
+    product of ``sparse_attention``: the two restatements check each other, and this one costs n[t] keys per row
+    whatever the segment length, so single rows of a very long sequence can be checked.  Differentiable in q, k, v.
+    """
+    T, Hq, D = q.shape
+    G = Hq // k.shape[1]
+    scale = softmax_scale if softmax_scale is not None else D ** -0.5
+    cdt = torch.float64 if q.dtype == torch.float64 else torch.float32
+    outs = []
+    for r in rows:
+        sel = idx[r, : int(n[r])].long()
+        ks = k[sel].to(cdt).repeat_interleave(G, dim=1)                         # (n,Hq,D): head h reads kv head h//G
+        vs = v[sel].to(cdt).repeat_interleave(G, dim=1)
+        logits = torch.einsum("hd,nhd->hn", q[r].to(cdt), ks) * scale
+        p = torch.softmax(logits, dim=-1)
+        outs.append(torch.einsum("hn,nhd->hd", p, vs))
+    return torch.stack(outs) if outs else q.new_zeros(0, Hq, D, dtype=cdt)
+
+
 def selected_scores(q_idx, k_idx, w, idx, n, cu_seqlens, index_scale: Optional[float] = None):
     """Indexer scores of the selected keys: sel[t,j] = score(t, idx[t,j]) (0 where idx = -1), fp32."""
     T, K = idx.shape

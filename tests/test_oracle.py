@@ -218,6 +218,23 @@ def test_sparse_matches_bruteforce():
             assert len(sel) == int(n[r]) == min(5, r - a + 1)
 
 
+def test_row_wise_gather_form_matches_bruteforce_and_the_masked_form():
+    """sparse_attention_rows (a gather per query row) against the pure-Python loop and against the masked dense
+    restatement, values and the gradient of the sampled rows."""
+    t = _toy(seed=24)
+    out, idx, n = R.dsa_varlen_attn_ref(t["q"], t["k"], t["v"], t["cu"], t["q_idx"], t["k_idx"], t["w"], 4,
+                                        return_indices=True)
+    rows = [0, 3, 10, 11, 12, 29, 30, 36]
+    got = R.sparse_attention_rows(t["q"], t["k"], t["v"], idx, n, rows)
+    assert torch.allclose(got.double(), brute_sparse(t["q"], t["k"], t["v"], idx)[rows], atol=1e-5)
+    assert torch.allclose(got, out[rows], atol=1e-5)
+    g = rnd(len(rows), 4, 8, seed=99)
+    q1, q2 = t["q"].clone().requires_grad_(True), t["q"].clone().requires_grad_(True)
+    (R.sparse_attention_rows(q1, t["k"], t["v"], idx, n, rows) * g).sum().backward()
+    (R.sparse_attention(q2, t["k"], t["v"], idx, n, t["cu"])[rows] * g).sum().backward()
+    assert torch.allclose(q1.grad, q2.grad, atol=1e-5)
+
+
 def test_k_at_least_longest_segment_equals_dense():
     t = _toy(seed=30)
     dense = R.dense_varlen_causal(t["q"], t["k"], t["v"], t["cu"])

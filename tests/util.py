@@ -56,3 +56,17 @@ def oracle_topk_from_gpu_scores(scores_cpu, cu, K):
         sc = sc.masked_fill(torch.triu(torch.ones(L, L, dtype=torch.bool), 1), float("-inf"))
         idx[a:b], n[a:b] = R.topk_select_segment(sc, K, base=a)
     return idx, n
+
+
+def oracle_grads_by_segment(t, idx, n, cu):
+    """(out, dq, dk, dv) of the fp32 oracle, one segment at a time (segments are independent; the autograd graph of
+    the longest one is what has to fit in host memory).  ``t``: dict of CPU tensors q, k, v, dout; ``idx``/``n``: the
+    selection with global packed row ids."""
+    outs, dqs, dks, dvs = [], [], [], []
+    for a, b in R.segments(cu):
+        if b == a:
+            continue
+        loc = torch.where(idx[a:b] >= 0, idx[a:b] - a, idx[a:b])
+        o, dq, dk, dv = R.sparse_attention_grads(t["q"][a:b], t["k"][a:b], t["v"][a:b], loc, n[a:b], [0, b - a], t["dout"][a:b])
+        outs.append(o); dqs.append(dq); dks.append(dk); dvs.append(dv)
+    return torch.cat(outs), torch.cat(dqs), torch.cat(dks), torch.cat(dvs)

@@ -22,10 +22,14 @@ __device__ __forceinline__ uint32_t score_key(float x) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);  // larger float <=> larger key
 }
 
+// `only`: 0 = every row of the launch; 1 = rows of at most lds_keys keys (the others belong to a second launch of the
+// uncached kernel); 2 = rows longer than skip_upto keys.  A launch whose bound on the longest row exceeds the LDS cache
+// is split this way, so that the rows that do fit are still read from HBM once - the bound may be far above the real
+// longest row (max_seqlen = the packed length when the caller holds no better one).
 template <bool CACHED>
 __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
     const float *__restrict__ scores, int64_t ld, int row_begin, const int32_t *__restrict__ cu, int N, int K, int lds_keys,
-    int32_t *__restrict__ idx_out, int32_t *__restrict__ n_out) {
+    int only, int skip_upto, int32_t *__restrict__ idx_out, int32_t *__restrict__ n_out) {
     __shared__ uint32_t hist[TOPK_BINS];
     __shared__ uint32_t wave_tot[4];
     __shared__ uint32_t sel_digit, sel_remaining;
@@ -40,6 +44,8 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
     // selection of the long rows is wrong, but nothing outside the score rows is read
     const int nvalid = (int)min((int64_t)(t - s0 + 1), ld);
     int32_t *orow = idx_out + (int64_t)t * K;
+    if (only == 1 && nvalid > lds_keys) return;
+    if (only == 2 && nvalid <= skip_upto) return;
 
     if (nvalid <= K) {
         for (int i = tid; i < K; i += TOPK_THREADS) orow[i] = (i < nvalid) ? (s0 + i) : -1;
@@ -199,12 +205,15 @@ extern "C" hipError_t dsa_launch_topk(const float *scores, int64_t ld, int row_b
                                       hipStream_t stream) {
     const int rows = row_end - row_begin;
     if (rows <= 0) return hipSuccess;
-    if (max_row <= TOPK_LDS_CAP)
+    if (max_row <= TOPK_LDS_CAP) {
         hipLaunchKernelGGL(dsa_topk_rows_kernel<true>, dim3(rows), dim3(TOPK_THREADS), (size_t)((max_row + 3) & ~3) * 4, stream,
-                           scores, ld, row_begin, cu, N, K, (max_row + 3) & ~3, idx, n);
-    else
-        hipLaunchKernelGGL(dsa_topk_rows_kernel<false>, dim3(rows), dim3(TOPK_THREADS), 16, stream, scores, ld,
-                           row_begin, cu, N, K, 0, idx, n);
+                           scores, ld, row_begin, cu, N, K, (max_row + 3) & ~3, 0, 0, idx, n);
+    } else {
+        hipLaunchKernelGGL(dsa_topk_rows_kernel<true>, dim3(rows), dim3(TOPK_THREADS), (size_t)TOPK_LDS_CAP * 4, stream, scores,
+                           ld, row_begin, cu, N, K, TOPK_LDS_CAP, 1, 0, idx, n);
+        hipLaunchKernelGGL(dsa_topk_rows_kernel<false>, dim3(rows), dim3(TOPK_THREADS), 16, stream, scores, ld, row_begin, cu,
+                           N, K, 0, 2, TOPK_LDS_CAP, idx, n);
+    }
     return hipGetLastError();
 }
 

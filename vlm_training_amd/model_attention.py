@@ -25,8 +25,11 @@ def varlen_attn(query, key, value, cu_seq_q, cu_seq_k, max_q, max_k, is_causal=N
     unknown = set(dsa) - set(_DSA_KEYS)
     if unknown:
         raise TypeError(f"unexpected arguments {sorted(unknown)}")
-    if cu_seq_q is not cu_seq_k and not torch.equal(cu_seq_q, cu_seq_k):
-        raise ValueError("self-attention only: cu_seq_q and cu_seq_k must agree")
+    # self-attention only: both offsets must be the same tensor, or two views of the same memory.  (Comparing the
+    # contents of two distinct tensors would copy from the device and stall the stream once per layer.)
+    if cu_seq_q is not cu_seq_k and not (cu_seq_q.data_ptr() == cu_seq_k.data_ptr() and cu_seq_q.shape == cu_seq_k.shape
+                                         and cu_seq_q.stride() == cu_seq_k.stride()):
+        raise ValueError("self-attention only: pass the same cu_seqlens tensor as cu_seq_q and cu_seq_k")
     if max_q != max_k:
         raise ValueError("self-attention only: max_q and max_k must agree")
     if window_size is not None:
@@ -58,8 +61,33 @@ def _hf_indexer_to_packed(x):
     return x if x is None or x.dim() < 3 or x.shape[0] != 1 else x.squeeze(0)
 
 
-def varlen_attention_forward(query, key, value, attention_mask, **dsa):
-    """(1,Hq,T,D),(1,Hkv,T,D),(1,Hkv,T,D), cu_seqlens -> ((1,T,Hq,D), None)."""
+_BOUND_CACHE = {}                     # (data_ptr, version, numel, device) of a cu_seqlens tensor -> its longest segment
+
+
+def longest_segment(cu_seqlens) -> int:
+    """Longest segment of a packed row, read back from the device once per ``cu_seqlens`` tensor: every layer of a
+    step hands over the same tensor, so the copy (and its stall) is paid once per batch instead of once per layer as
+    in the reference (train/model_attention.py:120-121).  While a stream is being captured nothing may be copied to
+    the host: the packed length, an upper bound, is returned instead."""
+    if torch.cuda.is_current_stream_capturing():
+        return None
+    key = (cu_seqlens.data_ptr(), cu_seqlens._version, cu_seqlens.numel(), str(cu_seqlens.device))
+    hit = _BOUND_CACHE.get(key)
+    if hit is None:
+        if len(_BOUND_CACHE) > 64:
+            _BOUND_CACHE.clear()
+        flat = cu_seqlens.reshape(-1)
+        hit = max(int((flat[1:] - flat[:-1]).max()), 1) if flat.numel() > 1 else 1
+        _BOUND_CACHE[key] = hit
+    return hit
+
+
+def varlen_attention_forward(query, key, value, attention_mask, max_seqlen=None, **dsa):
+    """(1,Hq,T,D),(1,Hkv,T,D),(1,Hkv,T,D), cu_seqlens -> ((1,T,Hq,D), None).
+
+    ``max_seqlen`` (keyword, not in the reference's signature): the longest segment if the caller holds it; otherwise
+    it is read from ``cu_seqlens`` once per tensor (``longest_segment``).  The selection bitmap and the score rows of
+    the DSA path are sized by it, so a tight bound matters there."""
     # tensor-parallel runs hand over DTensors sharded by head: the kernels see the local shard
     # (train/model_attention.py:104-106)
     query, key, value = (x.to_local() if hasattr(x, "to_local") else x for x in (query, key, value))
@@ -71,10 +99,11 @@ def varlen_attention_forward(query, key, value, attention_mask, **dsa):
     key = key.view(-1, key.size(-2), key.size(-1))
     value = value.view(-1, value.size(-2), value.size(-1))
     cu_seqlens = attention_mask.squeeze()
-    # The reference reads the longest segment back to the host here (train/model_attention.py:120-121,
-    # a device sync per layer).  The kernels only need an upper bound, so the packed length serves.
-    attn_output = varlen_attn(query, key, value, cu_seq_q=cu_seqlens, cu_seq_k=cu_seqlens, max_q=None,
-                              max_k=None, window_size=(-1, 0), **dsa)
+    # The reference reads the longest segment back to the host here, once per layer (train/model_attention.py:120-121).
+    # Any upper bound gives the same result; a tight one keeps the DSA workspaces small.
+    bound = int(max_seqlen) if max_seqlen is not None else longest_segment(cu_seqlens)
+    attn_output = varlen_attn(query, key, value, cu_seq_q=cu_seqlens, cu_seq_k=cu_seqlens, max_q=bound,
+                              max_k=bound, window_size=(-1, 0), **dsa)
     if isinstance(attn_output, tuple):
         return (attn_output[0].unsqueeze(0), None) + tuple(attn_output[1:])
     return attn_output.unsqueeze(0), None

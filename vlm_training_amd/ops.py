@@ -36,11 +36,23 @@ def _as_bf16(t: torch.Tensor) -> torch.Tensor:
     return (t if t.dtype == torch.bfloat16 else t.to(torch.bfloat16)).contiguous()
 
 
-def _check_cu(cu_seqlens: torch.Tensor, T: int):
+def _check_cu(cu_seqlens: torch.Tensor, T: int, max_seqlen: Optional[int] = None):
     if cu_seqlens.dim() != 1 or cu_seqlens.numel() < 2:
         raise ValueError("cu_seqlens must be 1-D with at least two entries")
     if cu_seqlens.dtype != torch.int32:
         cu_seqlens = cu_seqlens.to(torch.int32)
+    if os.environ.get("DSA_DEBUG_META"):
+        # The kernels trust the segment offsets (they hold every index to its buffer, so a bad table gives a wrong
+        # result, not a fault).  With this switch the table is copied to the host and checked - one stall per call,
+        # which is why it is not the default.
+        cu = cu_seqlens.tolist()
+        if cu[0] != 0 or cu[-1] != T:
+            raise ValueError(f"cu_seqlens must start at 0 and end at T={T}, got [{cu[0]} ... {cu[-1]}]")
+        if any(b < a for a, b in zip(cu[:-1], cu[1:])):
+            raise ValueError("cu_seqlens must be non-decreasing")
+        longest = max(b - a for a, b in zip(cu[:-1], cu[1:]))
+        if max_seqlen is not None and longest > max_seqlen:
+            raise ValueError(f"max_seqlen={max_seqlen} is below the longest segment ({longest})")
     return cu_seqlens.contiguous()
 
 
@@ -110,7 +122,7 @@ def index_topk(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen: int, top_k: int,
         raise ValueError("indexer tensor shapes disagree")
     if top_k < 1:
         raise ValueError("top_k must be >= 1")
-    cu = _check_cu(cu_seqlens, T)
+    cu = _check_cu(cu_seqlens, T, max_seqlen)
     scale = index_scale if index_scale is not None else (Di ** -0.5) * (Hi ** -0.5)
     lib = _lib.load()
     idx = torch.empty((T, top_k), dtype=torch.int32, device=q_idx.device)
@@ -415,9 +427,9 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, in
     """
     _require_cuda(q, k, v, cu_seqlens)
     T, Hq, Hkv, D = _check_qkv(q, k, v)
-    cu = _check_cu(cu_seqlens, T)
-    scale = float(softmax_scale) if softmax_scale is not None else D ** -0.5
     max_seqlen = T if max_seqlen is None else int(max_seqlen)
+    cu = _check_cu(cu_seqlens, T, max_seqlen)
+    scale = float(softmax_scale) if softmax_scale is not None else D ** -0.5
     sparse = indexer_q is not None or indexer_k is not None or indexer_w is not None
     idx = n = None
     if sparse and not causal:
