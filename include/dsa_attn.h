@@ -77,6 +77,22 @@ int dsa_index_topk(const void *q_idx, const void *k_idx, const void *w_idx, cons
                    int32_t *idx, int32_t *n, void *ws, size_t ws_bytes, void *stream);
 
 /*
+ * dsa_index_topk for callers that cannot allocate device memory or hand over a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): same arguments without `ws`, same idx and n, bit
+ * for bit.  It has no counterpart in the reference.  The score rows are kept in a static device array of
+ * dsa_index_topk_noalloc_scratch_bytes() = 32 MiB that every GPU the library runs on holds until the process ends;
+ * the rows are worked through in chunks that fit, so T is unlimited and only max_seqlen is bounded:
+ * max_seqlen > dsa_index_topk_noalloc_max_seqlen() (2 097 152) returns DSA_ERR_WORKSPACE.  The call allocates
+ * nothing and frees nothing.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (two
+ * streams, two threads) race and must be serialised by the caller; calls on different GPUs are independent.
+ */
+int dsa_index_topk_noalloc(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu_seqlens, int T,
+                           int N, int Hi, int Di, int K, float scale, int dtype, int max_seqlen, int32_t *idx,
+                           int32_t *n, void *stream);
+size_t dsa_index_topk_noalloc_scratch_bytes(void);
+int dsa_index_topk_noalloc_max_seqlen(void);
+
+/*
  * dsa_index_topk that also returns the indexer scores of the selected keys: sel_scores[t*K + j] = score of key
  * idx[t*K + j] (0 for j >= n[t]).  Every row is scored here, also those whose whole causal window is selected.
  * No reference counterpart (the reference holds no indexer); serves the indexer's training loss below.

@@ -25,6 +25,10 @@ _SIGNATURES = {
     "dsa_index_topk_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "dsa_index_topk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "dsa_index_topk_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
+                                       c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "dsa_index_topk_noalloc_scratch_bytes": (c_size_t, []),
+    "dsa_index_topk_noalloc_max_seqlen": (c_int, []),
     "dsa_index_topk_scores": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
                                       c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "dsa_indexer_kl": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p]),

@@ -1,5 +1,6 @@
 // C ABI of the library (declared in include/dsa_attn.h): argument checks, workspace layout, launches.
 #include <hip/hip_runtime.h>
+#include <mutex>
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -170,6 +171,51 @@ extern "C" int dsa_index_topk_scores(const void *q_idx, const void *k_idx, const
     if (!sel_scores) return fail(DSA_ERR_ARG, "null output pointer");
     return index_topk_impl(q_idx, k_idx, w_idx, cu, T, N, Hi, Di, K, scale, dtype, max_seqlen, idx, n, sel_scores, ws,
                            ws_bytes, stream);
+}
+
+// ---- dsa_index_topk for callers that cannot allocate -------------------------------------------------------
+// The score rows live in a file-scope device array instead of a caller's workspace.  Its name is a host-side handle,
+// not a device address: the address is looked up once per device (every GPU holds its own copy of the array) and only
+// that pointer is ever handed to a kernel.
+#define DSA_SCRATCH_BYTES ((size_t)32 << 20)
+#define DSA_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[DSA_SCRATCH_BYTES];
+static void *g_scratch_ptr[DSA_MAX_DEVICES];
+static std::mutex g_scratch_mu;
+
+static int scratch_of_current_device(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    if (dev < 0 || dev >= DSA_MAX_DEVICES) return fail(DSA_ERR_UNSUPPORTED, "device %d: the static scratch serves devices 0..%d", dev, DSA_MAX_DEVICES - 1);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return DSA_OK;
+}
+
+extern "C" size_t dsa_index_topk_noalloc_scratch_bytes(void) { return DSA_SCRATCH_BYTES; }
+// longest segment whose four score rows (the smallest chunk the chunked loop works on) fit the scratch
+extern "C" int dsa_index_topk_noalloc_max_seqlen(void) { return (int)(DSA_SCRATCH_BYTES / (4 * sizeof(float)) / 32 * 32); }
+
+extern "C" int dsa_index_topk_noalloc(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu, int T,
+                                      int N, int Hi, int Di, int K, float scale, int dtype, int max_seqlen, int32_t *idx,
+                                      int32_t *n, void *stream) {
+    if (max_seqlen > dsa_index_topk_noalloc_max_seqlen())
+        return fail(DSA_ERR_WORKSPACE, "max_seqlen=%d: the %zu-byte static scratch holds score rows of at most %d columns; "
+                    "use dsa_index_topk with a workspace of your own", max_seqlen, DSA_SCRATCH_BYTES,
+                    dsa_index_topk_noalloc_max_seqlen());
+    void *ws = nullptr;
+    if (int rc = scratch_of_current_device(&ws)) return rc;
+    // nothing in the scratch has to start at zero: the indexer writes every column [0, pos] of a row before the
+    // selection reads it, and rows whose whole window is selected are never read
+    return index_topk_impl(q_idx, k_idx, w_idx, cu, T, N, Hi, Di, K, scale, dtype, max_seqlen, idx, n, nullptr, ws,
+                           DSA_SCRATCH_BYTES, stream);
 }
 
 extern "C" int dsa_indexer_kl(const float *sel_scores, const float *mass, const int32_t *n, int T, int K, float grad_scale,
