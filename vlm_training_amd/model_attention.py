@@ -9,6 +9,10 @@
   (torch 2.11 ``window_size=(-1, 0)`` form used by the reference, torch 2.10 ``is_causal=`` form).
 * ``run_varlen_attn`` - models/qwen3_5/model.py:90-98 (``SelfAttention._run_varlen_attn``).
 
+* ``qwen3_forward`` / ``qwen3vl_forward`` / ``qwen3_5_forward`` - train/model_attention.py:146-252, the forwards
+  the reference installs on the HF attention classes, and ``replace_attention_qwenvl`` / ``return_mask``
+  (train/model_attention.py:255-299), the installer.
+
 All of them take the DSA extension as keyword-only arguments (default off = reference behaviour).
 """
 from __future__ import annotations
@@ -107,3 +111,82 @@ def varlen_attention_forward(query, key, value, attention_mask, max_seqlen=None,
     if isinstance(attn_output, tuple):
         return (attn_output[0].unsqueeze(0), None) + tuple(attn_output[1:])
     return attn_output.unsqueeze(0), None
+
+
+# ------------------------------------------------------------------------------------------------------------
+# forwards for the HF attention classes (train/model_attention.py:146-252) and their installer (:255-299)
+# ------------------------------------------------------------------------------------------------------------
+def _hf_layer_forward(self, hidden_states, position_embeddings, attention_mask, gated: bool, offset: bool):
+    """q/k/v projections -> fused norm + RoPE -> packed attention (-> gate) -> o_proj on an HF attention module
+    (``self`` holds q_proj, k_proj, v_proj, o_proj, q_norm, k_norm, head_dim).  ``attention_mask`` carries the 1-D
+    cu_seqlens (``return_mask`` below makes HF pass it through untouched).  Returns ``(attn_output, None)``."""
+    from .dtensor_utils import _dtensor_rewrap, _dtensor_unwrap
+    from .layers import attention_core
+    input_shape = hidden_states.shape[:-1]
+    D = self.head_dim
+    total = 1
+    for s_ in input_shape:
+        total *= s_
+    qp = self.q_proj(hidden_states)
+    if gated:                                              # per head [q | gate] (train/model_attention.py:156-158)
+        qg = qp.view(total, -1, 2 * D)
+        k = self.k_proj(hidden_states).view(total, -1, D)
+        v = self.v_proj(hidden_states).view(total, -1, D)
+        (qg, k, v), wrap = _dtensor_unwrap(qg, k, v)
+        q, gate = qg[..., :D], qg[..., D:]
+    else:
+        q = qp.view(total, -1, D)
+        k = self.k_proj(hidden_states).view(total, -1, D)
+        v = self.v_proj(hidden_states).view(total, -1, D)
+        (q, k, v), wrap = _dtensor_unwrap(q, k, v)
+        gate = None
+    cos, sin = position_embeddings
+    cu_seqlens = attention_mask.reshape(-1)
+    out = attention_core(self, q, k, v, cos, sin, cu_seqlens, longest_segment(cu_seqlens), x=hidden_states, gate=gate,
+                         offset=offset)
+    out = _dtensor_rewrap(out, wrap)
+    out = out.reshape(*input_shape, -1).to(hidden_states.dtype)
+    return self.o_proj(out), None
+
+
+def qwen3_5_forward(self, hidden_states, position_embeddings, attention_mask, **kwargs):
+    """train/model_attention.py:146-185: gated, (1 + weight) norms."""
+    return _hf_layer_forward(self, hidden_states, position_embeddings, attention_mask, gated=True, offset=True)
+
+
+def qwen3_forward(self, hidden_states, position_embeddings, attention_mask, **kwargs):
+    """train/model_attention.py:188-219."""
+    return _hf_layer_forward(self, hidden_states, position_embeddings, attention_mask, gated=False, offset=False)
+
+
+def qwen3vl_forward(self, hidden_states, position_embeddings, attention_mask, **kwargs):
+    """train/model_attention.py:221-252."""
+    return _hf_layer_forward(self, hidden_states, position_embeddings, attention_mask, gated=False, offset=False)
+
+
+def return_mask(attention_mask, **kwargs):
+    """Stands in for HF's ``create_causal_mask`` so that the raw cu_seqlens reaches the attention layers
+    (train/model_attention.py:255-262)."""
+    return attention_mask.unsqueeze_(0)
+
+
+def replace_attention_qwenvl():
+    """Install the forwards above on the HF Qwen3 / Qwen3-VL / Qwen3-VL-MoE / Qwen3.5 attention classes and replace
+    their ``create_causal_mask`` (train/model_attention.py:265-299).  Returns the list of (owner, attribute, previous
+    value) it replaced, so that a caller (or a test) can put everything back."""
+    import importlib
+    targets = (
+        ("transformers.models.qwen3.modeling_qwen3", "Qwen3Attention", qwen3vl_forward),
+        ("transformers.models.qwen3_vl.modeling_qwen3_vl", "Qwen3VLTextAttention", qwen3vl_forward),
+        ("transformers.models.qwen3_vl_moe.modeling_qwen3_vl_moe", "Qwen3VLMoeTextAttention", qwen3vl_forward),
+        ("transformers.models.qwen3_5.modeling_qwen3_5", "Qwen3_5Attention", qwen3_5_forward),
+    )
+    undo = []
+    for mod_name, cls_name, fwd in targets:
+        mod = importlib.import_module(mod_name)
+        cls = getattr(mod, cls_name)
+        undo.append((cls, "forward", cls.forward))
+        cls.forward = fwd
+        undo.append((mod, "create_causal_mask", mod.create_causal_mask))
+        mod.create_causal_mask = return_mask
+    return undo
