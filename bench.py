@@ -38,27 +38,46 @@ def timed(fn, iters, warmup=1):
     return beg.elapsed_time(end) / iters
 
 
-def cpu_baseline(w, threads):
-    """Oracle (fp32 torch, CPU) fwd+bwd on one segment of the workload, scaled by causal pairs."""
+def cpu_baseline(w, threads, sample_only=False):
+    """The CPU oracle (fp32 torch) fwd+bwd on this box's host cores: the whole workload, one segment at a time
+    (segments are independent), or - ``sample_only`` - one long segment scaled by causal pairs.  Beside it the dense
+    restatement of the operator the reference itself calls (per-segment causal attention with repeat_kv GQA,
+    models/qwen3/model.py:125-129,166-169), fwd+bwd on the same tensors."""
     from oracle import dsa_ref as R
     from vlm_training_amd import workloads as W
-    # sample: one long segment (rows below and above top_k), capped so that the default run stays short
-    cands = [L for L in w.seg_lens if L > w.top_k] or [max(w.seg_lens)]
-    L = min(max(cands), 6144)           # about 10 s of host work at the headline geometry
-    sw = W.scaled(w, (L,), name=w.name + "-cpu-sample")
-    t = W.make_inputs(sw, device="cpu")
     torch.set_num_threads(threads)
-    t0 = time.perf_counter()
-    idx, n = R.dsa_select(t["q_idx"], t["k_idx"], t["w_idx"], sw.cu, sw.top_k)
-    R.sparse_attention_grads(t["q"], t["k"], t["v"], idx, n, sw.cu, t["dout"])
-    dt = time.perf_counter() - t0
-    P_s, _ = sw.pair_counts()
     P, _ = w.pair_counts()
-    est_total = dt * P / P_s            # the oracle's cost is proportional to causal pairs
+    if sample_only or P > 2e8:                              # C4: 8.6e9 pairs do not finish in minutes
+        cands = [L for L in w.seg_lens if L > w.top_k] or [max(w.seg_lens)]
+        L = min(max(cands), 6144)
+        sw = W.scaled(w, (L,), name=w.name + "-cpu-sample")
+        what = f"one {L}-token segment of {w.name}"
+    else:
+        sw, what = w, f"the whole of {w.name}, segment by segment"
+    t = W.make_inputs(sw, device="cpu")
+    P_s, _ = sw.pair_counts()
+    cu = sw.cu
+    t0 = time.perf_counter()
+    for a, b in zip(cu[:-1], cu[1:]):
+        if b == a:
+            continue
+        idx, n = R.dsa_select(t["q_idx"][a:b], t["k_idx"][a:b], t["w_idx"][a:b], [0, b - a], sw.top_k)
+        R.sparse_attention_grads(t["q"][a:b], t["k"][a:b], t["v"][a:b], idx, n, [0, b - a], t["dout"][a:b])
+    dt = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    for a, b in zip(cu[:-1], cu[1:]):
+        if b == a:
+            continue
+        q, k, v = (t[x][a:b].float().requires_grad_(True) for x in ("q", "k", "v"))
+        R.dense_varlen_causal(q, k, v, [0, b - a]).backward(t["dout"][a:b].float())
+    dt_dense = time.perf_counter() - t0
+    est, est_dense = dt * P / P_s, dt_dense * P / P_s       # the oracle's cost is proportional to causal pairs
+    scaled = "" if sw is w else f"; scaled by causal pairs ({P_s} of {P}) to the whole batch"
     return {
-        "value": w.T / est_total, "unit": "tokens/s", "cores": threads, "kind": "port",
-        "sample": f"oracle fwd+bwd on one {L}-token segment of {w.name} ({P_s} of {P} causal pairs) took {dt:.2f} s; "
-                  f"scaled by causal pairs to the whole batch",
+        "value": w.T / est, "unit": "tokens/s", "cores": threads, "kind": "port",
+        "sample": f"DSA oracle (indexer, top-k, sparse attention fwd+bwd) on {what}: {dt:.2f} s{scaled}",
+        "dense_reference_operator": {"value": w.T / est_dense, "unit": "tokens/s", "seconds": dt_dense,
+                                     "what": "dense causal packed attention fwd+bwd (what the reference calls), same tensors"},
     }
 
 
@@ -201,10 +220,12 @@ def vision_tower_operator(dev, iters):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)   # the first steps after start-up run a few percent slower
     ap.add_argument("--workload", default="C3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample", action="store_true", help="time the CPU oracle on one segment only (about 10 s) instead of the whole workload")
+    ap.add_argument("--only-step", action="store_true", help="the timed steps and the roofline line only (for profiler runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy (a known-size kernel to scale rocprof's FETCH_SIZE/WRITE_SIZE by)")
     args = ap.parse_args()
@@ -241,19 +262,21 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     wall0 = time.perf_counter()
-    beg.record()
-    for _ in range(args.steps):
+    marks[0].record()
+    for i in range(args.steps):
         step()
-    end.record()
+        marks[i + 1].record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - wall0) * 1e3 / args.steps
-    ms_per_step = max(beg.elapsed_time(end) / args.steps, wall_ms)
+    ms_per_step = max(marks[0].elapsed_time(marks[-1]) / args.steps, wall_ms)
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+    pct = lambda f: per_step[min(len(per_step) - 1, int(f * len(per_step)))]
     tokens_per_s = w.T / (ms_per_step * 1e-3)
 
     # ---- per-stage times (each kernel alone, same stream) ------------------------------------
-    it = max(2, min(args.steps, 5))
+    it = max(2, min(args.steps, 20))
     with torch.no_grad():
         qd, kd, vd = q.detach(), k.detach(), v.detach()
         idx, n = ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k)
@@ -287,6 +310,7 @@ def main():
         "attn_bwd": max(wk["F4"] / (PEAK_MFMA_BF16_TFLOPS * 1e12), wk["B4"] / (PEAK_HBM_GBS * 1e9)) * 1e3,
     }
     roof_total = sum(t_roof_ms.values())
+    compute_bound_ms = (wk["F1"] + 3.5 * wk["F3"]) / (PEAK_MFMA_BF16_TFLOPS * 1e12) * 1e3
     traffic = None      # HBM bytes per launch as last measured with rocprofv3 --pmc (separate runs)
     try:
         with open(os.path.join(ROOT, "profiles", f"hbm_traffic_{args.workload}.json")) as fh:
@@ -302,22 +326,26 @@ def main():
                                f"indexer {w.Hi}x{w.Di}, top_k={w.top_k}, fwd+bwd"},
         "roofline": {"bound": "mfma", "kernel": dom_kernel, "achieved": achieved, "peak": PEAK_MFMA_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_BF16_TFLOPS, "traffic": traffic,
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command, scaled by a 1 GiB copy (profiles/)",
                      "algorithmic_flop": dom_flop, "avg_ms": stage_ms[dom]},
         "stage_ms": stage_ms,
-        "roofline_whole_op": {"t_roof_ms": t_roof_ms, "sum_ms": roof_total, "frac": roof_total / ms_per_step,
-                              "compute_only_bound_ms": (wk["F1"] + 3.5 * wk["F3"]) / (PEAK_MFMA_BF16_TFLOPS * 1e12) * 1e3,
-                              "note": "t_roof_ms prices the attention stages by the bytes a row gather of the selected keys "
-                                      "would move (the nominal roofline the target was derived from); the tile kernels "
-                                      "do not gather, so frac > 1 means that bound was left behind - roofline.frac is the "
-                                      "figure of merit of the dominant kernel"},
+        "ms_per_step_median": pct(0.5), "ms_per_step_p10": pct(0.1), "ms_per_step_p90": pct(0.9),
+        "roofline_whole_op": {"compute_only_bound_ms": compute_bound_ms, "frac_compute_only": compute_bound_ms / ms_per_step,
+                              "nominal_gather_roofline_ms": roof_total, "nominal_t_roof_ms": t_roof_ms,
+                              "note": "compute_only_bound = (F1 + 3.5*F3) / bf16 MFMA peak: selected-pair flop of indexer, "
+                                      "forward and backward, the ceiling that applies to the tile kernels; the nominal figure "
+                                      "prices the attention stages by the bytes a row gather of the selected keys would move, "
+                                      "which the tile kernels do not move (K and V stay in cache)"},
         "device": torch.cuda.get_device_name(0),
     }
-    result["adjacent_kernels"] = prologue_stage(w, dev, it)
-    result["reference_operator"] = reference_operator(w, t, it)
-    result["vision_tower_operator"] = vision_tower_operator(dev, it)
-    result["indexer_training"] = indexer_target_stage(w, t, it)
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(w, torch.get_num_threads())
+    if not args.only_step:
+        it = min(it, 5)
+        result["adjacent_kernels"] = prologue_stage(w, dev, it)
+        result["reference_operator"] = reference_operator(w, t, it)
+        result["vision_tower_operator"] = vision_tower_operator(dev, it)
+        result["indexer_training"] = indexer_target_stage(w, t, it)
+    if not args.no_cpu_baseline and not args.only_step:
+        result["cpu_baseline"] = cpu_baseline(w, torch.get_num_threads(), sample_only=args.cpu_sample)
     print(json.dumps(result))
 
 

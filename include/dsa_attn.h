@@ -244,6 +244,16 @@ int dsa_sigmoid_gate_bwd(const void *gy, const void *x, const void *gate, int64_
                          int64_t gate_head_stride, int T, int H, int D, void *dx, void *dgate, int64_t dgate_tok_stride,
                          int64_t dgate_head_stride, void *stream);
 
+/*
+ * fp32 operands on the bf16 kernels (no reference counterpart: the reference runs the operator in bf16 under autocast;
+ * this serves fp32 callers such as the CPU-runnable toy configuration).  x (rows, D) fp32 -> y (rows, 4*D) bf16 holding
+ * hi = bf16(x) and lo = bf16(x - hi) stacked along the last dimension: order 0 = [hi, lo, hi, 0] (q, v), order 1 =
+ * [hi, hi, lo, 0] (k, dO), so that <q', k'> = <q, k> - <q_lo, k_lo>.  dsa_split_bf16_combine is the way back:
+ * out[r, :] = y[r, 0:D] + y[r, part*D:(part+1)*D] in fp32 (part 1: out, dk; part 2: dq, dv).  D % 4 == 0.
+ */
+int dsa_split_bf16_stack(const float *x, int64_t rows, int D, int order, void *y, void *stream);
+int dsa_split_bf16_combine(const void *y, int64_t rows, int D, int part, float *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -60,6 +60,8 @@ hipError_t dsa_launch_qk_norm_rope_bwd(const void *gq, const void *gk, const voi
                                        float *dqw, float *dkw, float *part, hipStream_t stream);
 hipError_t dsa_launch_sigmoid_gate_fwd(const void *x, const void *gate, int64_t gate_tok, int64_t gate_head, int D, int H,
                                        int64_t rows, void *y, hipStream_t stream);
+hipError_t dsa_launch_split_stack(const float *x, int64_t rows, int D, int order, void *y, hipStream_t stream);
+hipError_t dsa_launch_split_combine(const void *y, int64_t rows, int D, int part, float *out, hipStream_t stream);
 hipError_t dsa_launch_sigmoid_gate_bwd(const void *gy, const void *x, const void *gate, int64_t gate_tok, int64_t gate_head,
                                        int D, int H, int64_t rows, void *dx, void *dgate, int64_t dgate_tok,
                                        int64_t dgate_head, hipStream_t stream);
@@ -509,4 +511,18 @@ extern "C" int dsa_sigmoid_gate_bwd(const void *gy, const void *x, const void *g
     hipError_t e = dsa_launch_sigmoid_gate_bwd(gy, x, gate, gate_tok, gate_head, D, H, T, dx, dgate, dgate_tok, dgate_head,
                                                (hipStream_t)stream);
     return e == hipSuccess ? DSA_OK : hip_fail(e, "sigmoid gate backward launch");
+}
+
+// ---- fp32 operands carried as stacked split-bf16 rows (the host operator's fp32 path for head_dim <= 64) ----
+extern "C" int dsa_split_bf16_stack(const float *x, int64_t rows, int D, int order, void *y, void *stream) {
+    if (rows < 0 || D < 4 || D % 4 || (order != 0 && order != 1)) return fail(DSA_ERR_ARG, "rows=%lld D=%d order=%d", (long long)rows, D, order);
+    if (rows > 0 && (!x || !y)) return fail(DSA_ERR_ARG, "null tensor pointer");
+    hipError_t e = dsa_launch_split_stack(x, rows, D, order, y, (hipStream_t)stream);
+    return e == hipSuccess ? DSA_OK : hip_fail(e, "split/stack launch");
+}
+extern "C" int dsa_split_bf16_combine(const void *y, int64_t rows, int D, int part, float *out, void *stream) {
+    if (rows < 0 || D < 4 || D % 4 || part < 1 || part > 3) return fail(DSA_ERR_ARG, "rows=%lld D=%d part=%d", (long long)rows, D, part);
+    if (rows > 0 && (!y || !out)) return fail(DSA_ERR_ARG, "null tensor pointer");
+    hipError_t e = dsa_launch_split_combine(y, rows, D, part, out, (hipStream_t)stream);
+    return e == hipSuccess ? DSA_OK : hip_fail(e, "split/combine launch");
 }

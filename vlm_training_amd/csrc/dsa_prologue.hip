@@ -309,3 +309,57 @@ extern "C" hipError_t dsa_launch_sigmoid_gate_bwd(const void *gy, const void *x,
                        dgate_head);
     return hipGetLastError();
 }
+
+// ---------------------------------------------------------------------------------------------------
+// fp32 operands on the bf16 kernels: x = hi + lo with hi = bf16(x), lo = bf16(x - hi), the parts stacked along
+// head_dim into rows of 4*D bf16 so that the products of the stacked operands give back near-fp32 logits:
+//   order 0: [hi, lo, hi, 0]  (q, v)        order 1: [hi, hi, lo, 0]  (k, dO)
+// and the way back, out[r, :] = y[r, 0:D] + y[r, part*D:(part+1)*D] in fp32.  One thread per 4 elements.
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void dsa_split_stack_kernel(const float *__restrict__ x, int64_t rows, int D, int order,
+                                                               bf16_t *__restrict__ y) {
+    const int64_t n4 = rows * (D / 4);
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
+        const int64_t r = i / (D / 4);
+        const int c = (int)(i % (D / 4)) * 4;
+        const f32x4 v = *reinterpret_cast<const f32x4 *>(x + r * D + c);
+        const uint32_t h0 = pack2bf(v[0], v[1]), h1 = pack2bf(v[2], v[3]);
+        const uint32_t l0 = pack2bf(v[0] - __uint_as_float(h0 << 16), v[1] - __uint_as_float(h0 & 0xffff0000u));
+        const uint32_t l1 = pack2bf(v[2] - __uint_as_float(h1 << 16), v[3] - __uint_as_float(h1 & 0xffff0000u));
+        bf16_t *o = y + r * 4 * D + c;
+        const u32x2 hi = {h0, h1}, lo = {l0, l1}, z = {0u, 0u};
+        *reinterpret_cast<u32x2 *>(o) = hi;
+        *reinterpret_cast<u32x2 *>(o + D) = order ? hi : lo;
+        *reinterpret_cast<u32x2 *>(o + 2 * D) = order ? lo : hi;
+        *reinterpret_cast<u32x2 *>(o + 3 * D) = z;
+    }
+}
+__global__ __launch_bounds__(256) void dsa_split_combine_kernel(const bf16_t *__restrict__ y, int64_t rows, int D, int part,
+                                                                 float *__restrict__ out) {
+    const int64_t n4 = rows * (D / 4);
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
+        const int64_t r = i / (D / 4);
+        const int c = (int)(i % (D / 4)) * 4;
+        const u32x2 a = *reinterpret_cast<const u32x2 *>(y + r * 4 * D + c);
+        const u32x2 b = *reinterpret_cast<const u32x2 *>(y + r * 4 * D + part * D + c);
+        const f32x4 o = {__uint_as_float(a[0] << 16) + __uint_as_float(b[0] << 16),
+                         __uint_as_float(a[0] & 0xffff0000u) + __uint_as_float(b[0] & 0xffff0000u),
+                         __uint_as_float(a[1] << 16) + __uint_as_float(b[1] << 16),
+                         __uint_as_float(a[1] & 0xffff0000u) + __uint_as_float(b[1] & 0xffff0000u)};
+        *reinterpret_cast<f32x4 *>(out + r * D + c) = o;
+    }
+}
+extern "C" hipError_t dsa_launch_split_stack(const float *x, int64_t rows, int D, int order, void *y, hipStream_t stream) {
+    const int64_t n4 = rows * (D / 4);
+    if (n4 == 0) return hipSuccess;
+    const int nb = (int)((n4 + 255) / 256 > 8192 ? 8192 : (n4 + 255) / 256);
+    hipLaunchKernelGGL(dsa_split_stack_kernel, dim3(nb), dim3(256), 0, stream, x, rows, D, order, (bf16_t *)y);
+    return hipGetLastError();
+}
+extern "C" hipError_t dsa_launch_split_combine(const void *y, int64_t rows, int D, int part, float *out, hipStream_t stream) {
+    const int64_t n4 = rows * (D / 4);
+    if (n4 == 0) return hipSuccess;
+    const int nb = (int)((n4 + 255) / 256 > 8192 ? 8192 : (n4 + 255) / 256);
+    hipLaunchKernelGGL(dsa_split_combine_kernel, dim3(nb), dim3(256), 0, stream, (const bf16_t *)y, rows, D, part, out);
+    return hipGetLastError();
+}

@@ -312,16 +312,24 @@ def attn_bwd(dout, q, k, v, out, lse, idx, n, cu_seqlens, max_seqlen: int, softm
 # ------------------------------------------------------------------------------------------------
 # the operator
 # ------------------------------------------------------------------------------------------------
-def _split_bf16(x: torch.Tensor):
-    hi = x.to(torch.bfloat16)
-    lo = (x.float() - hi.float()).to(torch.bfloat16)
-    return hi, lo
+def _split_stack(x: torch.Tensor, order: int) -> torch.Tensor:
+    """fp32 (T,H,D) -> bf16 (T,H,4D): hi = bf16(x), lo = bf16(x - hi) stacked along head_dim, order 0 = [hi, lo, hi, 0],
+    order 1 = [hi, hi, lo, 0] (one kernel)."""
+    x = x.contiguous()
+    T, H, D = x.shape
+    y = torch.empty((T, H, 4 * D), dtype=torch.bfloat16, device=x.device)
+    rc = _lib.load().dsa_split_bf16_stack(_ptr(x), T * H, D, order, _ptr(y), _stream(x.device))
+    _lib.check(rc, "dsa_split_bf16_stack")
+    return y
 
 
-def _stack(parts, D):
-    """Concatenate bf16 parts along head_dim and zero-pad to 4*D (a head_dim the kernels cover)."""
-    z = torch.zeros_like(parts[0])
-    return torch.cat(list(parts) + [z] * (4 - len(parts)), dim=-1).contiguous()
+def _split_combine(y: torch.Tensor, part: int) -> torch.Tensor:
+    """bf16 (T,H,4D) -> fp32 (T,H,D): y[..., :D] + y[..., part*D:(part+1)*D] (one kernel)."""
+    T, H, D4 = y.shape
+    out = torch.empty((T, H, D4 // 4), dtype=torch.float32, device=y.device)
+    rc = _lib.load().dsa_split_bf16_combine(_ptr(y), T * H, D4 // 4, part, _ptr(out), _stream(y.device))
+    _lib.check(rc, "dsa_split_bf16_combine")
+    return out
 
 
 class _DsaVarlenAttn(torch.autograd.Function):
@@ -339,8 +347,7 @@ class _DsaVarlenAttn(torch.autograd.Function):
         D = q.shape[-1]
         split = in_dtype == torch.float32 and 4 * D <= 256
         if split:
-            (qh, ql), (kh, kl), (vh, vl) = _split_bf16(q), _split_bf16(k), _split_bf16(v)
-            qb, kb, vb = _stack((qh, ql, qh), D), _stack((kh, kh, kl), D), _stack((vh, vl, vh), D)
+            qb, kb, vb = _split_stack(q, 0), _split_stack(k, 1), _split_stack(v, 0)
         else:
             qb, kb, vb = _as_bf16(q), _as_bf16(k), _as_bf16(v)
         bwd_ws = None
@@ -364,7 +371,7 @@ class _DsaVarlenAttn(torch.autograd.Function):
         ctx.split = split
         ctx.D = D
         if split:
-            res = out[..., :D].float() + out[..., D:2 * D].float()
+            res = _split_combine(out, 1)
         else:
             res = out if in_dtype == torch.bfloat16 else out.to(in_dtype)
         if not want_mass:
@@ -381,8 +388,7 @@ class _DsaVarlenAttn(torch.autograd.Function):
         idx, n = (saved[6], saved[7]) if ctx.has_idx else (None, None)
         D = ctx.D
         if ctx.split:
-            gh, gl = _split_bf16(dout)
-            db = _stack((gh, gh, gl), D)
+            db = _split_stack(dout.float(), 1)
         else:
             db = _as_bf16(dout)
         if ctx.bwd_ws is not None:                       # the forward left the selection bitmap in the workspace
@@ -394,9 +400,7 @@ class _DsaVarlenAttn(torch.autograd.Function):
             dq, dk, dv = attn_bwd(db, qb, kb, vb, out, lse, idx, n, cu, ctx.max_seqlen, ctx.softmax_scale,
                                   causal=ctx.causal)
         if ctx.split:
-            dq = dq[..., :D].float() + dq[..., 2 * D:3 * D].float()
-            dk = dk[..., :D].float() + dk[..., D:2 * D].float()
-            dv = dv[..., :D].float() + dv[..., 2 * D:3 * D].float()
+            dq, dk, dv = _split_combine(dq, 2), _split_combine(dk, 1), _split_combine(dv, 2)
         elif ctx.in_dtype != torch.bfloat16:
             dq, dk, dv = dq.to(ctx.in_dtype), dk.to(ctx.in_dtype), dv.to(ctx.in_dtype)
         return dq, dk, dv, None, None, None, None, None, None, None
