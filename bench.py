@@ -225,6 +225,8 @@ def main():
     ap.add_argument("--workload", default="C3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample", action="store_true", help="time the CPU oracle on one segment only (about 10 s) instead of the whole workload")
+    ap.add_argument("--crossover", type=int, default=None,
+                    help="tile/gather split (rows with pos < top_k * crossover run on the tile kernels; 0 = gather kernels only)")
     ap.add_argument("--only-step", action="store_true", help="the timed steps and the roofline line only (for profiler runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy (a known-size kernel to scale rocprof's FETCH_SIZE/WRITE_SIZE by)")
@@ -236,6 +238,8 @@ def main():
 
     from vlm_training_amd import ops, workloads as W
     w = W.WORKLOADS[args.workload]
+    if args.crossover is not None:
+        ops.set_tile_crossover(args.crossover)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     t = W.make_inputs(w, device=dev)
