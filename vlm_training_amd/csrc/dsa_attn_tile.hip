@@ -1279,6 +1279,445 @@ constexpr size_t dkvpc_lds_bytes() {
 }
 
 // ==================================================================================================
+// dK, dV for head_dim <= 128, "two chains" form.  The same key-stationary walk as dsa_tile_dkvpc_kernel
+// (a workgroup owns a 128-key tile of one segment and kv head and walks the later queries from the
+// segment end down, 32 (query, head) rows per step); the eight waves are split by GEMM chain, so that
+// neither P nor dS has to be handed over in full and every wave runs 16 MFMAs per step:
+//   waves 0-3 (P chain, one per 32-key group): S = Q K^T against the group's K rows in registers,
+//     started from -lse/scale so that P = exp2(S * scale*log2e) needs no subtraction, the selection bit
+//     applied before the exponential; dV^T += dO^T P with P going from the C layout of the first GEMM
+//     straight into the B operand of the second.  P also goes to LDS in bf16 for the other chain.
+//     Step s: S of block s, then the MFMAs of dV for block s-1 with the softmax of block s behind them.
+//   waves 4-7 (dS chain): dP = dO V^T against the group's V rows, started from -delta; dS = P (dP - delta)
+//     with the bf16 P read back from LDS; dK^T += Q^T dS, dS staying in registers.  Step s: block s-1.
+//     These waves also stage the q / dO blocks and the row data (two steps ahead in LDS, two more in
+//     registers).
+// One barrier per step; block s sits in ring slot s % 4 from step s-2 (staged) to step s+1 (last read),
+// P of block s in slot s % 2 of its ring from step s to step s+1.
+// Measured on this kernel's instruction mix (no memory traffic): one wave of each chain on a SIMD needs
+// about 1270 clocks per step against 1090 for the 32 MFMAs alone; the kernel runs at about 2000.
+// ==================================================================================================
+template <int D, bool HAS_IDX, int GSHIFT>
+__global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
+    const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
+    const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
+    const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
+    float scale, int causal, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    static_assert(D <= 128, "head_dim 256 runs dsa_tile_dkvpc_kernel");
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>();
+    constexpr int NCHUNK = 32 * CPR, STG = 256, CPT = NCHUNK / STG;
+    constexpr int Gp = 1 << GSHIFT, QB = 32 >> GSHIFT;
+    constexpr int QD_SLOT = 2 * TILE_B;                  // q block | dO block
+    constexpr int P_GROUP = 2 * 1024, P_SLOT = 4 * P_GROUP;   // per key group: P rows 0-15 | 16-31, 64 lanes x 16 B each
+    constexpr int AUX_SLOT = (32 + 32 + 4 * 32) * 4;     // lse | delta | selection words [key group][query]
+    static_assert(CPT >= 1 && NCHUNK % STG == 0, "every staging thread stages whole chunks");
+    extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
+    unsigned char *const qd_ring = dyn_lds;                          // 4 slots
+    unsigned char *const p_ring = dyn_lds + 4 * QD_SLOT;             // 2 slots
+    unsigned char *const aux_ring = p_ring + 2 * P_SLOT;             // 4 slots
+
+    const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5, j = lane & 31;
+    LaneOffsets<D> lo;
+    lo.init(lane);
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kg = wv & 3;
+    const int G = Hq / Hkv;
+    const int kvh = blockIdx.x % Hkv;
+    int s0, L, blk;
+    if (!locate_block(cu, N, blockIdx.x / Hkv, 128, false, s0, L, blk)) return;
+    if (HAS_IDX) L = min(L, ldw * 32);
+    if (blk * 128 >= L) return;                         // (whole workgroup, before its first barrier)
+    const int c0 = blk * 128, kc = c0 + kg * 32;
+    const int mykey = kc + j;
+    const bool key_ok = mykey < L;
+    const int64_t krow = (int64_t)(s0 + min(mykey, L - 1)) * Hkv + kvh;
+    const float scale_log2 = scale * LOG2E_F, inv_scale = 1.f / scale;
+    const int q0 = causal ? c0 : 0;
+    const int nblocks = (L - q0 + QB - 1) / QB;          // queries q0 .. L-1; step s handles block nblocks-1-s
+
+    // an accumulator in C layout that starts from a per-row value (lane (key, h) holds rows 8 g4 + 4 h + e)
+    auto rows_init = [&](const float *rowv) __attribute__((always_inline)) {
+        f32x16 c;
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            const f32x4 r = *reinterpret_cast<const f32x4 *>(&rowv[8 * g4 + 4 * h]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) c[4 * g4 + e] = r[e];
+        }
+        return c;
+    };
+    // Staging: 16-byte chunks of the q and dO blocks, CPT of each per thread, and one word of row data per thread of
+    // the first 64 + 4 QB (lse, delta, selection words).  Step b reads block nblocks-1-b; the walk starts at the
+    // segment end, so only block 0 (rows past the end) and the steps past the last block need their rows zeroed.
+    const int ctid = tid & 255;                          // used by the dS chain's waves
+    const int last = nblocks - 1;
+    const int64_t blk_bytes = (int64_t)QB * Hq * D * 2;
+    const unsigned char *qp[CPT], *dp[CPT];
+    int64_t dlast[CPT];
+    int lds_off[CPT];
+    bool row_dead_last[CPT], head_ok[CPT];
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+        const int c = i * STG + ctid, srow = c / CPR, sch = c % CPR;
+        const int hd = min(srow & (Gp - 1), G - 1);
+        const int qr = srow >> GSHIFT;
+        const int over = max(q0 + last * QB + qr - (L - 1), 0);      // rows past the end in the last block
+        const int64_t off = ((int64_t)(s0 + q0 + last * QB + qr - over) * Hq + kvh * G + hd) * D + sch * 8;
+        qp[i] = reinterpret_cast<const unsigned char *>(q + off);
+        dp[i] = reinterpret_cast<const unsigned char *>(dout + off);
+        dlast[i] = -(int64_t)over * Hq * D * 2;
+        row_dead_last[i] = over > 0;
+        head_ok[i] = (srow & (Gp - 1)) < G;
+        lds_off[i] = tile_off<D>(srow, sch);
+    }
+    // row data: every thread loads one word and stores one word, threads without a share into a spare LDS word.
+    // lse and delta go in as -lse/scale and -delta (the chains start their accumulators from them), selection words
+    // as they are (zero for key groups past the bitmap row)
+    const uint32_t *aux_base = reinterpret_cast<const uint32_t *>(lse);
+    int aux_q = 0, aux_stride = 0, aux_lds = 4 * AUX_SLOT;          // spare word behind the four slots
+    float aux_mul = 0.f;
+    uint32_t aux_and = 0u;
+    bool aux_is_word = false;
+    if (ctid < 64) {                                 // 0..31: lse of row ctid, 32..63: delta of row ctid-32
+        const int row = ctid & 31;
+        const int hd = min(row & (Gp - 1), G - 1);
+        aux_q = row >> GSHIFT;
+        aux_stride = 1;
+        aux_base = reinterpret_cast<const uint32_t *>((ctid < 32 ? lse : delta) + (int64_t)(kvh * G + hd) * T + s0);
+        aux_mul = ctid < 32 ? -inv_scale : -1.f;
+        aux_lds = ctid * 4;
+    } else if (HAS_IDX && ctid < 64 + 4 * QB) {      // selection word of (key group w, query qi)
+        const int w = (ctid - 64) / QB;
+        aux_q = (ctid - 64) % QB;
+        aux_stride = ldw;
+        const bool ok = (c0 >> 5) + w < ldw;
+        aux_base = bitmap + (int64_t)s0 * ldw + (ok ? (c0 >> 5) + w : 0);
+        aux_and = ok ? 0xffffffffu : 0u;
+        aux_is_word = true;
+        aux_lds = (64 + w * 32 + aux_q) * 4;
+    }
+    const int64_t aux_blk_bytes = (int64_t)aux_stride * QB * 4;
+    const int aux_over = max(q0 + last * QB + aux_q - (L - 1), 0);
+    const int64_t aux_dlast = -(int64_t)aux_stride * aux_over * 4;
+    const unsigned char *ap =
+        reinterpret_cast<const unsigned char *>(aux_base + (int64_t)aux_stride * (q0 + last * QB + aux_q - aux_over));
+    u32x4 qst0[CPT], dost0[CPT], qst1[CPT], dost1[CPT];     // two register sets: a load has two steps to land
+    uint32_t aux_st0, aux_st1;
+    auto aux_value = [&](uint32_t x) __attribute__((always_inline)) {
+        return aux_is_word ? (x & aux_and) : __float_as_uint(__uint_as_float(x) * aux_mul);
+    };
+    // general forms (first and last steps): gload is called with b = 0, 1, 2, ... in turn; past step `last` it reads
+    // the first block again and lstore zeroes what it stores
+    auto gload = [&](int b, u32x4 (&qst)[CPT], u32x4 (&dost)[CPT], uint32_t &aux_st) __attribute__((always_inline)) {
+        if (b >= 1 && b <= last) {
+#pragma unroll
+            for (int i = 0; i < CPT; ++i) { qp[i] -= blk_bytes; dp[i] -= blk_bytes; }
+            ap -= aux_blk_bytes;
+            if (b == 1) {                            // leaving the last block: undo its row clamp
+#pragma unroll
+                for (int i = 0; i < CPT; ++i) { qp[i] -= dlast[i]; dp[i] -= dlast[i]; }
+                ap -= aux_dlast;
+            }
+        }
+        aux_st = *reinterpret_cast<const uint32_t *>(ap);   // first: its consumer then never waits for younger loads
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            qst[i] = *reinterpret_cast<const u32x4 *>(qp[i]);
+            dost[i] = *reinterpret_cast<const u32x4 *>(dp[i]);
+        }
+    };
+    auto lstore = [&](int b, const u32x4 (&qst)[CPT], const u32x4 (&dost)[CPT], uint32_t aux_st) __attribute__((always_inline)) {
+        unsigned char *slot = qd_ring + (b & 3) * QD_SLOT;
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const bool live = head_ok[i] && !(b > last || (b == 0 && row_dead_last[i]));
+            const u32x4 z4 = {0u, 0u, 0u, 0u};
+            *reinterpret_cast<u32x4 *>(slot + lds_off[i]) = live ? qst[i] : z4;
+            *reinterpret_cast<u32x4 *>(slot + TILE_B + lds_off[i]) = live ? dost[i] : z4;
+        }
+        const bool word_dead = aux_is_word && (b > last || (b == 0 && aux_over > 0));
+        *reinterpret_cast<uint32_t *>(aux_ring + (aux_lds < 4 * AUX_SLOT ? (b & 3) * AUX_SLOT : 0) + aux_lds) =
+            word_dead ? 0u : aux_value(aux_st);
+    };
+    // steady forms (blocks 2 .. last of a group whose heads fill the padded group): no branch, no select
+    auto gload_steady = [&](u32x4 (&qst)[CPT], u32x4 (&dost)[CPT], uint32_t &aux_st) __attribute__((always_inline)) {
+        ap -= aux_blk_bytes;
+        aux_st = *reinterpret_cast<const uint32_t *>(ap);
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            qp[i] -= blk_bytes;
+            dp[i] -= blk_bytes;
+            qst[i] = *reinterpret_cast<const u32x4 *>(qp[i]);
+            dost[i] = *reinterpret_cast<const u32x4 *>(dp[i]);
+        }
+    };
+    auto lstore_steady = [&](int b, const u32x4 (&qst)[CPT], const u32x4 (&dost)[CPT], uint32_t aux_st) __attribute__((always_inline)) {
+        unsigned char *slot = qd_ring + (b & 3) * QD_SLOT;
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            *reinterpret_cast<u32x4 *>(slot + lds_off[i]) = qst[i];
+            *reinterpret_cast<u32x4 *>(slot + TILE_B + lds_off[i]) = dost[i];
+        }
+        *reinterpret_cast<uint32_t *>(aux_ring + (aux_lds < 4 * AUX_SLOT ? (b & 3) * AUX_SLOT : 0) + aux_lds) = aux_value(aux_st);
+    };
+    if (wv >= 4) {
+        // ================= dS chain: staging, then dP, dS, dK of the block the P chain finished a step earlier =================
+        gload(0, qst0, dost0, aux_st0);
+        gload(1, qst1, dost1, aux_st1);
+        bf16x8 vB[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) vB[ks] = load_bf16x8(v + krow * D + 16 * ks + 8 * h);
+        lstore(0, qst0, dost0, aux_st0);
+        lstore(1, qst1, dost1, aux_st1);
+        gload(2, qst0, dost0, aux_st0);
+        gload(3, qst1, dost1, aux_st1);
+        __syncthreads();                                 // steps 0 and 1 staged
+
+        f32x16 dkacc[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) dkacc[dt] = zero16();
+        // dS of elements 8 half .. 8 half + 7 (C layout) as an MFMA B operand: the other chain's bf16 P times this
+        // chain's dP - delta
+        auto ds_half = [&](const u32x4 &w, const f32x16 &pacc, int half) __attribute__((always_inline)) {
+            float ds[8];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                ds[2 * e] = __uint_as_float(w[e] << 16) * pacc[8 * half + 2 * e];
+                ds[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u) * pacc[8 * half + 2 * e + 1];
+            }
+            return pack8(ds);
+        };
+        // block b: dP = dO V^T starting from -delta, dS, dK^T += Q^T dS.  Operand reads run three to four MFMAs ahead
+        // (every MFMA step ends in an empty asm statement that the next operand passes through, which fixes the
+        // order); the second half of dS is formed behind the first MFMAs of dK.
+        auto block = [&](int b) __attribute__((always_inline)) {
+            const unsigned char *qt = qd_ring + (b & 3) * QD_SLOT, *dot = qt + TILE_B;
+            const unsigned char *pd = p_ring + (b & 1) * P_SLOT + kg * P_GROUP + lane * 16;
+            f32x16 pacc = rows_init(reinterpret_cast<const float *>(aux_ring + (b & 3) * AUX_SLOT) + 32);
+            bf16x8 a[4], t[4];
+#pragma unroll
+            for (int i = 0; i < 4 && i < KS; ++i) a[i] = lo.rowop(dot, i);
+            const u32x4 w0 = *reinterpret_cast<const u32x4 *>(pd), w1 = *reinterpret_cast<const u32x4 *>(pd + 1024);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                pacc = mfma32(a[ks & 3], vB[ks], pacc);
+                if (ks + 4 < KS) a[ks & 3] = lo.rowop(dot, ks + 4);
+                if (ks + 3 >= KS) t[ks + 3 - KS] = lo.trop(qt, (ks + 3 - KS) / DT, (ks + 3 - KS) % DT);
+                if (ks + 1 < KS) asm volatile("" : "+v"(a[(ks + 1) & 3]) : : "memory");
+                else asm volatile("" : "+v"(t[0]) : : "memory");
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            const bf16x8 dB0 = ds_half(w0, pacc, 0);
+            uint32_t dw[4];
+#pragma unroll
+            for (int m = 0; m < 2 * DT; ++m) {
+                if (m < DT) dkacc[m] = mfma32(t[m & 3], dB0, dkacc[m]);
+                else {
+                    const u32x4 d1 = {dw[0], dw[1], dw[2], dw[3]};
+                    dkacc[m - DT] = mfma32(t[m & 3], __builtin_bit_cast(bf16x8, d1), dkacc[m - DT]);
+                }
+                if (m + 3 < 2 * DT) t[(m + 3) & 3] = lo.trop(qt, (m + 3) / DT, (m + 3) % DT);
+                if (m < DT) {                            // 4 / DT pairs of the second half of dS behind this MFMA
+#pragma unroll
+                    for (int u = 0; u < 4 / DT; ++u) {
+                        const int e = m * (4 / DT) + u;
+                        dw[e] = pack2bf(__uint_as_float(w1[e] << 16) * pacc[8 + 2 * e], __uint_as_float(w1[e] & 0xffff0000u) * pacc[9 + 2 * e]);
+                        asm volatile("" : "+v"(dw[e]));
+                    }
+                }
+                if (m + 1 < 2 * DT) asm volatile("" : "+v"(t[(m + 1) & 3]) : : "memory");
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+#define DKV2_DS_STEP(S, QS, DS_, AS)                                                                \
+    {                                                                                              \
+        lstore((S) + 2, QS, DS_, AS); /* its slot was last read (as step S-2) before the previous barrier */ \
+        gload((S) + 4, QS, DS_, AS);                                                               \
+        if ((S) >= 1) block((S) - 1);                                                              \
+        __syncthreads();                                                                             \
+    }
+#define DKV2_DS_STEADY(S, QS, DS_, AS)                                                              \
+    {                                                                                              \
+        lstore_steady((S) + 2, QS, DS_, AS);                                                       \
+        gload_steady(QS, DS_, AS);                                                                 \
+        block((S) - 1);                                                                            \
+        __syncthreads();                                                                             \
+    }
+        DKV2_DS_STEP(0, qst0, dost0, aux_st0)
+        int s = 1;
+        if (s <= nblocks) {
+            DKV2_DS_STEP(1, qst1, dost1, aux_st1)
+            s = 2;
+        }
+        if (G == Gp)                                     // steps whose staged block is 2 .. last and whose loaded block is 2 .. last
+            for (; s + 5 <= last; s += 2) {
+                DKV2_DS_STEADY(s, qst0, dost0, aux_st0)
+                DKV2_DS_STEADY(s + 1, qst1, dost1, aux_st1)
+            }
+        for (; s + 1 <= nblocks; s += 2) {
+            DKV2_DS_STEP(s, qst0, dost0, aux_st0)
+            DKV2_DS_STEP(s + 1, qst1, dost1, aux_st1)
+        }
+        if (s <= nblocks) DKV2_DS_STEP(s, qst0, dost0, aux_st0)
+#undef DKV2_DS_STEP
+#undef DKV2_DS_STEADY
+        if (key_ok) {
+            bf16_t *pk = dk + krow * D;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) store_c_tile(pk + dt * 32, dkacc[dt], scale, h);
+        }
+        return;
+    }
+
+    // ================= P chain: S and softmax of block s, dV of block s-1 =================
+    bf16x8 kB[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) kB[ks] = load_bf16x8(k + krow * D + 16 * ks + 8 * h);
+    uint32_t mw[16];
+    auto read_aux = [&](int b) __attribute__((always_inline)) {                         // selection words of step b
+        const uint32_t *mask_s = reinterpret_cast<const uint32_t *>(aux_ring + (b & 3) * AUX_SLOT) + 64 + kg * 32;
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (HAS_IDX && (e == 0 || GSHIFT < 2)) mw[4 * g4 + e] = mask_s[(8 * g4 + 4 * h + e) >> GSHIFT];
+    };
+    f32x16 dvacc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) dvacc[dt] = zero16();
+    // P of element vi (C layout) of step b from its S accumulator (which started from -lse/scale); pm collects the
+    // block's largest P
+    auto element = [&](auto may_diag, int b, int vi, const f32x16 &sacc, float sl2, uint32_t &keep, float &pm) __attribute__((always_inline)) {
+        const int g4 = vi >> 2, e = vi & 3, row = 8 * g4 + 4 * h + e;
+        if (e == 0 || GSHIFT < 2) {                      // rows of one query share the mask bit
+            const int qcb = q0 + (nblocks - 1 - b) * QB, qi = row >> GSHIFT;
+            uint32_t w = HAS_IDX ? mw[vi] : 0xffffffffu;
+            if (decltype(may_diag)::value && causal && qcb < kc + 32) w &= causal_bits(qcb + qi - kc);
+            keep = bit_mask(w, j);
+        }
+        const float p = fast_exp2(keep_or_neginf(sacc[vi] * sl2, keep));
+        pm = fmaxf(pm, p);
+        return p;
+    };
+    auto store_p = [&](int b, int half, bf16x8 p) __attribute__((always_inline)) {
+        *reinterpret_cast<bf16x8 *>(p_ring + (b & 1) * P_SLOT + kg * P_GROUP + half * 1024 + lane * 16) = p;
+    };
+    // P goes on in bf16.  dV[s] = sum over (query, head) of P dO piles the rounding of P (2^-9 relative) onto one key
+    // row; where probabilities are large (few keys per query) and many rows meet in one key, that noise reaches
+    // several 1e-2.  A block whose largest P is at least DKV_SPLIT_MIN therefore also adds dO^T (P - bf16(P)).
+    constexpr float DKV_SPLIT_MIN = 0.015625f;
+    auto remainder = [&](auto may_diag, int b, const f32x16 &sc, float pm, bf16x8 p0, bf16x8 p1) __attribute__((always_inline)) {
+        if (__builtin_amdgcn_ballot_w64(pm >= DKV_SPLIT_MIN) != 0ull) {   // wave-uniform, rare: P is formed again
+            const u32x4 w0 = __builtin_bit_cast(u32x4, p0), w1 = __builtin_bit_cast(u32x4, p1);
+            float pv[16], lo_[16], pm2 = 0.f;
+            uint32_t keep = 0u;
+#pragma unroll
+            for (int vi = 0; vi < 16; ++vi) pv[vi] = element(may_diag, b, vi, sc, scale_log2, keep, pm2);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                lo_[2 * e] = pv[2 * e] - __uint_as_float(w0[e] << 16);
+                lo_[2 * e + 1] = pv[2 * e + 1] - __uint_as_float(w0[e] & 0xffff0000u);
+                lo_[8 + 2 * e] = pv[8 + 2 * e] - __uint_as_float(w1[e] << 16);
+                lo_[9 + 2 * e] = pv[9 + 2 * e] - __uint_as_float(w1[e] & 0xffff0000u);
+            }
+            const unsigned char *dot = qd_ring + (b & 3) * QD_SLOT + TILE_B;
+            const bf16x8 l0 = pack8(lo_), l1 = pack8(lo_ + 8);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                dvacc[dt] = mfma32(lo.trop(dot, 0, dt), l0, dvacc[dt]);
+                dvacc[dt] = mfma32(lo.trop(dot, 1, dt), l1, dvacc[dt]);
+            }
+        }
+    };
+    // Step s: S of block s (KS MFMAs), then the 2 DT MFMAs of dV^T += dO^T P of block s-1 with the softmax of
+    // 16 / (2 DT) elements of block s behind each of them (operand reads three MFMAs ahead; every MFMA step ends in
+    // empty asm statements that its results and the next MFMA's operand pass through, which fixes the order).
+    bf16x8 pq0 = zero_bf16x8(), pq1 = zero_bf16x8();     // P of the block before, as B operands (rows 0-15 | 16-31)
+    auto step = [&](auto may_diag, auto has_cur, auto has_prev, int s) __attribute__((always_inline)) {
+        constexpr bool CUR = decltype(has_cur)::value, PREV = decltype(has_prev)::value;
+        constexpr int NM = 2 * DT, EPM = 16 / NM;
+        const unsigned char *qt = qd_ring + (s & 3) * QD_SLOT, *dprev = qd_ring + ((s - 1) & 3) * QD_SLOT + TILE_B;
+        f32x16 sacc;
+        if (CUR) {
+            sacc = rows_init(reinterpret_cast<const float *>(aux_ring + (s & 3) * AUX_SLOT));
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) sacc = mfma32(lo.rowop(qt, ks), kB[ks], sacc);
+            sched_reads_ahead<KS, (KS >= 4 ? 4 : KS), 1, 4>();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        float pv[2], pm = 0.f, sl2 = scale_log2;
+        uint32_t keep = 0u, pw[8];
+        bf16x8 t[4];
+        if (PREV) {
+#pragma unroll
+            for (int i = 0; i < 3 && i < NM; ++i) t[i] = lo.trop(dprev, i / DT, i % DT);
+        }
+#pragma unroll
+        for (int m = 0; m < NM; ++m) {
+            if (PREV) {
+                dvacc[m % DT] = mfma32(t[m & 3], m < DT ? pq0 : pq1, dvacc[m % DT]);
+                if (m + 3 < NM) t[(m + 3) & 3] = lo.trop(dprev, (m + 3) / DT, (m + 3) % DT);
+            }
+            if (CUR) {
+#pragma unroll
+                for (int u = 0; u < EPM; ++u) {          // P is packed pair by pair as it is formed
+                    const int vi = m * EPM + u;
+                    pv[vi & 1] = element(may_diag, s, vi, sacc, sl2, keep, pm);
+                    if (vi & 1) {
+                        pw[vi >> 1] = pack2bf(pv[0], pv[1]);
+                        asm volatile("" : "+v"(pw[vi >> 1]));
+                    } else {
+                        asm volatile("" : "+v"(pv[0]));
+                    }
+                }
+            }
+            if (PREV && m + 1 < NM) asm volatile("" : "+v"(sl2), "+v"(pm), "+v"(t[(m + 1) & 3]) : : "memory");
+            else asm volatile("" : "+v"(sl2), "+v"(pm) : : "memory");
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (CUR) {
+            const u32x4 w0 = {pw[0], pw[1], pw[2], pw[3]}, w1 = {pw[4], pw[5], pw[6], pw[7]};
+            pq0 = __builtin_bit_cast(bf16x8, w0);
+            pq1 = __builtin_bit_cast(bf16x8, w1);
+            store_p(s, 0, pq0);
+            store_p(s, 1, pq1);
+            remainder(may_diag, s, sacc, pm, pq0, pq1);
+            if (s + 1 < nblocks) read_aux(s + 1);
+        }
+    };
+    const std::true_type yes;
+    const std::false_type no;
+    __syncthreads();                                     // steps 0 and 1 staged
+    read_aux(0);
+    // The blocks that can touch the causal diagonal come last; the steady loop before them has no mask
+    // arithmetic besides the selection bits.
+    const int nb_diag = causal ? (kc + 32 - q0 + QB - 1) / QB : 0;
+    const int steady = max(nblocks - nb_diag, 1);        // steps [1, steady) see blocks fully past the diagonal
+    step(yes, yes, no, 0);
+    __syncthreads();
+    int s = 1;
+    for (; s < steady; ++s) {
+        step(no, yes, yes, s);
+        __syncthreads();
+    }
+    for (; s < nblocks; ++s) {
+        step(yes, yes, yes, s);
+        __syncthreads();
+    }
+    step(yes, no, yes, nblocks);
+    __syncthreads();
+    if (key_ok) {
+        bf16_t *pv_ = dv + krow * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) store_c_tile(pv_ + dt * 32, dvacc[dt], 1.f, h);
+    }
+}
+template <int D>
+constexpr size_t dkv2_lds_bytes() {   // q/dO ring, P ring, row-data ring and one spare word
+    return 4 * ((size_t)2 * tile_bytes<D>() + (32 + 32 + 4 * 32) * 4) + 2 * (4 * 2 * 1024) + 16;
+}
+
+// ==================================================================================================
 // launchers: instantiate per head_dim, mask kind and (power-of-two padded) group size
 // ==================================================================================================
 static inline int group_shift(int Hq, int Hkv) {
@@ -1317,6 +1756,15 @@ static hipError_t launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, 
                          int T, int Hq, int Hkv, float scale, int causal, void *dk, void *dv) {
     // LDS above 64 KiB has to be requested per kernel and device; asked for on every launch (a host-side table
     // lookup), so that neither a second device nor a second thread can meet a kernel that was never configured
+    if constexpr (D <= 128) {
+        const hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void *>(&dsa_tile_dkv2_kernel<D, HAS_IDX, GS>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkv2_lds_bytes<D>());
+        if (e2 != hipSuccess) return e2;
+        hipLaunchKernelGGL((dsa_tile_dkv2_kernel<D, HAS_IDX, GS>), grid, dim3(512), dkv2_lds_bytes<D>(), stream,
+                           (const bf16_t *)dout, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap,
+                           ldw, cu, N, T, Hq, Hkv, scale, causal, (bf16_t *)dk, (bf16_t *)dv);
+        return hipSuccess;
+    } else {
     const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(&dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkvpc_lds_bytes<D>());
     if (ea != hipSuccess) return ea;
@@ -1326,6 +1774,7 @@ static hipError_t launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, 
                            (const bf16_t *)dout, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap,
                            ldw, cu, N, T, Hq, Hkv, scale, causal, dhalf, (bf16_t *)dk, (bf16_t *)dv);
     return hipSuccess;
+    }
 }
 
 #define GS_SWITCH(FN, DD, HI, ...)                                    \
