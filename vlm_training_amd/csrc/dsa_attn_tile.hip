@@ -784,8 +784,10 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
         qB[ks] = row_ok ? load_bf16x8(q + off) : zero_bf16x8();
         doB[ks] = row_ok ? load_bf16x8(dout + off) : zero_bf16x8();
     }
-    const float lse2 = lse[(int64_t)hq * T + t] * LOG2E_F;
-    const float dlt = delta[(int64_t)hq * T + t];
+    // the two accumulators of a tile start from -lse/scale and -delta of the lane's row, so that S - lse/scale and
+    // dP - delta come out of the MFMAs (one multiply per element instead of a multiply-add and a subtraction)
+    const float neg_lse = -lse[(int64_t)hq * T + t] / scale;
+    const float neg_dlt = -delta[(int64_t)hq * T + t];
     const int ntiles = (causal ? min(qc0 + QBW - 1, L - 1) : L - 1) / 32 + 1;
     const int klim = causal ? qcol : L - 1;             // last key column this row may attend (dense mode)
     const uint32_t *wrow = bitmap + (int64_t)t * ldw;
@@ -810,7 +812,8 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
         if (HAS_IDX) word_next = wrow[min((TILE) + 1, ntiles - 1)];                                \
         if (!HAS_IDX) word = row_ok ? causal_bits(klim - kc0) : 0u;                                \
         word >>= 4 * h;                                                                            \
-        f32x16 sacc = zero16(), pacc = zero16();                                                   \
+        f32x16 sacc, pacc;                                                                         \
+        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) { sacc[vi] = neg_lse; pacc[vi] = neg_dlt; } \
         _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
             sacc = mfma32(lo.rowop(kt, ks), qB[ks], sacc);                              \
             pacc = mfma32(lo.rowop(vt, ks), doB[ks], pacc);                             \
@@ -818,9 +821,9 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
         sched_reads_ahead<2 * KS, 4, 1>();                                                         \
         float ds[16];                                                                              \
         _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
-            const float x = keep_or_neginf(fmaf(sacc[vi], scale_log2, -lse2),                      \
+            const float x = keep_or_neginf(sacc[vi] * scale_log2,                                  \
                                            bit_mask(word, 8 * (vi >> 2) + (vi & 3)));              \
-            ds[vi] = fast_exp2(x) * (pacc[vi] - dlt);                                              \
+            ds[vi] = fast_exp2(x) * pacc[vi];                                                      \
         }                                                                                          \
         const bf16x8 dB0 = pack8(ds), dB1 = pack8(ds + 8);                                         \
         _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
