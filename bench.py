@@ -303,7 +303,8 @@ def main():
     kern = {   # algorithmic flop per launch of the three attention kernels (selected pairs only)
         "attn_fwd": ("dsa_tile_fwd_kernel", 4 * unit),          # QK^T + PV
         "bwd_dq": ("dsa_tile_dq_kernel", 6 * unit),             # QK^T + dO V^T + dS K
-        "bwd_dkv": ("dsa_tile_dkvpc_kernel", 8 * unit),         # QK^T + dO V^T + P^T dO + dS^T Q
+        # QK^T + dO V^T + P^T dO + dS^T Q (head_dim 256 runs the producer/consumer form, twice)
+        "bwd_dkv": ("dsa_tile_dkv2_kernel" if w.D <= 128 else "dsa_tile_dkvpc_kernel", 8 * unit),
     }
     dom = max(kern, key=lambda name: stage_ms[name])
     dom_kernel, dom_flop = kern[dom]
