@@ -34,8 +34,9 @@ def test_workspace_sizes_without_a_gpu():
     b4 = lib.dsa_index_topk_workspace_bytes(131072, 131072, 2048)
     assert b4 == 2048 * 131072 * 4                         # chunked: 1 GiB of score rows at a time
     up = lambda x: (x + 255) // 256 * 256                  # both parts are 256-byte aligned
-    assert lib.dsa_attn_bwd_workspace_bytes(1000, 8, 640, 0) == up(1000 * 8 * 4)
-    assert lib.dsa_attn_bwd_workspace_bytes(1000, 8, 640, 1) == up(1000 * 8 * 4) + up(1000 * 20 * 4)
+    order = up(((1000 // 128 + 4096 + 1) * 2 + 2) * 4)   # launch order of the key tiles: (segment, tile) pairs and a count
+    assert lib.dsa_attn_bwd_workspace_bytes(1000, 8, 640, 0) == up(1000 * 8 * 4) + order
+    assert lib.dsa_attn_bwd_workspace_bytes(1000, 8, 640, 1) == up(1000 * 8 * 4) + up(1000 * 20 * 4) + order
     assert lib.dsa_attn_fwd_workspace_bytes(1000, 640, 1) == up(1000 * 20 * 4)
     assert lib.dsa_attn_bwd_bitmap_offset(1000, 8) == up(1000 * 8 * 4)   # forward workspace fits behind it
     assert lib.dsa_attn_fwd_workspace_bytes(1000, 640, 0) == 0

@@ -186,6 +186,35 @@ def test_sparse_path_odd_head_groups(Hq, Hkv, D):
         ops.set_tile_crossover(old)
 
 
+@pytest.mark.parametrize("n_short", [300, 4500])
+def test_many_segments_in_every_launch_order_of_the_key_tiles(n_short):
+    """dK/dV lists its key tiles longest walk first; 300 segments go through the order table, 4500 are more than
+    it holds (plain order).  Lengths 0-3 with two long segments between them."""
+    _log(f"many segments {n_short}")
+    g = torch.Generator().manual_seed(23 + n_short)
+    lens = torch.randint(0, 4, (n_short,), generator=g).tolist()
+    lens[n_short // 3] = 333
+    lens[2 * n_short // 3] = 130
+    cu = [0]
+    for L in lens:
+        cu.append(cu[-1] + L)
+    T, Hq, Hkv, D = cu[-1], 4, 2, 64
+    q = (torch.randn(T, Hq, D, generator=g) * 0.7).bfloat16()
+    k = (torch.randn(T, Hkv, D, generator=g) * 0.7).bfloat16()
+    v = (torch.randn(T, Hkv, D, generator=g) * 0.7).bfloat16()
+    do = torch.randn(T, Hq, D, generator=g).bfloat16()
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    out = ops.dsa_varlen_attn(qd, kd, vd, torch.tensor(cu, dtype=torch.int32, device=DEV), 333)
+    out.backward(do.to(DEV))
+    qr, kr, vr = (x.float().requires_grad_(True) for x in (q, k, v))
+    ref = R.dense_varlen_causal(qr, kr, vr, cu)
+    ref.backward(do.float())
+    assert_close_bf16(out, ref, "out")
+    assert_close_bf16(qd.grad, qr.grad, "dq")
+    assert_close_bf16(kd.grad, kr.grad, "dk")
+    assert_close_bf16(vd.grad, vr.grad, "dv")
+
+
 @pytest.mark.parametrize("D,Hq,Hkv,segs,K,sparse", [
     (64, 16, 1, (128, 64), 4, True),                       # sixteen heads and a few hundred queries on the same four keys
     (256, 16, 2, (716, 65, 73, 512, 300), 4, True),        # the head geometry of C5 (group of 8, head_dim 256)

@@ -845,6 +845,146 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
 }
 
 // ==================================================================================================
+// Launch order of the key-stationary workgroups.  A key tile's walk is as long as the part of its segment
+// behind it, and the hardware starts workgroups in grid order: handed out segment by segment, the long
+// walks of a late long segment start late and the launch ends on them.  This kernel (one workgroup) lists
+// the 128-key tiles of all segments longest walk first - `by_segment` = 0: by the number of tiles behind
+// them, across segments (best balance; for launches of a few rounds of workgroups), `by_segment` = 1: the
+// segments by length, each one's tiles together (workgroups that run side by side then walk the same q / dO
+// rows and share them in L2, which is worth more than the balance once a launch runs for many rounds):
+//   order[0] = number of tiles (or -1: too many segments or tiles for the table, use the plain order),
+//   order[2 + 2 s], order[3 + 2 s] = segment and tile of slot s.
+// The order changes the schedule only; every tile is still reduced by one workgroup in a fixed order.
+// ==================================================================================================
+#define DSA_ORDER_MAX_SEGS 4096
+#define DSA_ORDER_MAX_TILES 8192                         // tiles of the longest segment
+static_assert(DSA_ORDER_MAX_TILES + 1 >= 2 * DSA_ORDER_MAX_SEGS, "the rank tables of the by-segment order share cnt[]");
+__global__ __launch_bounds__(1024) void dsa_tile_order_kernel(const int32_t *__restrict__ cu, int N, int cap, int by_segment,
+                                                              int32_t *__restrict__ order) {
+    __shared__ int nt[DSA_ORDER_MAX_SEGS];               // tiles per segment
+    __shared__ int cnt[DSA_ORDER_MAX_TILES + 1];         // cnt[r]: segments with at least r tiles; then: slots before rank r
+    __shared__ int part[1024];
+    __shared__ int maxnt_s;
+    const int tid = threadIdx.x;
+    if (N > DSA_ORDER_MAX_SEGS) {
+        if (tid == 0) order[0] = -1;
+        return;
+    }
+    if (tid == 0) maxnt_s = 0;
+    __syncthreads();
+    int mx = 0;
+    for (int i = tid; i < N; i += 1024) {
+        const int L = cu[i + 1] - cu[i];
+        nt[i] = L > 0 ? (L + 127) / 128 : 0;
+        mx = max(mx, nt[i]);
+    }
+    atomicMax(&maxnt_s, mx);
+    __syncthreads();
+    const int maxnt = maxnt_s;
+    if (maxnt > DSA_ORDER_MAX_TILES) {
+        if (tid == 0) order[0] = -1;
+        return;
+    }
+    if (by_segment) {
+        // rank of a segment = segments that are longer, or as long and earlier; cnt[rank] = segment, then its first slot
+        int *seg_of = cnt, *first = cnt + DSA_ORDER_MAX_SEGS;     // (both fit: DSA_ORDER_MAX_TILES + 1 >= 2 * DSA_ORDER_MAX_SEGS)
+        for (int i = tid; i < N; i += 1024) {
+            int rk = 0;
+            for (int o = 0; o < N; ++o) rk += nt[o] > nt[i] || (nt[o] == nt[i] && o < i);
+            seg_of[rk] = i;
+        }
+        __syncthreads();
+        if (tid == 0) {                                  // N <= 4096 additions
+            int run = 0;
+            for (int rk = 0; rk < N; ++rk) {
+                first[rk] = run;
+                run += nt[seg_of[rk]];
+            }
+            maxnt_s = run;
+        }
+        __syncthreads();
+        const int total = maxnt_s;
+        if (total > cap) {
+            if (tid == 0) order[0] = -1;
+            return;
+        }
+        if (tid == 0) order[0] = total;
+        for (int rk = 0; rk < N; ++rk) {
+            const int seg = seg_of[rk], f = first[rk];
+            for (int j = tid; j < nt[seg]; j += 1024) {
+                order[2 + 2 * (f + j)] = seg;
+                order[3 + 2 * (f + j)] = j;
+            }
+        }
+        return;
+    }
+    for (int r = 1 + tid; r <= maxnt; r += 1024) {
+        int c = 0;
+        for (int i = 0; i < N; ++i) c += nt[i] >= r;
+        cnt[r] = c;
+    }
+    __syncthreads();
+    // slots before rank r = sum of cnt[r'] over r' > r: ranks are cut into 1024 runs (run t = the ranks
+    // maxnt - t per .. downwards), a scan over the runs' sums, then each thread finishes its run
+    const int per = (maxnt + 1023) / 1024;
+    int sum = 0;
+    for (int u = 0; u < per; ++u) {
+        const int r = maxnt - (tid * per + u);
+        if (r >= 1) sum += cnt[r];
+    }
+    part[tid] = sum;
+    __syncthreads();
+    for (int d = 1; d < 1024; d <<= 1) {
+        const int add = tid >= d ? part[tid - d] : 0;
+        __syncthreads();
+        part[tid] += add;
+        __syncthreads();
+    }
+    int before = part[tid] - sum;                        // slots of the runs with larger ranks
+    const int total = part[1023];
+    __syncthreads();
+    for (int u = 0; u < per; ++u) {
+        const int r = maxnt - (tid * per + u);
+        if (r >= 1) {
+            const int c = cnt[r];
+            cnt[r] = before;
+            before += c;
+        }
+    }
+    __syncthreads();
+    if (total > cap) {
+        if (tid == 0) order[0] = -1;
+        return;
+    }
+    if (tid == 0) order[0] = total;
+    for (int r = 1 + tid; r <= maxnt; r += 1024) {
+        int slot = cnt[r];
+        for (int i = 0; i < N; ++i)
+            if (nt[i] >= r) {
+                order[2 + 2 * slot] = i;
+                order[3 + 2 * slot] = nt[i] - r;
+                ++slot;
+            }
+    }
+}
+extern "C" size_t dsa_tile_order_bytes(int T) { return ((size_t)(T / 128 + DSA_ORDER_MAX_SEGS + 1) * 2 + 2) * sizeof(int32_t); }
+// the tile of workgroup slot `slot`: from the order table when there is one, else segment by segment
+__device__ __forceinline__ bool locate_key_tile(const int32_t *order, const int32_t *cu, int N, int slot, int &s0, int &L, int &blk) {
+    if (order) {
+        const int total = order[0];
+        if (total >= 0) {
+            if (slot >= total) return false;
+            const int seg = min(max(order[2 + 2 * slot], 0), N - 1);
+            blk = order[3 + 2 * slot];
+            s0 = cu[seg];
+            L = cu[seg + 1] - s0;
+            return blk >= 0;
+        }
+    }
+    return locate_block(cu, N, slot, 128, false, s0, L, blk);
+}
+
+// ==================================================================================================
 // dK, dV, producer/consumer form, key-stationary ("scatter by key": every key row is reduced by exactly
 // one wave, in a fixed query order, so the result needs no atomics and is bit-reproducible).  A
 // workgroup owns a 128-key tile (4 groups of 32 keys) of one segment and kv head and walks the later
@@ -874,7 +1014,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
-    float scale, int causal, int dhalf, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    float scale, int causal, int dhalf, const int32_t *__restrict__ order, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>();
     // head_dim 256: a consumer's accumulators cover one half of head_dim per launch (`dhalf`), the
     // q/dO ring holds three blocks instead of four and the producers run GEMMs and softmax of one block
@@ -907,7 +1047,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     const int G = Hq / Hkv;
     const int kvh = blockIdx.x % Hkv;
     int s0, L, blk;
-    if (!locate_block(cu, N, blockIdx.x / Hkv, 128, false, s0, L, blk)) return;
+    if (!locate_key_tile(order, cu, N, blockIdx.x / Hkv, s0, L, blk)) return;
     if (HAS_IDX) L = min(L, ldw * 32);                  // a bitmap row has ldw words whatever the caller's max_seqlen
     if (blk * 128 >= L) return;                         // (whole workgroup, before its first barrier)
     const int c0 = blk * 128, kc = c0 + kg * 32;
@@ -1305,7 +1445,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
     const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
-    float scale, int causal, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    float scale, int causal, const int32_t *__restrict__ order, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
     static_assert(D <= 128, "head_dim 256 runs dsa_tile_dkvpc_kernel");
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>();
     constexpr int NCHUNK = 32 * CPR, STG = 256, CPT = NCHUNK / STG;
@@ -1327,7 +1467,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
     const int G = Hq / Hkv;
     const int kvh = blockIdx.x % Hkv;
     int s0, L, blk;
-    if (!locate_block(cu, N, blockIdx.x / Hkv, 128, false, s0, L, blk)) return;
+    if (!locate_key_tile(order, cu, N, blockIdx.x / Hkv, s0, L, blk)) return;
     if (HAS_IDX) L = min(L, ldw * 32);
     if (blk * 128 >= L) return;                         // (whole workgroup, before its first barrier)
     const int c0 = blk * 128, kc = c0 + kg * 32;
@@ -1756,7 +1896,7 @@ static hipError_t launch_dq_i(dim3 grid, hipStream_t stream, const void *dout, c
 template <int D, bool HAS_IDX, int GS>
 static hipError_t launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
                          const float *lse, const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N,
-                         int T, int Hq, int Hkv, float scale, int causal, void *dk, void *dv) {
+                         int T, int Hq, int Hkv, float scale, int causal, const int32_t *order, void *dk, void *dv) {
     // LDS above 64 KiB has to be requested per kernel and device; asked for on every launch (a host-side table
     // lookup), so that neither a second device nor a second thread can meet a kernel that was never configured
     if constexpr (D <= 128) {
@@ -1765,7 +1905,7 @@ static hipError_t launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, 
         if (e2 != hipSuccess) return e2;
         hipLaunchKernelGGL((dsa_tile_dkv2_kernel<D, HAS_IDX, GS>), grid, dim3(512), dkv2_lds_bytes<D>(), stream,
                            (const bf16_t *)dout, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap,
-                           ldw, cu, N, T, Hq, Hkv, scale, causal, (bf16_t *)dk, (bf16_t *)dv);
+                           ldw, cu, N, T, Hq, Hkv, scale, causal, order, (bf16_t *)dk, (bf16_t *)dv);
         return hipSuccess;
     } else {
     const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(&dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>),
@@ -1775,7 +1915,7 @@ static hipError_t launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, 
     for (int dhalf = 0; dhalf < (D > 128 ? 2 : 1); ++dhalf)
         hipLaunchKernelGGL((dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>), grid, dim3(512), dkvpc_lds_bytes<D>(), stream,
                            (const bf16_t *)dout, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap,
-                           ldw, cu, N, T, Hq, Hkv, scale, causal, dhalf, (bf16_t *)dk, (bf16_t *)dv);
+                           ldw, cu, N, T, Hq, Hkv, scale, causal, dhalf, order, (bf16_t *)dk, (bf16_t *)dv);
     return hipSuccess;
     }
 }
@@ -1876,9 +2016,15 @@ extern "C" hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const 
 extern "C" hipError_t dsa_launch_tile_dkv(const void *dout, const void *q, const void *k, const void *v,
                                           const float *lse, const float *delta, const uint32_t *bitmap, int ldw,
                                           const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale, int causal,
-                                          void *dk, void *dv, hipStream_t stream) {
+                                          int32_t *order, void *dk, void *dv, hipStream_t stream) {
     const int gs = group_shift(Hq, Hkv);
     const dim3 grid((unsigned)(((int64_t)T / 128 + N + 1) * Hkv));
-    TILE_SWITCH(launch_dkv_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, causal, dk, dv)
+    // `order` (dsa_tile_order_bytes(T) bytes, or null): the tiles are listed longest walk first before the launch
+    if (order && N > 1)
+        hipLaunchKernelGGL(dsa_tile_order_kernel, dim3(1), dim3(1024), 0, stream, cu, N, T / 128 + DSA_ORDER_MAX_SEGS + 1,
+                           grid.x > 4 * 256 ? 1 : 0, order);
+    else
+        order = nullptr;                                 // one segment: its tiles are in order already
+    TILE_SWITCH(launch_dkv_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, causal, order, dk, dv)
     return hipGetLastError();
 }
