@@ -985,29 +985,24 @@ __device__ __forceinline__ bool locate_key_tile(const int32_t *order, const int3
 }
 
 // ==================================================================================================
-// dK, dV, producer/consumer form, key-stationary ("scatter by key": every key row is reduced by exactly
-// one wave, in a fixed query order, so the result needs no atomics and is bit-reproducible).  A
-// workgroup owns a 128-key tile (4 groups of 32 keys) of one segment and kv head and walks the later
-// queries in blocks of 32 (query, head) rows, from the end of the segment down to the key tile:
-// workgroups that run side by side then read the same q / dO rows at about the same time and share
+// dK, dV for head_dim 256, producer/consumer form, key-stationary ("scatter by key": every key row is
+// reduced by exactly one wave, in a fixed query order, so the result needs no atomics and is
+// bit-reproducible).  A workgroup owns a 128-key tile (4 groups of 32 keys) of one segment and kv head and
+// walks the later queries in blocks of 32 (query, head) rows, from the end of the segment down to the key
+// tile: workgroups that run side by side then read the same q / dO rows at about the same time and share
 // them in L2.
 //   waves 0-3 (producers, one per key group): S = Q K^T and dP = dO V^T against the group's K / V rows
-//     held in registers, then P and dS = P * (dP - delta) in bf16, written to LDS in MFMA B layout.
-//     The two GEMMs of block b+1 are issued between the softmax arithmetic of block b: a SIMD overlaps
-//     matrix and vector instructions of one instruction stream far better than those of two waves.
+//     held in registers (128 of them), then P and dS = P * (dP - delta) in bf16, written to LDS in MFMA B
+//     layout.
 //   waves 4-7 (consumers, one per key group): dV^T += dO^T P and dK^T += Q^T dS for block b-1,
 //     A operands read transposed from the staged q / dO block, B operands read back from LDS.  They
-//     also do all the staging (global -> registers two blocks ahead -> LDS), so the producers' stream
-//     holds nothing but the GEMMs and the softmax.
-// Nothing is computed twice (32 MFMAs per 32x32 block pair), each wave stays under 256 registers.
-// LDS (dynamic, ~131 KiB): q/dO blocks in a ring of four (b+2 being staged, b+1 read row-wise by the
-// producers, b-1 read transposed by the consumers), P/dS (and, for blocks of large probabilities, the
-// bf16 rounding remainder of P) in a ring of two, row statistics and selection words in a ring of four.
-// One barrier per block.
-// head_dim 256: the K and V rows of a producer fill 128 registers and a consumer's accumulators would
-// fill 256, so the kernel is launched once per half of head_dim (`dhalf`: the consumers accumulate and
-// write that half, the producers repeat S and dP), the q/dO ring has three slots (~158 KiB) and the
-// producers run GEMMs and softmax of a block in turn.
+//     also do all the staging (global -> registers -> LDS one block ahead).
+// A consumer's accumulators for all of head_dim would fill 256 registers, so the kernel is launched once
+// per half of head_dim (`dhalf`: the consumers accumulate and write that half, the producers repeat S and
+// dP: 48 instead of 32 MFMAs per 32x32 block pair and launch).
+// LDS (dynamic, ~158 KiB): q/dO blocks in a ring of three, P/dS (and, for blocks of large probabilities,
+// the bf16 rounding remainder of P) in a ring of two, row statistics and selection words in a ring of
+// three.  One barrier per block.  (head_dim <= 128 runs dsa_tile_dkv2_kernel below.)
 // ==================================================================================================
 template <int D, bool HAS_IDX, int GSHIFT>
 __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
@@ -1015,13 +1010,10 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
     float scale, int causal, int dhalf, const int32_t *__restrict__ order, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    static_assert(D == 256, "head_dim <= 128 runs dsa_tile_dkv2_kernel");
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>();
-    // head_dim 256: a consumer's accumulators cover one half of head_dim per launch (`dhalf`), the
-    // q/dO ring holds three blocks instead of four and the producers run GEMMs and softmax of one block
-    // in turn (the ring has no room for the block a pipelined producer would read ahead)
-    constexpr bool PIPE = D <= 128;
-    constexpr int NQD = PIPE ? 4 : 3, LEAD = PIPE ? 2 : 1;
-    constexpr int DTC = DT > 4 ? 4 : DT;
+    constexpr int NQD = 3, LEAD = 1;                     // q/dO ring slots; blocks staged ahead of the producers
+    constexpr int DTC = DT / 2;                          // d-tiles of one half of head_dim
     const int dt0 = dhalf * DTC;
     constexpr int NCHUNK = 32 * CPR;                     // 16-byte chunks per staged operand
     constexpr int CPT = NCHUNK / 256;                    // chunks per consumer thread and operand
@@ -1036,7 +1028,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     unsigned char *const pd_ring = dyn_lds + NQD * QD_SLOT;          // 2 slots
     unsigned char *const aux_ring = pd_ring + 2 * PD_SLOT;           // NQD slots
     uint32_t *const split_flag = reinterpret_cast<uint32_t *>(aux_ring + NQD * AUX_SLOT);   // [P/dS slot][key group]
-    auto qslot = [](int b) { return PIPE ? (b & 3) : (b % 3); };
+    auto qslot = [](int b) { return b % 3; };
 
     const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5, j = lane & 31;
     LaneOffsets<D> lo;
@@ -1106,9 +1098,9 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
         const int64_t aux_dlast = -(int64_t)aux_stride * aux_over * 4;
         const unsigned char *ap =
             reinterpret_cast<const unsigned char *>(aux_base + (int64_t)aux_stride * (q0 + last * QB + aux_q - aux_over));
-        // two register sets: a global load has two block-times to land before its LDS store
-        u32x4 qst0[CPT], dost0[CPT], qst1[CPT], dost1[CPT];
-        uint32_t aux_st0, aux_st1;
+        // one register set (four chunks per operand and thread): a global load has one block-time to land
+        u32x4 qst0[CPT], dost0[CPT];
+        uint32_t aux_st0;
         // loads the block of step b (block last - b), called with b = 0, 1, 2, ... in turn; past step
         // `last` it reads block 0 again
         auto gload = [&](int b, u32x4 (&qst)[CPT], u32x4 (&dost)[CPT], uint32_t &aux_st) {
@@ -1129,7 +1121,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
             }
             aux_st = *reinterpret_cast<const uint32_t *>(ap);
         };
-        auto lstore = [&](int b, const u32x4 (&qst)[CPT], const u32x4 (&dost)[CPT], uint32_t aux_st) {   // step b -> ring slot b % 4
+        auto lstore = [&](int b, const u32x4 (&qst)[CPT], const u32x4 (&dost)[CPT], uint32_t aux_st) {   // step b -> ring slot b % 3
             unsigned char *slot = qd_ring + qslot(b) * QD_SLOT;
             float *lse_s = reinterpret_cast<float *>(aux_ring + qslot(b) * AUX_SLOT);
             float *dlt_s = lse_s + 32;
@@ -1154,32 +1146,14 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
                 mask_s[((ctid - 64) / QB) * 32 + (ctid - 64) % QB] =
                     (aux_mask_ok && !(b > last || (b == 0 && aux_over > 0))) ? aux_st : 0u;
         };
-        if (PIPE) {
-            gload(0, qst0, dost0, aux_st0);
-            gload(1, qst1, dost1, aux_st1);
-            lstore(0, qst0, dost0, aux_st0);
-            lstore(1, qst1, dost1, aux_st1);
-            gload(2, qst0, dost0, aux_st0);
-            gload(3, qst1, dost1, aux_st1);
-        } else {                                         // head_dim 256: one register set (four chunks per operand and thread)
-            gload(0, qst0, dost0, aux_st0);
-            lstore(0, qst0, dost0, aux_st0);
-            gload(1, qst0, dost0, aux_st0);
-        }
-        __syncthreads();                                 // the first LEAD steps staged
+        gload(0, qst0, dost0, aux_st0);
+        lstore(0, qst0, dost0, aux_st0);
+        gload(1, qst0, dost0, aux_st0);
+        __syncthreads();                                 // the first step staged
 
         f32x16 dkacc[DTC], dvacc[DTC];
 #pragma unroll
         for (int dt = 0; dt < DTC; ++dt) { dkacc[dt] = zero16(); dvacc[dt] = zero16(); }
-        // one consumer step: stage step B+LEAD from the register set that holds it, refill the set (two sets:
-        // with step B+LEAD+2, one set: with step B+LEAD+1), then the MFMAs of step B-1
-#define DKV_CONSUMER_STEP(B, QS, DS, AS)                                                            \
-    {                                                                                              \
-        lstore((B) + LEAD, QS, DS, AS); /* its slot was last read (as step B+LEAD-NQD) before the previous barrier */ \
-        gload((B) + LEAD + (PIPE ? 2 : 1), QS, DS, AS);                                            \
-        if ((B) >= 1) consume((B) - 1);                                                            \
-        __syncthreads();                                                                           \
-    }
         auto consume = [&](int b) {
             const unsigned char *qt = qd_ring + qslot(b) * QD_SLOT + dt0 * 64;
             lds_u8 *pt[4];                  // lane addresses in the q block; the dO block sits TILE_B behind
@@ -1209,17 +1183,13 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
                 }
             }
         };
-        int b = 0;
-        if (PIPE) {                                      // step b + 2 sits in set b % 2
-            for (; b + 1 <= nblocks; b += 2) {
-                DKV_CONSUMER_STEP(b, qst0, dost0, aux_st0)
-                DKV_CONSUMER_STEP(b + 1, qst1, dost1, aux_st1)
-            }
-            if (b <= nblocks) DKV_CONSUMER_STEP(b, qst0, dost0, aux_st0)
-        } else {
-            for (; b <= nblocks; ++b) DKV_CONSUMER_STEP(b, qst0, dost0, aux_st0)
+        // one consumer step: stage step b+1 from the register set, refill the set with step b+2, then the MFMAs of step b-1
+        for (int b = 0; b <= nblocks; ++b) {
+            lstore(b + LEAD, qst0, dost0, aux_st0);      // its slot was last read (as step b+1-3) before the previous barrier
+            gload(b + LEAD + 1, qst0, dost0, aux_st0);
+            if (b >= 1) consume(b - 1);
+            __syncthreads();
         }
-#undef DKV_CONSUMER_STEP
         if (key_ok) {
             bf16_t *pk = dk + krow * D + dt0 * 32, *pv_ = dv + krow * D + dt0 * 32;
 #pragma unroll
@@ -1231,54 +1201,13 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
         return;
     }
 
-    // ================= producers: S, dP of block b+1 between the softmax of block b =================
+    // ================= producers: S and dP of a block, then its softmax =================
     bf16x8 kB[KS], vB[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         kB[ks] = load_bf16x8(k + krow * D + 16 * ks + 8 * h);
         vB[ks] = load_bf16x8(v + krow * D + 16 * ks + 8 * h);
     }
-    // row statistics and selection words of a block are read from LDS one block ahead
-    f32x4 l4[4], d4[4];
-    uint32_t mw[16];
-    auto read_aux = [&](int b) {
-        const float *lse_s = reinterpret_cast<const float *>(aux_ring + qslot(b) * AUX_SLOT);
-        const float *dlt_s = lse_s + 32;
-        const uint32_t *mask_s = reinterpret_cast<const uint32_t *>(dlt_s + 32) + kg * 32;
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-            l4[g4] = *reinterpret_cast<const f32x4 *>(&lse_s[8 * g4 + 4 * h]);
-            d4[g4] = *reinterpret_cast<const f32x4 *>(&dlt_s[8 * g4 + 4 * h]);
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (HAS_IDX && (e == 0 || GSHIFT < 2)) mw[4 * g4 + e] = mask_s[(8 * g4 + 4 * h + e) >> GSHIFT];
-        }
-    };
-    auto gemms = [&](int b, f32x16 &sacc, f32x16 &pacc) {            // S and dP of block b
-        const unsigned char *qt = qd_ring + qslot(b) * QD_SLOT, *dot = qt + TILE_B;
-        sacc = zero16();
-        pacc = zero16();
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            sacc = mfma32(lo.rowop(qt, ks), kB[ks], sacc);
-            pacc = mfma32(lo.rowop(dot, ks), vB[ks], pacc);
-        }
-        sched_reads_ahead<2 * KS, 4, 1>();
-    };
-    // P and dS of element vi (C layout) of block b from its S and dP accumulators
-    auto element = [&](auto may_diag, int b, int vi, const f32x16 &sacc, const f32x16 &pacc, float sl2, uint32_t &keep,
-                       float *pv, float *dsv) {
-        const int g4 = vi >> 2, e = vi & 3, row = 8 * g4 + 4 * h + e;
-        if (e == 0 || GSHIFT < 2) {                      // rows of one query share the mask bit
-            const int qcb = q0 + (nblocks - 1 - b) * QB, qi = row >> GSHIFT;
-            uint32_t w = HAS_IDX ? mw[vi] : 0xffffffffu;
-            if (decltype(may_diag)::value && causal && qcb < kc + 32) w &= causal_bits(qcb + qi - kc);
-            keep = bit_mask(w, j);
-        }
-        const float p = fast_exp2(keep_or_neginf(fmaf(sacc[vi], sl2, -l4[g4][e]), keep));
-        pv[vi] = p;
-        dsv[vi] = p * (pacc[vi] - d4[g4][e]);
-    };
     // P and dS go to the consumers in bf16.  dV[s] = sum over (query, head) of P dO piles the rounding of P (2^-9
     // relative) onto one key row; where probabilities are large (few keys per query: short rows, small top-k) and many
     // rows meet in one key, that noise reaches several 1e-2.  A block whose largest P is at least DKV_SPLIT_MIN
@@ -1311,114 +1240,52 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
         }
         if (lane == 0) split_flag[(b & 1) * 4 + kg] = big ? 1u : 0u;
     };
-    auto softmax = [&](auto may_diag, int b, const f32x16 &sacc, const f32x16 &pacc) {
-        float pv[16], dsv[16];
-        uint32_t keep = 0u;
+    __syncthreads();                                     // the first step staged
+    // GEMMs, then softmax, block by block; the row statistics are taken from LDS group by group (the K and V rows
+    // leave no registers to hold them across the GEMMs)
+    for (int b = 0; b <= nblocks; ++b) {
+        if (b < nblocks) {
+            const unsigned char *qt = qd_ring + qslot(b) * QD_SLOT, *dot = qt + TILE_B;
+            f32x16 sacc = zero16(), pacc = zero16();
 #pragma unroll
-        for (int vi = 0; vi < 16; ++vi) element(may_diag, b, vi, sacc, pacc, scale_log2, keep, pv, dsv);
-        store_pd(b, pv, dsv);
-    };
-    // GEMMs of block b+1 into (sn, pn) with the softmax of block b from (sc, pc) between them: after
-    // every MFMA the vector work of 16 / (2 KS) elements, operand reads four MFMAs ahead.  The order
-    // is fixed by hand: every step ends in an empty asm statement that the step's results, the next
-    // MFMA's operand and the scale used by the next step's arithmetic pass through.
-    auto fused = [&](auto may_diag, int b, const f32x16 &sc, const f32x16 &pc, f32x16 &sn, f32x16 &pn) {
-        constexpr int NM = 2 * KS, EPM = 16 / NM;
-        const unsigned char *qt = qd_ring + qslot(b + 1) * QD_SLOT, *dot = qt + TILE_B;
-        float pv[16], dsv[16], sl2 = scale_log2;
-        uint32_t keep = 0u;
-        bf16x8 a[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) a[i] = lo.rowop((i & 1) ? dot : qt, i >> 1);
-        sn = zero16();
-        pn = zero16();
-#pragma unroll
-        for (int i = 0; i < NM; ++i) {
-            if (i & 1) pn = mfma32(a[i & 3], vB[i >> 1], pn);
-            else sn = mfma32(a[i & 3], kB[i >> 1], sn);
-            if (i + 4 < NM) a[i & 3] = lo.rowop((i & 1) ? dot : qt, (i + 4) >> 1);
-#pragma unroll
-            for (int u = 0; u < EPM; ++u) element(may_diag, b, i * EPM + u, sc, pc, sl2, keep, pv, dsv);
-            if (EPM == 1)
-                asm volatile("" : "+v"(sl2), "+v"(pv[i]), "+v"(dsv[i]), "+v"(a[(i + 1) & 3]) : : "memory");
-            else
-                asm volatile("" : "+v"(sl2), "+v"(pv[2 * i]), "+v"(dsv[2 * i]), "+v"(pv[2 * i + 1]), "+v"(dsv[2 * i + 1]),
-                             "+v"(a[(i + 1) & 3]) : : "memory");
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        store_pd(b, pv, dsv);
-    };
-    // one producer step
-#define DKV_PRODUCER_STEP(B, SC, PC, SN, PN, MAY_DIAG)                                              \
-    {                                                                                              \
-        if ((B) + 1 < nblocks) fused(MAY_DIAG, B, SC, PC, SN, PN);                                 \
-        else if ((B) < nblocks) softmax(MAY_DIAG, B, SC, PC);                                      \
-        if ((B) + 1 < nblocks) read_aux((B) + 1);                                                  \
-        __syncthreads();                                                                           \
-    }
-    f32x16 s_a, p_a, s_b, p_b;
-    __syncthreads();                                     // the first LEAD steps staged
-    const std::true_type diag_y;
-    const std::false_type diag_n;
-    if (!PIPE) {
-        // GEMMs, then softmax, block by block (the row statistics of a block are staged one step before)
-        for (int b = 0; b <= nblocks; ++b) {
-            if (b < nblocks) {
-                gemms(b, s_a, p_a);
-                // softmax with the row statistics taken from LDS group by group (K and V rows of head_dim 256
-                // leave no registers to hold them across the GEMMs)
-                const float *lse_s = reinterpret_cast<const float *>(aux_ring + qslot(b) * AUX_SLOT);
-                const float *dlt_s = lse_s + 32;
-                const uint32_t *mask_s = reinterpret_cast<const uint32_t *>(dlt_s + 32) + kg * 32;
-                const int qcb = q0 + (nblocks - 1 - b) * QB;
-                const bool diag = causal && qcb < kc + 32;
-                float pv[16], dsv[16];
-#pragma unroll
-                for (int g4 = 0; g4 < 4; ++g4) {
-                    const f32x4 l4g = *reinterpret_cast<const f32x4 *>(&lse_s[8 * g4 + 4 * h]);
-                    const f32x4 d4g = *reinterpret_cast<const f32x4 *>(&dlt_s[8 * g4 + 4 * h]);
-                    uint32_t keep = 0u;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int vi = 4 * g4 + e, row = 8 * g4 + 4 * h + e;
-                        if (e == 0 || GSHIFT < 2) {
-                            const int qi = row >> GSHIFT;
-                            uint32_t w = HAS_IDX ? mask_s[qi] : 0xffffffffu;
-                            if (diag) w &= causal_bits(qcb + qi - kc);
-                            keep = bit_mask(w, j);
-                        }
-                        const float p = fast_exp2(keep_or_neginf(fmaf(s_a[vi], scale_log2, -l4g[e]), keep));
-                        pv[vi] = p;
-                        dsv[vi] = p * (p_a[vi] - d4g[e]);
-                    }
-                }
-                store_pd(b, pv, dsv);
+            for (int ks = 0; ks < KS; ++ks) {
+                sacc = mfma32(lo.rowop(qt, ks), kB[ks], sacc);
+                pacc = mfma32(lo.rowop(dot, ks), vB[ks], pacc);
             }
-            __syncthreads();
+            sched_reads_ahead<2 * KS, 4, 1>();
+            const float *lse_s = reinterpret_cast<const float *>(aux_ring + qslot(b) * AUX_SLOT);
+            const float *dlt_s = lse_s + 32;
+            const uint32_t *mask_s = reinterpret_cast<const uint32_t *>(dlt_s + 32) + kg * 32;
+            const int qcb = q0 + (nblocks - 1 - b) * QB;
+            const bool diag = causal && qcb < kc + 32;
+            float pv[16], dsv[16];
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const f32x4 l4g = *reinterpret_cast<const f32x4 *>(&lse_s[8 * g4 + 4 * h]);
+                const f32x4 d4g = *reinterpret_cast<const f32x4 *>(&dlt_s[8 * g4 + 4 * h]);
+                uint32_t keep = 0u;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int vi = 4 * g4 + e, row = 8 * g4 + 4 * h + e;
+                    if (e == 0 || GSHIFT < 2) {          // rows of one query share the mask bit
+                        const int qi = row >> GSHIFT;
+                        uint32_t w = HAS_IDX ? mask_s[qi] : 0xffffffffu;
+                        if (diag) w &= causal_bits(qcb + qi - kc);
+                        keep = bit_mask(w, j);
+                    }
+                    const float p = fast_exp2(keep_or_neginf(fmaf(sacc[vi], scale_log2, -l4g[e]), keep));
+                    pv[vi] = p;
+                    dsv[vi] = p * (pacc[vi] - d4g[e]);
+                }
+            }
+            store_pd(b, pv, dsv);
         }
-        return;
+        __syncthreads();
     }
-    gemms(0, s_a, p_a);
-    read_aux(0);
-    // The blocks that can touch the causal diagonal come last; the steady loop before them has no mask
-    // arithmetic besides the selection bits and is one basic block.
-    const int nb_diag = causal ? (kc + 32 - q0 + QB - 1) / QB : 0;
-    const int steady = max(nblocks - nb_diag, 0) & ~1;   // steps [0, steady) see blocks fully past the diagonal
-    int b = 0;
-    for (; b < steady; b += 2) {
-        DKV_PRODUCER_STEP(b, s_a, p_a, s_b, p_b, diag_n)
-        DKV_PRODUCER_STEP(b + 1, s_b, p_b, s_a, p_a, diag_n)
-    }
-    for (; b + 1 <= nblocks; b += 2) {
-        DKV_PRODUCER_STEP(b, s_a, p_a, s_b, p_b, diag_y)
-        DKV_PRODUCER_STEP(b + 1, s_b, p_b, s_a, p_a, diag_y)
-    }
-    if (b <= nblocks) DKV_PRODUCER_STEP(b, s_a, p_a, s_b, p_b, diag_y)
-#undef DKV_PRODUCER_STEP
 }
 template <int D>
-constexpr size_t dkvpc_lds_bytes() {
-    return (D <= 128 ? 4 : 3) * ((size_t)2 * tile_bytes<D>() + (32 + 32 + 4 * 32) * 4) + 2 * (4 * 6 * 1024) + 2 * 4 * 4;
+constexpr size_t dkvpc_lds_bytes() {   // three q/dO and row-data slots, two P/dS slots, the split flags
+    return 3 * ((size_t)2 * tile_bytes<D>() + (32 + 32 + 4 * 32) * 4) + 2 * (4 * 6 * 1024) + 2 * 4 * 4;
 }
 
 // ==================================================================================================
@@ -1912,7 +1779,7 @@ static hipError_t launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, 
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkvpc_lds_bytes<D>());
     if (ea != hipSuccess) return ea;
     // head_dim 256: one launch per half of head_dim (a consumer wave holds 128 accumulator registers)
-    for (int dhalf = 0; dhalf < (D > 128 ? 2 : 1); ++dhalf)
+    for (int dhalf = 0; dhalf < 2; ++dhalf)
         hipLaunchKernelGGL((dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>), grid, dim3(512), dkvpc_lds_bytes<D>(), stream,
                            (const bf16_t *)dout, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap,
                            ldw, cu, N, T, Hq, Hkv, scale, causal, dhalf, order, (bf16_t *)dk, (bf16_t *)dv);
