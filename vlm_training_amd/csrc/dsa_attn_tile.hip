@@ -997,9 +997,9 @@ __device__ __forceinline__ bool locate_key_tile(const int32_t *order, const int3
 //   waves 4-7 (consumers, one per key group): dV^T += dO^T P and dK^T += Q^T dS for block b-1,
 //     A operands read transposed from the staged q / dO block, B operands read back from LDS.  They
 //     also do all the staging (global -> registers -> LDS one block ahead).
-// A consumer's accumulators for all of head_dim would fill 256 registers, so the kernel is launched once
-// per half of head_dim (`dhalf`: the consumers accumulate and write that half, the producers repeat S and
-// dP: 48 instead of 32 MFMAs per 32x32 block pair and launch).
+// A consumer's accumulators for all of head_dim would fill 256 registers, so a workgroup covers one half
+// of head_dim (`dhalf`, the low bit of its index: the consumers accumulate and write that half, the producers
+// repeat S and dP: 48 instead of 32 MFMAs per 32x32 block pair and half).
 // LDS (dynamic, ~158 KiB): q/dO blocks in a ring of three, P/dS (and, for blocks of large probabilities,
 // the bf16 rounding remainder of P) in a ring of two, row statistics and selection words in a ring of
 // three.  One barrier per block.  (head_dim <= 128 runs dsa_tile_dkv2_kernel below.)
@@ -1009,11 +1009,13 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
-    float scale, int causal, int dhalf, const int32_t *__restrict__ order, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    float scale, int causal, const int32_t *__restrict__ order, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
     static_assert(D == 256, "head_dim <= 128 runs dsa_tile_dkv2_kernel");
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>();
     constexpr int NQD = 3, LEAD = 1;                     // q/dO ring slots; blocks staged ahead of the producers
     constexpr int DTC = DT / 2;                          // d-tiles of one half of head_dim
+    // the two halves of head_dim are neighbours in the grid, so that the longest walks of both start in the first round
+    const int dhalf = blockIdx.x & 1, bx = blockIdx.x >> 1;
     const int dt0 = dhalf * DTC;
     constexpr int NCHUNK = 32 * CPR;                     // 16-byte chunks per staged operand
     constexpr int CPT = NCHUNK / 256;                    // chunks per consumer thread and operand
@@ -1037,9 +1039,9 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     const int kg = wv & 3;
     const bool consumer = wv >= 4;
     const int G = Hq / Hkv;
-    const int kvh = blockIdx.x % Hkv;
+    const int kvh = bx % Hkv;
     int s0, L, blk;
-    if (!locate_key_tile(order, cu, N, blockIdx.x / Hkv, s0, L, blk)) return;
+    if (!locate_key_tile(order, cu, N, bx / Hkv, s0, L, blk)) return;
     if (HAS_IDX) L = min(L, ldw * 32);                  // a bitmap row has ldw words whatever the caller's max_seqlen
     if (blk * 128 >= L) return;                         // (whole workgroup, before its first barrier)
     const int c0 = blk * 128, kc = c0 + kg * 32;
@@ -1778,11 +1780,10 @@ static hipError_t launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, 
     const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(&dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkvpc_lds_bytes<D>());
     if (ea != hipSuccess) return ea;
-    // head_dim 256: one launch per half of head_dim (a consumer wave holds 128 accumulator registers)
-    for (int dhalf = 0; dhalf < 2; ++dhalf)
-        hipLaunchKernelGGL((dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>), grid, dim3(512), dkvpc_lds_bytes<D>(), stream,
-                           (const bf16_t *)dout, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap,
-                           ldw, cu, N, T, Hq, Hkv, scale, causal, dhalf, order, (bf16_t *)dk, (bf16_t *)dv);
+    // two workgroups per key tile and kv head, one per half of head_dim (a consumer wave holds 128 accumulator registers)
+    hipLaunchKernelGGL((dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>), dim3(grid.x * 2), dim3(512), dkvpc_lds_bytes<D>(), stream,
+                       (const bf16_t *)dout, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap,
+                       ldw, cu, N, T, Hq, Hkv, scale, causal, order, (bf16_t *)dk, (bf16_t *)dv);
     return hipSuccess;
     }
 }
