@@ -971,13 +971,14 @@ extern "C" size_t dsa_tile_order_bytes(int T) { return ((size_t)(T / 128 + DSA_O
 // the tile of workgroup slot `slot`: from the order table when there is one, else segment by segment
 __device__ __forceinline__ bool locate_key_tile(const int32_t *order, const int32_t *cu, int N, int slot, int &s0, int &L, int &blk) {
     if (order) {
-        const int total = order[0];
+        const int total = __builtin_amdgcn_readfirstlane(order[0]);
         if (total >= 0) {
             if (slot >= total) return false;
-            const int seg = min(max(order[2 + 2 * slot], 0), N - 1);
-            blk = order[3 + 2 * slot];
-            s0 = cu[seg];
-            L = cu[seg + 1] - s0;
+            // (every lane reads the same words; the lane reads tell the compiler that the results are wave-uniform)
+            const int seg = min(max(__builtin_amdgcn_readfirstlane(order[2 + 2 * slot]), 0), N - 1);
+            blk = __builtin_amdgcn_readfirstlane(order[3 + 2 * slot]);
+            s0 = __builtin_amdgcn_readfirstlane(cu[seg]);
+            L = __builtin_amdgcn_readfirstlane(cu[seg + 1]) - s0;
             return blk >= 0;
         }
     }
