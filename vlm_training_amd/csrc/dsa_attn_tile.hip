@@ -820,10 +820,15 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
         }                                                                                          \
         sched_reads_ahead<2 * KS, 4, 1>();                                                         \
         float ds[16];                                                                              \
-        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
-            const float x = keep_or_neginf(sacc[vi] * scale_log2,                                  \
-                                           bit_mask(word, 8 * (vi >> 2) + (vi & 3)));              \
-            ds[vi] = fast_exp2(x) * pacc[vi];                                                      \
+        /* tiles in which every live row keeps all 32 keys skip the mask arithmetic */             \
+        if (__builtin_amdgcn_ballot_w64(row_ok && (word & 0x0f0f0f0fu) != 0x0f0f0f0fu) == 0ull) {     \
+            _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) ds[vi] = fast_exp2(sacc[vi] * scale_log2) * pacc[vi]; \
+        } else {                                                                                   \
+            _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                    \
+                const float x = keep_or_neginf(sacc[vi] * scale_log2,                              \
+                                               bit_mask(word, 8 * (vi >> 2) + (vi & 3)));          \
+                ds[vi] = fast_exp2(x) * pacc[vi];                                                  \
+            }                                                                                      \
         }                                                                                          \
         const bf16x8 dB0 = pack8(ds), dB1 = pack8(ds + 8);                                         \
         _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
