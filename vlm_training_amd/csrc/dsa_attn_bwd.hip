@@ -6,9 +6,9 @@
 //                                                         for the rows where the selection is sparse
 //                                                         (dsa_bwd_dq_kernel; dense rows: dsa_tile_dq_kernel)
 //   inverted selection: bitmap[t][w] bit b <=> query t selected key column 32w+b of its segment
-//                                                         (dsa_bitmap_kernel); the key-side pass
-//                                                         dsa_tile_dkv_kernel reduces every key row from it
-//                                                         without atomics.
+//                                                         (dsa_bitmap_kernel); the key-side passes
+//                                                         dsa_tile_dkv2_kernel / dsa_tile_dkvpc_kernel reduce
+//                                                         every key row from it without atomics.
 #include "dsa_common.h"
 
 // ------------------------------------------------------------------------------------------------
