@@ -315,6 +315,17 @@ def main():
         "attn_bwd": max(wk["F4"] / (PEAK_MFMA_BF16_TFLOPS * 1e12), wk["B4"] / (PEAK_HBM_GBS * 1e9)) * 1e3,
     }
     roof_total = sum(t_roof_ms.values())
+    # per stage: measured time against the stage's nominal roofline (the larger of flop / MFMA peak and bytes / HBM
+    # peak, the bytes being those a row gather of the selected keys would move) and against its flop alone
+    stage_time = {"index_topk": stage_ms["index_topk"], "attn_fwd": stage_ms["attn_fwd"],
+                  "attn_bwd": stage_ms["bwd_delta"] + stage_ms["bwd_bitmap"] + stage_ms["bwd_dq"] + stage_ms["bwd_dkv"]}
+    stage_work = {"index_topk": (wk["F1"], wk["B2"]), "attn_fwd": (wk["F3"], wk["B3"]), "attn_bwd": (wk["F4"], wk["B4"])}
+    stage_roofline = {}
+    for name, (flop, nbytes) in stage_work.items():
+        t_mfma, t_hbm = flop / (PEAK_MFMA_BF16_TFLOPS * 1e12) * 1e3, nbytes / (PEAK_HBM_GBS * 1e9) * 1e3
+        stage_roofline[name] = {"ms": stage_time[name], "flop": flop, "bytes": nbytes, "t_mfma_ms": t_mfma, "t_hbm_ms": t_hbm,
+                                "bound": "mfma" if t_mfma >= t_hbm else "hbm", "frac_nominal": max(t_mfma, t_hbm) / stage_time[name],
+                                "frac_mfma": t_mfma / stage_time[name]}
     compute_bound_ms = (wk["F1"] + 3.5 * wk["F3"]) / (PEAK_MFMA_BF16_TFLOPS * 1e12) * 1e3
     traffic = None      # HBM bytes per launch as last measured with rocprofv3 --pmc (separate runs)
     try:
@@ -336,7 +347,7 @@ def main():
         "stage_ms": stage_ms,
         "ms_per_step_median": pct(0.5), "ms_per_step_p10": pct(0.1), "ms_per_step_p90": pct(0.9),
         "roofline_whole_op": {"compute_only_bound_ms": compute_bound_ms, "frac_compute_only": compute_bound_ms / ms_per_step,
-                              "nominal_gather_roofline_ms": roof_total, "nominal_t_roof_ms": t_roof_ms,
+                              "nominal_gather_roofline_ms": roof_total, "nominal_t_roof_ms": t_roof_ms, "stages": stage_roofline,
                               "note": "compute_only_bound = (F1 + 3.5*F3) / bf16 MFMA peak: selected-pair flop of indexer, "
                                       "forward and backward, the ceiling that applies to the tile kernels; the nominal figure "
                                       "prices the attention stages by the bytes a row gather of the selected keys would move, "
