@@ -228,6 +228,9 @@ def main():
     ap.add_argument("--crossover", type=int, default=None,
                     help="tile/gather split (rows with pos < top_k * crossover run on the tile kernels; 0 = gather kernels only)")
     ap.add_argument("--only-step", action="store_true", help="the timed steps and the roofline line only (for profiler runs)")
+    ap.add_argument("--head-shard", type=int, default=1,
+                    help="measure one GPU's share of the workload with the attention heads split this many ways (the "
+                         "reference's tensor parallelism); implies --only-step")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy (a known-size kernel to scale rocprof's FETCH_SIZE/WRITE_SIZE by)")
     args = ap.parse_args()
@@ -238,6 +241,9 @@ def main():
 
     from vlm_training_amd import ops, workloads as W
     w = W.WORKLOADS[args.workload]
+    if args.head_shard > 1:
+        w = W.head_shard(w, args.head_shard)
+        args.only_step = True
     if args.crossover is not None:
         ops.set_tile_crossover(args.crossover)
     dev = torch.device("cuda:0")
@@ -329,6 +335,8 @@ def main():
     compute_bound_ms = (wk["F1"] + 3.5 * wk["F3"]) / (PEAK_MFMA_BF16_TFLOPS * 1e12) * 1e3
     traffic = None      # HBM bytes per launch as last measured with rocprofv3 --pmc (separate runs)
     try:
+        if args.head_shard > 1:
+            raise OSError("no counter run for head shards")
         with open(os.path.join(ROOT, "profiles", f"hbm_traffic_{args.workload}.json")) as fh:
             traffic = json.load(fh).get(dom_kernel)
     except OSError:

@@ -159,8 +159,9 @@ size_t dsa_attn_mass_workspace_bytes(int T, int Hkv, int K, int max_seqlen);
 int dsa_set_tile_crossover(int crossover);
 int dsa_get_tile_crossover(void);
 
-/* Bytes of workspace dsa_attn_bwd needs (softmax row terms, the inverted selection bitmap, and the launch order of
- * the dK/dV key tiles: a few KiB + T/16 bytes). */
+/* Bytes of workspace dsa_attn_bwd needs: softmax row terms, the inverted selection bitmap, the launch order of the
+ * dK/dV key tiles (about 128 KiB + T/8 bytes) and, up to 131072 tokens, fp32 partial sums for key-tile walks that a
+ * small launch cuts into pieces (16 KiB per token, at most 128 MiB). */
 size_t dsa_attn_bwd_workspace_bytes(int T, int Hq, int max_seqlen, int has_idx);
 /*
  * Byte offset of the selection bitmap inside the backward workspace.  A forward call handed

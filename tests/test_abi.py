@@ -34,9 +34,14 @@ def test_workspace_sizes_without_a_gpu():
     b4 = lib.dsa_index_topk_workspace_bytes(131072, 131072, 2048)
     assert b4 == 2048 * 131072 * 4                         # chunked: 1 GiB of score rows at a time
     up = lambda x: (x + 255) // 256 * 256                  # both parts are 256-byte aligned
-    order = up(((1000 // 128 + 4096 + 1) * 2 + 2) * 4)   # launch order of the key tiles: (segment, tile) pairs and a count
+    # launch order of the key tiles (five words per entry and a header), and fp32 partial sums for key-tile walks
+    # that a small launch cuts into pieces (16 KiB per token, at most 128 MiB, none above 131072 tokens)
+    order = up(((1000 // 128 + 4096 + 1 + 4096) * 5 + 4) * 4) + up(1000 * 16384)
     assert lib.dsa_attn_bwd_workspace_bytes(1000, 8, 640, 0) == up(1000 * 8 * 4) + order
     assert lib.dsa_attn_bwd_workspace_bytes(1000, 8, 640, 1) == up(1000 * 8 * 4) + up(1000 * 20 * 4) + order
+    big = lib.dsa_attn_bwd_workspace_bytes(32768, 32, 7168, 0) - up(32768 * 32 * 4) - up(((32768 // 128 + 4096 + 1 + 4096) * 5 + 4) * 4)
+    assert big == 128 << 20
+    assert lib.dsa_attn_bwd_workspace_bytes(262144, 1, 8, 0) == up(262144 * 4) + up(((262144 // 128 + 4096 + 1 + 4096) * 5 + 4) * 4)
     assert lib.dsa_attn_fwd_workspace_bytes(1000, 640, 1) == up(1000 * 20 * 4)
     assert lib.dsa_attn_bwd_bitmap_offset(1000, 8) == up(1000 * 8 * 4)   # forward workspace fits behind it
     assert lib.dsa_attn_fwd_workspace_bytes(1000, 640, 0) == 0

@@ -2,6 +2,7 @@
 
 Bars: top-k index sets bit-exact given identical fp32 scores; outputs and gradients within
 max-abs 2e-2 and cosine > 0.9995 of the fp32 oracle."""
+import ctypes
 import math
 
 import pytest
@@ -213,6 +214,51 @@ def test_many_segments_in_every_launch_order_of_the_key_tiles(n_short):
     assert_close_bf16(qd.grad, qr.grad, "dq")
     assert_close_bf16(kd.grad, kr.grad, "dk")
     assert_close_bf16(vd.grad, vr.grad, "dv")
+
+
+@pytest.mark.parametrize("D,Hq,Hkv,segs,K", [
+    (128, 4, 1, (3000, 700, 1), 256),                      # one GPU's share of an 8-way head-sharded layer: 31 workgroups
+    (256, 8, 1, (1669, 300), 128),                         # head_dim 256, both halves of head_dim write one partial slot
+    (64, 2, 2, (2500,), 0),                                # dense, a single segment, one head per kv head
+    (128, 12, 3, (1100, 1300, 90), 64),                    # three heads per kv head (padded to four)
+])
+def test_key_tile_walks_cut_into_pieces_match_the_oracle(D, Hq, Hkv, segs, K):
+    """A dK/dV launch of few workgroups cuts long key-tile walks into pieces (fp32 partial sums added in piece order by a
+    second kernel).  The launch-order table in the workspace must say that walks were cut here; out, dq, dk, dv against
+    the oracle as everywhere; a second run is bit-identical."""
+    _log(f"pieces D={D} {Hq}/{Hkv} segs={segs} K={K}")
+    w = W.Workload("pieces", torch.bfloat16, segs, Hq, Hkv, D, 8, 32, max(K, 1), 0.5, 901)
+    t = W.make_inputs(w, device="cpu")
+    d = {k_: (v_.to(DEV) if torch.is_tensor(v_) else v_) for k_, v_ in t.items()}
+    scale = D ** -0.5
+    if K:
+        idx, n = ops.index_topk(d["q_idx"], d["k_idx"], d["w_idx"], d["cu_seqlens"], w.max_seqlen, K)
+    else:
+        idx, n = None, None
+    out, lse = ops.attn_fwd(d["q"], d["k"], d["v"], idx, n, d["cu_seqlens"], w.max_seqlen, scale)
+    lib = ops._lib.load()
+    ws_bytes = lib.dsa_attn_bwd_workspace_bytes(w.T, Hq, w.max_seqlen, 1 if K else 0)
+    ws = torch.zeros((ws_bytes,), dtype=torch.uint8, device=DEV)
+    bufs = (torch.empty_like(d["q"]), torch.empty_like(d["k"]), torch.empty_like(d["v"]), ws)
+    dq, dk, dv, _ = ops.attn_bwd(d["dout"], d["q"], d["k"], d["v"], out, lse, idx, n, d["cu_seqlens"], w.max_seqlen, scale, 15, bufs)
+    torch.cuda.synchronize()
+    lib.dsa_tile_order_bytes.restype = ctypes.c_size_t
+    order_bytes = (lib.dsa_tile_order_bytes(w.T) + 255) // 256 * 256
+    header = ws[ws_bytes - order_bytes: ws_bytes - order_bytes + 16].view(torch.int32).cpu().tolist()
+    assert header[0] > 0 and header[1] >= 32 and header[2] > 0, header      # entries, steps per piece, tiles that were cut
+    if K:
+        wi, wn = idx.cpu(), n.cpu()
+        ro, rq, rk, rv = R.sparse_attention_grads(t["q"], t["k"], t["v"], wi, wn, t["cu_seqlens"], t["dout"])
+    else:
+        qf, kf, vf = (t[x].float().requires_grad_(True) for x in ("q", "k", "v"))
+        ro = R.dense_varlen_causal(qf, kf, vf, t["cu_seqlens"])
+        ro.backward(t["dout"].float())
+        rq, rk, rv, ro = qf.grad, kf.grad, vf.grad, ro.detach()
+    for name, got, want in (("out", out, ro), ("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
+        assert_close_bf16(got, want, name)
+    dk1, dv1 = dk.clone(), dv.clone()
+    ops.attn_bwd(d["dout"], d["q"], d["k"], d["v"], out, lse, idx, n, d["cu_seqlens"], w.max_seqlen, scale, 15, bufs)
+    assert torch.equal(dk, dk1) and torch.equal(dv, dv1)
 
 
 @pytest.mark.parametrize("D,Hq,Hkv,segs,K,sparse", [

@@ -43,9 +43,10 @@ hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const void *k, co
                               int Hq, int Hkv, int D, float scale, int pos_split, int causal, void *dq, hipStream_t stream);
 hipError_t dsa_launch_tile_dkv(const void *dout, const void *q, const void *k, const void *v, const float *lse,
                                const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T,
-                               int Hq, int Hkv, int D, float scale, int causal, int32_t *order, void *dk, void *dv,
-                               hipStream_t stream);
+                               int Hq, int Hkv, int D, float scale, int causal, int32_t *order, float *partial,
+                               size_t partial_bytes, void *dk, void *dv, hipStream_t stream);
 size_t dsa_tile_order_bytes(int T);
+size_t dsa_tile_dkv_partial_bytes(int T);
 }
 
 extern "C" {
@@ -369,6 +370,7 @@ extern "C" size_t dsa_attn_bwd_workspace_bytes(int T, int Hq, int max_seqlen, in
     if (T <= 0) return 0;
     size_t b = align_up((size_t)T * Hq * 4, 256);                                     // delta
     if (has_idx) b += align_up((size_t)T * bitmap_ldw(max_seqlen) * 4, 256);          // selection bitmap
+    b += align_up(dsa_tile_dkv_partial_bytes(T), 256);                                // dK / dV of key-tile walks in pieces
     return b + align_up(dsa_tile_order_bytes(T), 256);                                // launch order of the key tiles
 }
 
@@ -394,6 +396,8 @@ extern "C" int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k
     float *delta = (float *)ws;
     uint32_t *bitmap = idx ? (uint32_t *)((char *)ws + dsa_attn_bwd_bitmap_offset(T, Hq)) : nullptr;
     int32_t *order = (int32_t *)((char *)ws + need - align_up(dsa_tile_order_bytes(T), 256));
+    const size_t partial_bytes = dsa_tile_dkv_partial_bytes(T);
+    float *partial = partial_bytes ? (float *)((char *)order - align_up(partial_bytes, 256)) : nullptr;
     const int split = pos_split_for(idx, K);
     hipStream_t st = (hipStream_t)stream;
     hipError_t e = hipSuccess;
@@ -416,7 +420,8 @@ extern "C" int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k
         }
     }
     if (parts & DSA_BWD_DKV) {
-        e = dsa_launch_tile_dkv(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, causal, order, dk, dv, st);
+        e = dsa_launch_tile_dkv(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, causal, order, partial,
+                                partial_bytes, dk, dv, st);
         if (e != hipSuccess) return hip_fail(e, "tile dkv launch");
     }
     return DSA_OK;

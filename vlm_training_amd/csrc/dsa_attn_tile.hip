@@ -853,29 +853,51 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
 // Launch order of the key-stationary workgroups.  A key tile's walk is as long as the part of its segment
 // behind it, and the hardware starts workgroups in grid order: handed out segment by segment, the long
 // walks of a late long segment start late and the launch ends on them.  This kernel (one workgroup) lists
-// the 128-key tiles of all segments longest walk first - `by_segment` = 0: by the number of tiles behind
-// them, across segments (best balance; for launches of a few rounds of workgroups), `by_segment` = 1: the
-// segments by length, each one's tiles together (workgroups that run side by side then walk the same q / dO
-// rows and share them in L2, which is worth more than the balance once a launch runs for many rounds):
-//   order[0] = number of tiles (or -1: too many segments or tiles for the table, use the plain order),
-//   order[2 + 2 s], order[3 + 2 s] = segment and tile of slot s.
-// The order changes the schedule only; every tile is still reduced by one workgroup in a fixed order.
+// the 128-key tiles of all segments longest walk first -
+//   mode 0: by the number of tiles behind them, across segments (best balance; for launches of a few rounds
+//           of workgroups),
+//   mode 1: the segments by length, each one's tiles together (workgroups that run side by side then walk the
+//           same q / dO rows and share them in L2, which is worth more than the balance once a launch runs
+//           for many rounds),
+//   mode 2: as mode 0, and long walks cut into pieces of `pb` steps (a step = `qb` queries), for launches with
+//           fewer workgroups than a few rounds of the chip: a launch then ends with its longest walk, however
+//           few the workgroups.  A tile in pieces leaves one fp32 partial dK / dV per piece, added in piece
+//           order by dsa_dkv_pieces_reduce_kernel.  Walks are cut only if the longest is more than twice the
+//           steps a CU gets in a balanced launch (all walks x `wg_per_tile` workgroups / 256); pb = the largest
+//           power of two up to half of that (at least 32), doubled until at most `item_cap` entries and
+//           `slot_cap` partial slots are needed; it depends on cu_seqlens and these parameters only.
+// Table:
+//   order[0] = number of entries (or -1: too many segments or tiles for the table, use the plain order),
+//   order[1] = pb (0: no walk is cut), order[2] = number of tiles that are cut,
+//   order[4 + 4 s .. 7 + 4 s] = segment, tile, piece, first partial slot of the tile (-1: not cut) of entry s,
+//   behind the `cap` entries: the entry of the first piece of every cut tile.
+// The pieces of a tile are counted from the walk's length bound 128 r / qb of its rank r (tiles behind it,
+// itself included); a tile whose own walk is shorter leaves its last pieces empty (the kernels and the
+// reduction count the pieces from the walk itself).
+// The order changes the schedule only; every tile is still reduced in a fixed order.
 // ==================================================================================================
 #define DSA_ORDER_MAX_SEGS 4096
 #define DSA_ORDER_MAX_TILES 8192                         // tiles of the longest segment
+#define DSA_ORDER_EXTRA 4096                             // entries beyond one per tile (pieces)
+#define DSA_ORDER_SPLIT_MAX_TILES 1024                   // mode 2: one thread per rank
 static_assert(DSA_ORDER_MAX_TILES + 1 >= 2 * DSA_ORDER_MAX_SEGS, "the rank tables of the by-segment order share cnt[]");
-__global__ __launch_bounds__(1024) void dsa_tile_order_kernel(const int32_t *__restrict__ cu, int N, int cap, int by_segment,
+__device__ __forceinline__ void order_entry(int32_t *order, int slot, int seg, int tile, int piece, int mslot) {
+    *reinterpret_cast<int4 *>(order + 4 + 4 * slot) = make_int4(seg, tile, piece, mslot);
+}
+__global__ __launch_bounds__(1024) void dsa_tile_order_kernel(const int32_t *__restrict__ cu, int N, int cap, int mode, int qb,
+                                                              int wg_per_tile, int item_cap, int slot_cap,
                                                               int32_t *__restrict__ order) {
     __shared__ int nt[DSA_ORDER_MAX_SEGS];               // tiles per segment
     __shared__ int cnt[DSA_ORDER_MAX_TILES + 1];         // cnt[r]: segments with at least r tiles; then: slots before rank r
     __shared__ int part[1024];
-    __shared__ int maxnt_s;
+    __shared__ unsigned long long part64[16];
+    __shared__ int maxnt_s, sum_a, sum_b;
     const int tid = threadIdx.x;
     if (N > DSA_ORDER_MAX_SEGS) {
-        if (tid == 0) order[0] = -1;
+        if (tid == 0) { order[0] = -1; order[1] = 0; order[2] = 0; }
         return;
     }
-    if (tid == 0) maxnt_s = 0;
+    if (tid == 0) { maxnt_s = 0; order[1] = 0; order[2] = 0; }
     __syncthreads();
     int mx = 0;
     for (int i = tid; i < N; i += 1024) {
@@ -890,7 +912,7 @@ __global__ __launch_bounds__(1024) void dsa_tile_order_kernel(const int32_t *__r
         if (tid == 0) order[0] = -1;
         return;
     }
-    if (by_segment) {
+    if (mode == 1) {
         // rank of a segment = segments that are longer, or as long and earlier; cnt[rank] = segment, then its first slot
         int *seg_of = cnt, *first = cnt + DSA_ORDER_MAX_SEGS;     // (both fit: DSA_ORDER_MAX_TILES + 1 >= 2 * DSA_ORDER_MAX_SEGS)
         for (int i = tid; i < N; i += 1024) {
@@ -916,10 +938,7 @@ __global__ __launch_bounds__(1024) void dsa_tile_order_kernel(const int32_t *__r
         if (tid == 0) order[0] = total;
         for (int rk = 0; rk < N; ++rk) {
             const int seg = seg_of[rk], f = first[rk];
-            for (int j = tid; j < nt[seg]; j += 1024) {
-                order[2 + 2 * (f + j)] = seg;
-                order[3 + 2 * (f + j)] = j;
-            }
+            for (int j = tid; j < nt[seg]; j += 1024) order_entry(order, f + j, seg, j, 0, -1);
         }
         return;
     }
@@ -929,6 +948,76 @@ __global__ __launch_bounds__(1024) void dsa_tile_order_kernel(const int32_t *__r
         cnt[r] = c;
     }
     __syncthreads();
+    if (mode == 2 && maxnt <= DSA_ORDER_SPLIT_MAX_TILES) {
+        // thread tid owns rank r = maxnt - tid; pieces of a tile of rank r: ceil((128 r / qb) / pb)
+        const int r = maxnt - tid;
+        const int c = r >= 1 ? cnt[r] : 0, steps = r >= 1 ? r * (128 / qb) : 0;
+        // steps of all walks against the longest one: with `ideal` steps per CU in a balanced launch, walks are cut
+        // only if the longest is more than twice that (below, the pieces' own cost - a pipeline fill each, fp32 partial
+        // sums written and read back - outweighs the balance), into pieces of about half of it
+        if (tid == 0) sum_a = 0;
+        __syncthreads();
+        if (c) atomicAdd(&sum_a, c * steps);
+        __syncthreads();
+        const int longest = maxnt * (128 / qb);
+        const int ideal = (int)(((int64_t)sum_a * wg_per_tile + 255) / 256);
+        __syncthreads();
+        int pb = 32;
+        while (2 * pb <= ideal / 2) pb <<= 1;            // the largest power of two up to ideal / 2, at least 32
+        if (longest <= 2 * ideal) pb = 1 << 30;
+        for (;; pb <<= 1) {
+            const int np = (steps + pb - 1) / pb;
+            if (tid == 0) { sum_a = 0; sum_b = 0; }
+            __syncthreads();
+            if (c) {
+                atomicAdd(&sum_a, c * np);
+                if (np > 1) atomicAdd(&sum_b, c * np);
+            }
+            __syncthreads();
+            const bool fits = sum_a <= item_cap && sum_a <= cap && sum_b <= slot_cap;
+            const bool whole = pb >= longest;                     // no walk is cut any more
+            __syncthreads();
+            if (fits || whole) break;
+        }
+        const int np = (steps + pb - 1) / pb, items = c * np, mults = np > 1 ? c * np : 0;
+        // entries, partial slots and cut tiles of the larger ranks: one scan over the triple (21 bits each of a 64-bit
+        // word: the caps keep every sum below 2^21)
+        const unsigned long long mine = (unsigned long long)items | ((unsigned long long)mults << 21) | ((unsigned long long)(np > 1 ? c : 0) << 42);
+        unsigned long long incl = mine;                  // inclusive scan: inside the wave by lane shifts, then over the 16 waves
+        const int ln = tid & 63, wvi = tid >> 6;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const unsigned int lo32 = __shfl_up((unsigned int)incl, d, 64), hi32 = __shfl_up((unsigned int)(incl >> 32), d, 64);
+            if (ln >= d) incl += (unsigned long long)lo32 | ((unsigned long long)hi32 << 32);
+        }
+        if (ln == 63) part64[wvi] = incl;
+        __syncthreads();
+        unsigned long long wave_before = 0ull, all = 0ull;
+        for (int w2 = 0; w2 < 16; ++w2) {
+            const unsigned long long t2 = part64[w2];
+            if (w2 < wvi) wave_before += t2;
+            all += t2;
+        }
+        const unsigned long long excl = wave_before + incl - mine;
+        const int before[3] = {(int)(excl & 0x1fffffull), (int)((excl >> 21) & 0x1fffffull), (int)(excl >> 42)};
+        const int total = (int)(all & 0x1fffffull);
+        if (total > cap || total > item_cap) {           // (only when even whole walks do not fit)
+            if (tid == 0) order[0] = -1;
+            return;
+        }
+        if (tid == 0) { order[0] = total; order[1] = pb >= longest ? 0 : pb; order[2] = (int)(all >> 42); }
+        if (c) {
+            int slot = before[0], ms = before[1], mt = before[2];
+            int32_t *cut = order + 4 + 4 * cap;          // entries of the first pieces of the cut tiles, for the reduction
+            for (int i = 0; i < N; ++i)
+                if (nt[i] >= r) {
+                    if (np > 1) cut[mt++] = slot;
+                    for (int pc = 0; pc < np; ++pc) order_entry(order, slot++, i, nt[i] - r, pc, np > 1 ? ms : -1);
+                    if (np > 1) ms += np;
+                }
+        }
+        return;
+    }
     // slots before rank r = sum of cnt[r'] over r' > r: ranks are cut into 1024 runs (run t = the ranks
     // maxnt - t per .. downwards), a scan over the runs' sums, then each thread finishes its run
     const int per = (maxnt + 1023) / 1024;
@@ -965,29 +1054,123 @@ __global__ __launch_bounds__(1024) void dsa_tile_order_kernel(const int32_t *__r
     for (int r = 1 + tid; r <= maxnt; r += 1024) {
         int slot = cnt[r];
         for (int i = 0; i < N; ++i)
-            if (nt[i] >= r) {
-                order[2 + 2 * slot] = i;
-                order[3 + 2 * slot] = nt[i] - r;
-                ++slot;
-            }
+            if (nt[i] >= r) order_entry(order, slot++, i, nt[i] - r, 0, -1);
     }
 }
-extern "C" size_t dsa_tile_order_bytes(int T) { return ((size_t)(T / 128 + DSA_ORDER_MAX_SEGS + 1) * 2 + 2) * sizeof(int32_t); }
-// the tile of workgroup slot `slot`: from the order table when there is one, else segment by segment
-__device__ __forceinline__ bool locate_key_tile(const int32_t *order, const int32_t *cu, int N, int slot, int &s0, int &L, int &blk) {
+static inline int order_entries_cap(int T) { return T / 128 + DSA_ORDER_MAX_SEGS + 1 + DSA_ORDER_EXTRA; }
+extern "C" size_t dsa_tile_order_bytes(int T) { return ((size_t)order_entries_cap(T) * 5 + 4) * sizeof(int32_t); }
+// the tile (and the piece of its walk) of workgroup slot `slot`: from the order table when there is one, else
+// segment by segment
+__device__ __forceinline__ bool locate_key_tile(const int32_t *order, const int32_t *cu, int N, int slot, int &s0, int &L, int &blk,
+                                                int &piece, int &mslot, int &pb) {
+    piece = 0;
+    mslot = -1;
+    pb = 0;
     if (order) {
         const int total = __builtin_amdgcn_readfirstlane(order[0]);
         if (total >= 0) {
             if (slot >= total) return false;
             // (every lane reads the same words; the lane reads tell the compiler that the results are wave-uniform)
-            const int seg = min(max(__builtin_amdgcn_readfirstlane(order[2 + 2 * slot]), 0), N - 1);
-            blk = __builtin_amdgcn_readfirstlane(order[3 + 2 * slot]);
+            const int4 e = *reinterpret_cast<const int4 *>(order + 4 + 4 * slot);
+            const int seg = min(max(__builtin_amdgcn_readfirstlane(e.x), 0), N - 1);
+            blk = __builtin_amdgcn_readfirstlane(e.y);
+            piece = max(__builtin_amdgcn_readfirstlane(e.z), 0);
+            mslot = __builtin_amdgcn_readfirstlane(e.w);
+            pb = max(__builtin_amdgcn_readfirstlane(order[1]), 0);
             s0 = __builtin_amdgcn_readfirstlane(cu[seg]);
             L = __builtin_amdgcn_readfirstlane(cu[seg + 1]) - s0;
             return blk >= 0;
         }
     }
     return locate_block(cu, N, slot, 128, false, s0, L, blk);
+}
+// A walk of `nblocks` steps (block nblocks-1-b at step b, `QB` queries each, the queries q0 .. Lq-1) cut into pieces
+// of `pb` steps: narrows q0, Lq and nblocks to piece `piece` and returns the number of pieces (1: the whole walk,
+// 0: this piece is empty).  Block boundaries stay where they are, so a piece's blocks are the walk's own.
+__device__ __forceinline__ int walk_piece(int pb, int piece, int QB, int &q0, int &Lq, int &nblocks) {
+    if (pb <= 0 || nblocks <= pb) return piece == 0 ? 1 : 0;
+    const int np = (nblocks + pb - 1) / pb;
+    if (piece >= np) return 0;
+    const int b_lo = piece * pb, b_hi = min(b_lo + pb, nblocks);
+    if (b_lo > 0) Lq = q0 + (nblocks - b_lo) * QB;
+    q0 += (nblocks - b_hi) * QB;
+    nblocks = b_hi - b_lo;
+    return np;
+}
+// one 32-column d-tile of a C-layout accumulator as fp32 (lane = row j; a lane holds the four columns
+// 8*g4 + 4*h + {0..3} of every group g4)
+__device__ __forceinline__ void store_c_tile_f32(float *row_dt, const f32x16 &acc, int h) {
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4) {
+        const f32x4 w = {acc[4 * g4], acc[4 * g4 + 1], acc[4 * g4 + 2], acc[4 * g4 + 3]};
+        *reinterpret_cast<f32x4 *>(row_dt + 8 * g4 + 4 * h) = w;
+    }
+}
+// fp32 partial dK / dV of piece `piece` of a tile in pieces: [slot][kv head][dK | dV][128 keys][D]
+__device__ __forceinline__ float *piece_partial(float *partial, int mslot, int piece, int Hkv, int kvh, int D) {
+    return partial + ((int64_t)(mslot + piece) * Hkv + kvh) * (2 * 128 * (int64_t)D);
+}
+// Adds the pieces of every tile that was cut, in piece order, and writes its dK (times the softmax scale) and dV
+// rows.  Grid: (cut tiles at most, kv heads, DSA_PIECES_Z slices of a tile's rows).
+#define DSA_PIECES_Z 4
+__global__ __launch_bounds__(256) void dsa_dkv_pieces_reduce_kernel(const int32_t *__restrict__ order, int cap,
+                                                                    const float *__restrict__ partial, const int32_t *__restrict__ cu,
+                                                                    int N, int Hkv, int D, int qb, int seq_clamp, float scale,
+                                                                    bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    if ((int)blockIdx.x >= __builtin_amdgcn_readfirstlane(order[2])) return;
+    const int entry = __builtin_amdgcn_readfirstlane(order[4 + 4 * cap + blockIdx.x]);
+    int s0, L, blk, piece, mslot, pb;
+    if (!locate_key_tile(order, cu, N, entry, s0, L, blk, piece, mslot, pb)) return;
+    if (piece != 0 || mslot < 0 || pb <= 0) return;
+    L = min(L, seq_clamp);
+    const int c0 = blk * 128;
+    if (c0 >= L) return;
+    const int nblocks = (L - c0 + qb - 1) / qb;          // (pieces only exist for causal launches: the walk starts at the tile)
+    if (nblocks <= pb) return;                           // (its walk fits one piece after all: piece 0 wrote the rows itself)
+    const int np = (nblocks + pb - 1) / pb, kvh = blockIdx.y;
+    const int keys = min(128, L - c0), cpr = D / 4;      // 16-byte chunks per row
+    const int64_t slot_f = 2 * 128 * (int64_t)D;         // floats per (slot, kv head)
+    const float *base = partial + ((int64_t)mslot * Hkv + kvh) * slot_f;
+    constexpr int U = 4;                                 // independent chunks per thread and pass
+    const int chunks = 2 * keys * cpr;                   // dK rows, then dV rows
+    for (int c0_ = (blockIdx.z * 256 + threadIdx.x) * U; c0_ < chunks; c0_ += DSA_PIECES_Z * 256 * U) {
+        f32x4 acc[U];
+        int64_t off[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = min(c0_ + u, chunks - 1);
+            const int m = c / (keys * cpr), rest = c % (keys * cpr);
+            off[u] = ((int64_t)m * 128 + rest / cpr) * D + (rest % cpr) * 4;
+            acc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        for (int pc = 0; pc < np; pc += 2) {             // piece order: the sum does not depend on the schedule
+            const bool two = pc + 1 < np;
+            const float *src0 = base + (int64_t)pc * Hkv * slot_f, *src1 = base + (int64_t)(two ? pc + 1 : pc) * Hkv * slot_f;
+            f32x4 x0[U], x1[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                x0[u] = *reinterpret_cast<const f32x4 *>(src0 + off[u]);
+                x1[u] = *reinterpret_cast<const f32x4 *>(src1 + off[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                acc[u] += x0[u];
+                if (two) acc[u] += x1[u];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = c0_ + u;
+            if (c < chunks) {
+                const int m = c / (keys * cpr), rest = c % (keys * cpr);
+                const float mul = m ? 1.f : scale;
+                bf16_t *outp = m ? dv : dk;
+                uint32_t *dst = reinterpret_cast<uint32_t *>(outp + ((int64_t)(s0 + c0 + rest / cpr) * Hkv + kvh) * D + (rest % cpr) * 4);
+                dst[0] = pack2bf(acc[u][0] * mul, acc[u][1] * mul);
+                dst[1] = pack2bf(acc[u][2] * mul, acc[u][3] * mul);
+            }
+        }
+    }
 }
 
 // ==================================================================================================
@@ -1015,7 +1198,8 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
-    float scale, int causal, const int32_t *__restrict__ order, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    float scale, int causal, const int32_t *__restrict__ order, float *__restrict__ partial, bf16_t *__restrict__ dk,
+    bf16_t *__restrict__ dv) {
     static_assert(D == 256, "head_dim <= 128 runs dsa_tile_dkv2_kernel");
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>();
     constexpr int NQD = 3, LEAD = 1;                     // q/dO ring slots; blocks staged ahead of the producers
@@ -1046,8 +1230,8 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     const bool consumer = wv >= 4;
     const int G = Hq / Hkv;
     const int kvh = bx % Hkv;
-    int s0, L, blk;
-    if (!locate_key_tile(order, cu, N, bx / Hkv, s0, L, blk)) return;
+    int s0, L, blk, piece, mslot, pb;
+    if (!locate_key_tile(order, cu, N, bx / Hkv, s0, L, blk, piece, mslot, pb)) return;
     if (HAS_IDX) L = min(L, ldw * 32);                  // a bitmap row has ldw words whatever the caller's max_seqlen
     if (blk * 128 >= L) return;                         // (whole workgroup, before its first barrier)
     const int c0 = blk * 128, kc = c0 + kg * 32;
@@ -1055,8 +1239,11 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
     const bool key_ok = mykey < L;
     const int64_t krow = (int64_t)(s0 + min(mykey, L - 1)) * Hkv + kvh;
     const float scale_log2 = scale * LOG2E_F;
-    const int q0 = causal ? c0 : 0;                      // first query column that can see this key tile
-    const int nblocks = (L - q0 + QB - 1) / QB;          // queries q0 .. L-1
+    // the walk: queries q0 .. Lq-1 in nblocks steps - all queries that can see this key tile, or one piece of them
+    int q0_ = causal ? c0 : 0, Lq_ = L, nblocks_ = (L - q0_ + QB - 1) / QB;
+    const int npieces = walk_piece((causal && partial && mslot >= 0) ? pb : 0, piece, QB, q0_, Lq_, nblocks_);
+    if (npieces == 0) return;
+    const int q0 = q0_, Lq = Lq_, nblocks = nblocks_;
 
     if (consumer) {
         // ================= consumers: stage block b+2, then dV^T, dK^T of block b-1 =================
@@ -1092,7 +1279,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
             const int c = i * 256 + ctid, srow = c / CPR, sch = c % CPR;
             const int hd = min(srow & (Gp - 1), G - 1);
             const int qr = srow >> GSHIFT;
-            const int over = max(q0 + last * QB + qr - (L - 1), 0);      // rows past the end in the last block
+            const int over = max(q0 + last * QB + qr - (Lq - 1), 0);     // rows past the end in the last block
             const int64_t off = ((int64_t)(s0 + q0 + last * QB + qr - over) * Hq + kvh * G + hd) * D + sch * 8;
             qp[i] = reinterpret_cast<const unsigned char *>(q + off);
             dp[i] = reinterpret_cast<const unsigned char *>(dout + off);
@@ -1102,7 +1289,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
             lds_off[i] = tile_off<D>(srow, sch);
         }
         const int64_t aux_blk_bytes = (int64_t)aux_stride * QB * 4;
-        const int aux_over = max(q0 + last * QB + aux_q - (L - 1), 0);
+        const int aux_over = max(q0 + last * QB + aux_q - (Lq - 1), 0);
         const int64_t aux_dlast = -(int64_t)aux_stride * aux_over * 4;
         const unsigned char *ap =
             reinterpret_cast<const unsigned char *>(aux_base + (int64_t)aux_stride * (q0 + last * QB + aux_q - aux_over));
@@ -1198,7 +1385,14 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
             if (b >= 1) consume(b - 1);
             __syncthreads();
         }
-        if (key_ok) {
+        if (npieces > 1) {                               // a piece of the walk: fp32 partial sums, added by the reduction
+            float *pk = piece_partial(partial, mslot, piece, Hkv, kvh, D) + (kg * 32 + j) * D + dt0 * 32, *pv_ = pk + 128 * D;
+#pragma unroll
+            for (int dt = 0; dt < DTC; ++dt) {
+                store_c_tile_f32(pk + dt * 32, dkacc[dt], h);
+                store_c_tile_f32(pv_ + dt * 32, dvacc[dt], h);
+            }
+        } else if (key_ok) {
             bf16_t *pk = dk + krow * D + dt0 * 32, *pv_ = dv + krow * D + dt0 * 32;
 #pragma unroll
             for (int dt = 0; dt < DTC; ++dt) {
@@ -1320,7 +1514,8 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
     const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
-    float scale, int causal, const int32_t *__restrict__ order, bf16_t *__restrict__ dk, bf16_t *__restrict__ dv) {
+    float scale, int causal, const int32_t *__restrict__ order, float *__restrict__ partial, bf16_t *__restrict__ dk,
+    bf16_t *__restrict__ dv) {
     static_assert(D <= 128, "head_dim 256 runs dsa_tile_dkvpc_kernel");
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>();
     constexpr int NCHUNK = 32 * CPR, STG = 256, CPT = NCHUNK / STG;
@@ -1341,8 +1536,8 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
     const int kg = wv & 3;
     const int G = Hq / Hkv;
     const int kvh = blockIdx.x % Hkv;
-    int s0, L, blk;
-    if (!locate_key_tile(order, cu, N, blockIdx.x / Hkv, s0, L, blk)) return;
+    int s0, L, blk, piece, mslot, pb;
+    if (!locate_key_tile(order, cu, N, blockIdx.x / Hkv, s0, L, blk, piece, mslot, pb)) return;
     if (HAS_IDX) L = min(L, ldw * 32);
     if (blk * 128 >= L) return;                         // (whole workgroup, before its first barrier)
     const int c0 = blk * 128, kc = c0 + kg * 32;
@@ -1350,8 +1545,12 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
     const bool key_ok = mykey < L;
     const int64_t krow = (int64_t)(s0 + min(mykey, L - 1)) * Hkv + kvh;
     const float scale_log2 = scale * LOG2E_F, inv_scale = 1.f / scale;
-    const int q0 = causal ? c0 : 0;
-    const int nblocks = (L - q0 + QB - 1) / QB;          // queries q0 .. L-1; step s handles block nblocks-1-s
+    // the walk: queries q0 .. Lq-1 in nblocks steps (step s handles block nblocks-1-s) - all queries that can see
+    // this key tile, or one piece of them
+    int q0_ = causal ? c0 : 0, Lq_ = L, nblocks_ = (L - q0_ + QB - 1) / QB;
+    const int npieces = walk_piece((causal && partial && mslot >= 0) ? pb : 0, piece, QB, q0_, Lq_, nblocks_);
+    if (npieces == 0) return;
+    const int q0 = q0_, Lq = Lq_, nblocks = nblocks_;
 
     // an accumulator in C layout that starts from a per-row value (lane (key, h) holds rows 8 g4 + 4 h + e)
     auto rows_init = [&](const float *rowv) __attribute__((always_inline)) {
@@ -1379,7 +1578,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
         const int c = i * STG + ctid, srow = c / CPR, sch = c % CPR;
         const int hd = min(srow & (Gp - 1), G - 1);
         const int qr = srow >> GSHIFT;
-        const int over = max(q0 + last * QB + qr - (L - 1), 0);      // rows past the end in the last block
+        const int over = max(q0 + last * QB + qr - (Lq - 1), 0);     // rows past the end in the last block
         const int64_t off = ((int64_t)(s0 + q0 + last * QB + qr - over) * Hq + kvh * G + hd) * D + sch * 8;
         qp[i] = reinterpret_cast<const unsigned char *>(q + off);
         dp[i] = reinterpret_cast<const unsigned char *>(dout + off);
@@ -1415,7 +1614,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
         aux_lds = (64 + w * 32 + aux_q) * 4;
     }
     const int64_t aux_blk_bytes = (int64_t)aux_stride * QB * 4;
-    const int aux_over = max(q0 + last * QB + aux_q - (L - 1), 0);
+    const int aux_over = max(q0 + last * QB + aux_q - (Lq - 1), 0);
     const int64_t aux_dlast = -(int64_t)aux_stride * aux_over * 4;
     const unsigned char *ap =
         reinterpret_cast<const unsigned char *>(aux_base + (int64_t)aux_stride * (q0 + last * QB + aux_q - aux_over));
@@ -1579,7 +1778,11 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
         if (s <= nblocks) DKV2_DS_STEP(s, qst0, dost0, aux_st0)
 #undef DKV2_DS_STEP
 #undef DKV2_DS_STEADY
-        if (key_ok) {
+        if (npieces > 1) {                               // a piece of the walk: fp32 partial sums, added by the reduction
+            float *pk = piece_partial(partial, mslot, piece, Hkv, kvh, D) + (kg * 32 + j) * D;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) store_c_tile_f32(pk + dt * 32, dkacc[dt], h);
+        } else if (key_ok) {
             bf16_t *pk = dk + krow * D;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) store_c_tile(pk + dt * 32, dkacc[dt], scale, h);
@@ -1709,7 +1912,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
     read_aux(0);
     // The blocks that can touch the causal diagonal come last; the steady loop before them has no mask
     // arithmetic besides the selection bits.
-    const int nb_diag = causal ? (kc + 32 - q0 + QB - 1) / QB : 0;
+    const int nb_diag = causal ? max(kc + 32 - q0 + QB - 1, 0) / QB : 0;   // (none for a piece that starts past the diagonal)
     const int steady = max(nblocks - nb_diag, 1);        // steps [1, steady) see blocks fully past the diagonal
     step(yes, yes, no, 0);
     __syncthreads();
@@ -1724,7 +1927,11 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
     }
     step(yes, no, yes, nblocks);
     __syncthreads();
-    if (key_ok) {
+    if (npieces > 1) {
+        float *pv_ = piece_partial(partial, mslot, piece, Hkv, kvh, D) + (128 + kg * 32 + j) * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) store_c_tile_f32(pv_ + dt * 32, dvacc[dt], h);
+    } else if (key_ok) {
         bf16_t *pv_ = dv + krow * D;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) store_c_tile(pv_ + dt * 32, dvacc[dt], 1.f, h);
@@ -1771,7 +1978,8 @@ static hipError_t launch_dq_i(dim3 grid, hipStream_t stream, const void *dout, c
 template <int D, bool HAS_IDX, int GS>
 static hipError_t launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
                          const float *lse, const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N,
-                         int T, int Hq, int Hkv, float scale, int causal, const int32_t *order, void *dk, void *dv) {
+                         int T, int Hq, int Hkv, float scale, int causal, const int32_t *order, float *partial, void *dk,
+                         void *dv) {
     // LDS above 64 KiB has to be requested per kernel and device; asked for on every launch (a host-side table
     // lookup), so that neither a second device nor a second thread can meet a kernel that was never configured
     if constexpr (D <= 128) {
@@ -1780,7 +1988,7 @@ static hipError_t launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, 
         if (e2 != hipSuccess) return e2;
         hipLaunchKernelGGL((dsa_tile_dkv2_kernel<D, HAS_IDX, GS>), grid, dim3(512), dkv2_lds_bytes<D>(), stream,
                            (const bf16_t *)dout, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap,
-                           ldw, cu, N, T, Hq, Hkv, scale, causal, order, (bf16_t *)dk, (bf16_t *)dv);
+                           ldw, cu, N, T, Hq, Hkv, scale, causal, order, partial, (bf16_t *)dk, (bf16_t *)dv);
         return hipSuccess;
     } else {
     const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(&dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>),
@@ -1789,7 +1997,7 @@ static hipError_t launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, 
     // two workgroups per key tile and kv head, one per half of head_dim (a consumer wave holds 128 accumulator registers)
     hipLaunchKernelGGL((dsa_tile_dkvpc_kernel<D, HAS_IDX, GS>), dim3(grid.x * 2), dim3(512), dkvpc_lds_bytes<D>(), stream,
                        (const bf16_t *)dout, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap,
-                       ldw, cu, N, T, Hq, Hkv, scale, causal, order, (bf16_t *)dk, (bf16_t *)dv);
+                       ldw, cu, N, T, Hq, Hkv, scale, causal, order, partial, (bf16_t *)dk, (bf16_t *)dv);
     return hipSuccess;
     }
 }
@@ -1887,18 +2095,43 @@ extern "C" hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const 
     TILE_SWITCH(launch_dq_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, pos_split, causal, dq)
     return hipGetLastError();
 }
+// bytes of fp32 partial sums a launch of T tokens may use for key-tile walks in pieces (0: launches of this size are
+// never cut); a slot = the dK and dV of one 128-key tile and kv head
+extern "C" size_t dsa_tile_dkv_partial_bytes(int T) {
+    if (T <= 0 || T > 131072) return 0;
+    const size_t b = (size_t)T * 16384;
+    return b < ((size_t)128 << 20) ? b : ((size_t)128 << 20);
+}
 extern "C" hipError_t dsa_launch_tile_dkv(const void *dout, const void *q, const void *k, const void *v,
                                           const float *lse, const float *delta, const uint32_t *bitmap, int ldw,
                                           const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale, int causal,
-                                          int32_t *order, void *dk, void *dv, hipStream_t stream) {
+                                          int32_t *order, float *partial, size_t partial_bytes, void *dk, void *dv,
+                                          hipStream_t stream) {
     const int gs = group_shift(Hq, Hkv);
-    const dim3 grid((unsigned)(((int64_t)T / 128 + N + 1) * Hkv));
-    // `order` (dsa_tile_order_bytes(T) bytes, or null): the tiles are listed longest walk first before the launch
-    if (order && N > 1)
-        hipLaunchKernelGGL(dsa_tile_order_kernel, dim3(1), dim3(1024), 0, stream, cu, N, T / 128 + DSA_ORDER_MAX_SEGS + 1,
-                           grid.x > 4 * 256 ? 1 : 0, order);
-    else
+    const int tiles_ub = T / 128 + N;                    // 128-key tiles of all segments, at most
+    dim3 grid((unsigned)((tiles_ub + 1) * Hkv));
+    // `order` (dsa_tile_order_bytes(T) bytes, or null): the tiles are listed longest walk first before the launch.
+    // A launch of at most four workgroups per CU may also cut long walks into pieces (`partial`: fp32 partial sums), so
+    // that it does not end on a few long walks with most of the chip idle.
+    const int wg_per_tile = Hkv * (D > 128 ? 2 : 1);
+    const int64_t slot_pairs = partial ? (int64_t)(partial_bytes / ((size_t)2 * 128 * D * sizeof(float))) : 0;
+    const bool pieces = order && causal && slot_pairs >= Hkv && (int64_t)tiles_ub * wg_per_tile <= 4 * 256;
+    int item_cap = 0;
+    if (order && (N > 1 || pieces)) {
+        const int cap = order_entries_cap(T);
+        item_cap = pieces ? std::min(cap, tiles_ub + (1024 + wg_per_tile - 1) / wg_per_tile) : cap;
+        hipLaunchKernelGGL(dsa_tile_order_kernel, dim3(1), dim3(1024), 0, stream, cu, N, cap,
+                           pieces ? 2 : (grid.x > 4 * 256 ? 1 : 0), 32 >> gs, wg_per_tile, item_cap, (int)(slot_pairs / Hkv < (1 << 20) ? slot_pairs / Hkv : (1 << 20)),   /* (sums stay below 2^21) */
+                           order);
+        if (pieces) grid.x = (unsigned)(item_cap * Hkv);
+    } else {
         order = nullptr;                                 // one segment: its tiles are in order already
-    TILE_SWITCH(launch_dkv_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, causal, order, dk, dv)
+    }
+    if (!pieces) partial = nullptr;
+    TILE_SWITCH(launch_dkv_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, causal, order, partial, dk, dv)
+    if (pieces)
+        hipLaunchKernelGGL(dsa_dkv_pieces_reduce_kernel, dim3(tiles_ub, Hkv, DSA_PIECES_Z), dim3(256), 0, stream, order,
+                           order_entries_cap(T), partial, cu, N, Hkv, D, 32 >> gs, bitmap ? ldw * 32 : 0x7fffffff, scale,
+                           (bf16_t *)dk, (bf16_t *)dv);
     return hipGetLastError();
 }

@@ -87,6 +87,17 @@ def scaled(w: Workload, seg_lens, top_k=None, name=None) -> Workload:
                     top_k if top_k is not None else w.top_k, w.sigma, w.seed, w.image_runs)
 
 
+def head_shard(w: Workload, ways: int) -> Workload:
+    """One GPU's share when the attention heads are split ``ways`` ways, as the reference's tensor parallelism does
+    (``train/infra.py:385-469``: q/k/v projections column-parallel, so the operator sees Hq/ways and Hkv/ways heads of
+    the same packed rows).  The indexer is left whole: its selection is shared by all heads."""
+    if ways < 1 or w.Hq % ways or (w.Hkv % ways and ways % w.Hkv):
+        raise ValueError(f"cannot split {w.Hq}/{w.Hkv} heads {ways} ways")
+    hkv = max(w.Hkv // ways, 1)                         # kv heads are replicated once there are fewer than ranks
+    return Workload(f"{w.name}-heads/{ways}", w.dtype, w.seg_lens, w.Hq // ways, hkv, w.D, w.Hi, w.Di, w.top_k, w.sigma, w.seed,
+                    w.image_runs)
+
+
 def make_inputs(w: Workload, device="cpu", with_dout: bool = True):
     """Returns dict(q,k,v,q_idx,k_idx,w_idx,dout,cu_seqlens,max_seqlen) on ``device``."""
     g = torch.Generator(device="cpu").manual_seed(w.seed)
