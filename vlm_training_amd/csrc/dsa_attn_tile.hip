@@ -1175,8 +1175,9 @@ __global__ __launch_bounds__(256) void dsa_dkv_pieces_reduce_kernel(const int32_
 
 // ==================================================================================================
 // dK, dV for head_dim 256, producer/consumer form, key-stationary ("scatter by key": every key row is
-// reduced by exactly one wave, in a fixed query order, so the result needs no atomics and is
-// bit-reproducible).  A workgroup owns a 128-key tile (4 groups of 32 keys) of one segment and kv head and
+// reduced by one wave, in a fixed query order - or, when the launch cuts the walk into pieces, by one wave per
+// piece and a sum over the pieces in piece order - so the result needs no atomics and is bit-reproducible).
+// A workgroup owns a 128-key tile (4 groups of 32 keys) of one segment and kv head and
 // walks the later queries in blocks of 32 (query, head) rows, from the end of the segment down to the key
 // tile: workgroups that run side by side then read the same q / dO rows at about the same time and share
 // them in L2.
