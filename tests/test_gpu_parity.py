@@ -314,6 +314,49 @@ def test_dense_path_equals_reference_semantics():
         assert_close_bf16(vd.grad, vr.grad, "dv")
 
 
+@pytest.mark.parametrize("Hq,Hkv,D,causal,segs", [
+    (16, 16, 72, False, (1024, 300, 77)),                  # the 1152 / 16 vision tower: padded to the head_dim-96 kernels
+    (8, 2, 96, True, (700, 1, 333, 1500)),                 # head_dim 96 itself, causal, four heads per kv head
+    (6, 2, 80, True, (513, 129)),                          # three heads per kv head (padded to four)
+    (4, 1, 96, True, (3000, 700)),                         # few workgroups: dK/dV walks in pieces at head_dim 96
+    (2, 2, 88, False, (2, 31, 64, 5)),                     # tiny segments
+])
+def test_head_dim_96_kernels_without_a_selection(Hq, Hkv, D, causal, segs):
+    """Head dims between 64 and 96 run on head_dim-96 instantiations of the three tile kernels when no keys are selected
+    (rows padded with zero columns by the operator; the 72-wide heads of the vision towers wasted 44 % of the matrix
+    work at 128).  out, dq, dk, dv against the oracle; the kernels refuse head_dim 96 with a selection."""
+    _log(f"head_dim 96 path: {Hq}/{Hkv}/{D} causal={causal} segs={segs}")
+    g = torch.Generator().manual_seed(D * 7 + Hq)
+    cu = [0]
+    for L in segs:
+        cu.append(cu[-1] + L)
+    T = cu[-1]
+    q = (torch.randn(T, Hq, D, generator=g) * 0.6).bfloat16()
+    k = (torch.randn(T, Hkv, D, generator=g) * 0.6).bfloat16()
+    v = (torch.randn(T, Hkv, D, generator=g) * 0.6).bfloat16()
+    do = torch.randn(T, Hq, D, generator=g).bfloat16()
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    cud = torch.tensor(cu, dtype=torch.int32, device=DEV)
+    out = ops.dsa_varlen_attn(qd, kd, vd, cud, max(segs), causal=causal)
+    assert out.shape == (T, Hq, D)
+    out.backward(do.to(DEV))
+    qr, kr, vr = (x.float().requires_grad_(True) for x in (q, k, v))
+    ref = R.dense_varlen_causal(qr, kr, vr, cu, causal=causal)
+    ref.backward(do.float())
+    assert_close_bf16(out, ref, "out")
+    assert_close_bf16(qd.grad, qr.grad, "dq")
+    assert_close_bf16(kd.grad, kr.grad, "dk")
+    assert_close_bf16(vd.grad, vr.grad, "dv")
+    if D == 96:                                             # the C ABI takes head_dim 96 as it is, and only without idx
+        q96, k96, v96 = qd.detach(), kd.detach(), vd.detach()
+        o2, lse2 = ops.attn_fwd(q96, k96, v96, None, None, cud, max(segs), D ** -0.5, causal=causal)
+        assert torch.equal(o2, out.detach())
+        idx = torch.zeros(T, 4, dtype=torch.int32, device=DEV)
+        nn = torch.ones(T, dtype=torch.int32, device=DEV)
+        with pytest.raises(RuntimeError):
+            ops.attn_fwd(q96, k96, v96, idx, nn, cud, max(segs), D ** -0.5)
+
+
 def test_non_causal_packed_attention_for_the_vision_towers():
     """causal=False: every key of the own segment (models/qwen3_vl/model.py:423-428 calls
     dispatch_varlen_attention(..., causal=False) with cu_seqlens built from grid_thw)."""
@@ -451,10 +494,11 @@ def test_argument_errors_cross_the_boundary_as_exceptions(monkeypatch):
     k = torch.zeros(8, 2, 96, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ValueError):
         ops.dsa_varlen_attn(q, k, k, cu, 8)
-    q = torch.zeros(8, 4, 96, dtype=torch.bfloat16, device=DEV)
-    assert ops.dsa_varlen_attn(q, k, k, cu, 8).shape == q.shape        # padded to head_dim 128 and cut back
+    q = torch.zeros(8, 4, 80, dtype=torch.bfloat16, device=DEV)
+    k = torch.zeros(8, 2, 80, dtype=torch.bfloat16, device=DEV)
+    assert ops.dsa_varlen_attn(q, k, k, cu, 8).shape == q.shape        # padded to head_dim 96 and cut back
     with pytest.raises(RuntimeError):
-        ops.attn_fwd(q, k, k, None, None, cu, 8, 0.1)  # the C ABI itself covers head_dim 64 / 128 / 256 only
+        ops.attn_fwd(q, k, k, None, None, cu, 8, 0.1)  # the C ABI itself covers head_dim 64 / 128 / 256 (and 96 without idx)
     big = torch.zeros(8, 2, 320, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ValueError):
         ops.dsa_varlen_attn(big, big, big, cu, 8)

@@ -237,7 +237,8 @@ static int check_attn(int T, int N, const int32_t *cu, int Hq, int Hkv, int D, i
     if (dtype != DSA_DTYPE_BF16) return fail(DSA_ERR_UNSUPPORTED, "q/k/v must be bf16 (dtype code %d)", dtype);
     if (Hq < 1 || Hkv < 1 || Hq % Hkv) return fail(DSA_ERR_ARG, "Hq=%d must be a positive multiple of Hkv=%d", Hq, Hkv);
     if (Hq / Hkv > 16) return fail(DSA_ERR_UNSUPPORTED, "Hq/Hkv=%d: at most 16 query heads per kv head", Hq / Hkv);
-    if (!(D == 64 || D == 128 || D == 256)) return fail(DSA_ERR_UNSUPPORTED, "head_dim=%d: need 64, 128 or 256", D);
+    if (!(D == 64 || D == 128 || D == 256 || (D == 96 && !idx)))
+        return fail(DSA_ERR_UNSUPPORTED, "head_dim=%d: need 64, 128 or 256 (96 as well without a key selection)", D);
     if ((idx == nullptr) != (n == nullptr)) return fail(DSA_ERR_ARG, "idx and n must both be given or both be null");
     if (idx && K < 1) return fail(DSA_ERR_ARG, "top_k=%d must be >= 1", K);
     if ((int64_t)T * Hkv >= ((int64_t)1 << 31)) return fail(DSA_ERR_UNSUPPORTED, "T*Hkv too large for one launch");

@@ -18,13 +18,14 @@
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }   // v_exp_f32; exp2(-inf) = 0
 
-// ---- LDS tile: 32 rows of D bf16 with a pitch of D*2 + 64 bytes; chunk = 16 bytes ------------------
+// ---- LDS tile: 32 rows of D bf16 with a pitch of D*2 + 64 bytes (+ 128 at head_dim 96); chunk = 16 bytes ----
 // The LDS of gfx950 has 64 four-byte banks (256 B per clock).  A 16-byte read is served 16 lanes at a
 // time and a transposed 8-byte read 32 lanes at a time, so a row-wise operand read (16 consecutive rows,
 // same chunk) and a transposed read (4 consecutive rows x 64 B) must each cover all banks once.  The
 // 64-byte skew per row separates 4 consecutive rows, the XOR of the chunk's two low bits with row bits
 // 2-3 separates rows 4 apart: both read patterns and the row-wise staging writes are conflict-free.
-template <int D> constexpr int tile_pitch() { return D * 2 + 64; }
+// (The skew needs a pitch of 64 modulo 256 bytes: head_dim 96 pads its rows to the pitch of head_dim 128.)
+template <int D> constexpr int tile_pitch() { return D == 96 ? 320 : D * 2 + 64; }
 template <int D> constexpr int tile_bytes() { return 32 * tile_pitch<D>(); }
 __device__ __forceinline__ int tile_sw(int row) { return (row >> 2) & 3; }
 template <int D>
@@ -193,10 +194,11 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
     float scale_log2, int pos_split, int causal, bf16_t *__restrict__ out, float *__restrict__ lse) {
-    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / (NW * 64);
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>();
     constexpr int NBUF = (D > 128) ? 1 : 2;           // double buffering where 64 KiB of static LDS allow it
     constexpr int NT = NW * 64, Gp = 1 << GSHIFT, QBW = (NW * 32) >> GSHIFT;
-    static_assert(LOADS >= 1, "tile must give every thread a chunk");
+    constexpr int CH = 32 * CPR, LOADS = (CH + NT - 1) / NT;   // 16-byte chunks per matrix; per thread (head_dim 96: not all threads)
+    static_assert(CH % 64 == 0, "whole waves stage or do not");
     __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];   // [buffer][K|V]
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
@@ -216,7 +218,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     const int t = s0 + min(qcol, L - 1), hq = kvh * G + min(head, G - 1);
     u32x4 kst[2][LOADS], vst[2][LOADS];
 #define FWD_LOAD(SET, TILE)                                                                         \
-    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) if (CH % NT == 0 || i * NT + tid < CH) {     \
         const int c = i * NT + tid;                                                               \
         const int row = c / CPR, ch = c % CPR;                                                     \
         const int64_t off = ((int64_t)(s0 + min((TILE) * 32 + row, L - 1)) * Hkv + kvh) * D + ch * 8; \
@@ -239,7 +241,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     uint32_t word_next = HAS_IDX ? wrow[0] : 0u;        // unconditional loads; rows that are not live are masked at use
 
 #define FWD_STORE(SET, BUF, TILE)                                                                        \
-    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) if (CH % NT == 0 || i * NT + tid < CH) {     \
         const int c = i * NT + tid;                                                               \
         const int row = c / CPR, ch = c % CPR;                                                     \
         *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(row, ch)]) = kst[SET][i];              \
@@ -746,9 +748,11 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
     float scale, int pos_split, int causal, bf16_t *__restrict__ dq) {
-    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / (NW * 64);
+    constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>();
     constexpr int NBUF = (D > 128) ? 1 : 2;
     constexpr int NT = NW * 64, Gp = 1 << GSHIFT, QBW = (NW * 32) >> GSHIFT;
+    constexpr int CH = 32 * CPR, LOADS = (CH + NT - 1) / NT;   // 16-byte chunks per matrix; per thread (head_dim 96: not all threads)
+    static_assert(CH % 64 == 0, "whole waves stage or do not");
     __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][2][TILE_B];
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
@@ -769,7 +773,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     const float scale_log2 = scale * LOG2E_F;
     u32x4 kst[2][LOADS], vst[2][LOADS];
 #define DQ_LOAD(SET, TILE)                                                                          \
-    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) if (CH % NT == 0 || i * NT + tid < CH) {     \
         const int c = i * NT + tid;                                                               \
         const int row = c / CPR, ch = c % CPR;                                                     \
         const int64_t off = ((int64_t)(s0 + min((TILE) * 32 + row, L - 1)) * Hkv + kvh) * D + ch * 8; \
@@ -798,7 +802,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     uint32_t word_next = HAS_IDX ? wrow[0] : 0u;        // unconditional loads; rows that are not live are masked at use
 
 #define DQ_STORE(SET, BUF, TILE)                                                                         \
-    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) if (CH % NT == 0 || i * NT + tid < CH) {     \
         const int c = i * NT + tid;                                                               \
         const int row = c / CPR, ch = c % CPR;                                                     \
         *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(row, ch)]) = kst[SET][i];              \
@@ -1519,12 +1523,13 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
     bf16_t *__restrict__ dv) {
     static_assert(D <= 128, "head_dim 256 runs dsa_tile_dkvpc_kernel");
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>();
-    constexpr int NCHUNK = 32 * CPR, STG = 256, CPT = NCHUNK / STG;
+    constexpr int NCHUNK = 32 * CPR, STG = 256, CPT = (NCHUNK + STG - 1) / STG;
+    constexpr bool ALL_STAGE = NCHUNK % STG == 0;        // (head_dim 96: the last chunk of half of the staging threads is spare)
     constexpr int Gp = 1 << GSHIFT, QB = 32 >> GSHIFT;
     constexpr int QD_SLOT = 2 * TILE_B;                  // q block | dO block
     constexpr int P_GROUP = 2 * 1024, P_SLOT = 4 * P_GROUP;   // per key group: P rows 0-15 | 16-31, 64 lanes x 16 B each
     constexpr int AUX_SLOT = (32 + 32 + 4 * 32) * 4;     // lse | delta | selection words [key group][query]
-    static_assert(CPT >= 1 && NCHUNK % STG == 0, "every staging thread stages whole chunks");
+    static_assert(CPT >= 1 && NCHUNK % 64 == 0, "whole waves stage a chunk or do not");
     extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
     unsigned char *const qd_ring = dyn_lds;                          // 4 slots
     unsigned char *const p_ring = dyn_lds + 4 * QD_SLOT;             // 2 slots
@@ -1573,10 +1578,11 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
     const unsigned char *qp[CPT], *dp[CPT];
     int64_t dlast[CPT];
     int lds_off[CPT];
-    bool row_dead_last[CPT], head_ok[CPT];
+    bool row_dead_last[CPT], head_ok[CPT], staged[CPT];
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
-        const int c = i * STG + ctid, srow = c / CPR, sch = c % CPR;
+        staged[i] = ALL_STAGE || i * STG + ctid < NCHUNK; // a spare chunk loads the tile's last chunk again and stores nothing
+        const int c = min(i * STG + ctid, NCHUNK - 1), srow = c / CPR, sch = c % CPR;
         const int hd = min(srow & (Gp - 1), G - 1);
         const int qr = srow >> GSHIFT;
         const int over = max(q0 + last * QB + qr - (Lq - 1), 0);     // rows past the end in the last block
@@ -1650,8 +1656,10 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
         for (int i = 0; i < CPT; ++i) {
             const bool live = head_ok[i] && !(b > last || (b == 0 && row_dead_last[i]));
             const u32x4 z4 = {0u, 0u, 0u, 0u};
-            *reinterpret_cast<u32x4 *>(slot + lds_off[i]) = live ? qst[i] : z4;
-            *reinterpret_cast<u32x4 *>(slot + TILE_B + lds_off[i]) = live ? dost[i] : z4;
+            if (ALL_STAGE || staged[i]) {
+                *reinterpret_cast<u32x4 *>(slot + lds_off[i]) = live ? qst[i] : z4;
+                *reinterpret_cast<u32x4 *>(slot + TILE_B + lds_off[i]) = live ? dost[i] : z4;
+            }
         }
         const bool word_dead = aux_is_word && (b > last || (b == 0 && aux_over > 0));
         *reinterpret_cast<uint32_t *>(aux_ring + (aux_lds < 4 * AUX_SLOT ? (b & 3) * AUX_SLOT : 0) + aux_lds) =
@@ -1672,10 +1680,11 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
     auto lstore_steady = [&](int b, const u32x4 (&qst)[CPT], const u32x4 (&dost)[CPT], uint32_t aux_st) __attribute__((always_inline)) {
         unsigned char *slot = qd_ring + (b & 3) * QD_SLOT;
 #pragma unroll
-        for (int i = 0; i < CPT; ++i) {
-            *reinterpret_cast<u32x4 *>(slot + lds_off[i]) = qst[i];
-            *reinterpret_cast<u32x4 *>(slot + TILE_B + lds_off[i]) = dost[i];
-        }
+        for (int i = 0; i < CPT; ++i)
+            if (ALL_STAGE || staged[i]) {
+                *reinterpret_cast<u32x4 *>(slot + lds_off[i]) = qst[i];
+                *reinterpret_cast<u32x4 *>(slot + TILE_B + lds_off[i]) = dost[i];
+            }
         *reinterpret_cast<uint32_t *>(aux_ring + (aux_lds < 4 * AUX_SLOT ? (b & 3) * AUX_SLOT : 0) + aux_lds) = aux_value(aux_st);
     };
     if (wv >= 4) {
@@ -1735,10 +1744,9 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
                     dkacc[m - DT] = mfma32(t[m & 3], __builtin_bit_cast(bf16x8, d1), dkacc[m - DT]);
                 }
                 if (m + 3 < 2 * DT) t[(m + 3) & 3] = lo.trop(qt, (m + 3) / DT, (m + 3) % DT);
-                if (m < DT) {                            // 4 / DT pairs of the second half of dS behind this MFMA
+                if (m < DT) {                            // the four pairs of the second half of dS, spread behind these MFMAs
 #pragma unroll
-                    for (int u = 0; u < 4 / DT; ++u) {
-                        const int e = m * (4 / DT) + u;
+                    for (int e = 4 * m / DT; e < 4 * (m + 1) / DT; ++e) {
                         dw[e] = pack2bf(__uint_as_float(w1[e] << 16) * pacc[8 + 2 * e], __uint_as_float(w1[e] & 0xffff0000u) * pacc[9 + 2 * e]);
                         asm volatile("" : "+v"(dw[e]));
                     }
@@ -1857,7 +1865,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
     bf16x8 pq0 = zero_bf16x8(), pq1 = zero_bf16x8();     // P of the block before, as B operands (rows 0-15 | 16-31)
     auto step = [&](auto may_diag, auto has_cur, auto has_prev, int s) __attribute__((always_inline)) {
         constexpr bool CUR = decltype(has_cur)::value, PREV = decltype(has_prev)::value;
-        constexpr int NM = 2 * DT, EPM = 16 / NM;
+        constexpr int NM = 2 * DT;                       // elements 16 m / NM .. 16 (m + 1) / NM behind MFMA m
         const unsigned char *qt = qd_ring + (s & 3) * QD_SLOT, *dprev = qd_ring + ((s - 1) & 3) * QD_SLOT + TILE_B;
         f32x16 sacc;
         if (CUR) {
@@ -1882,8 +1890,7 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
             }
             if (CUR) {
 #pragma unroll
-                for (int u = 0; u < EPM; ++u) {          // P is packed pair by pair as it is formed
-                    const int vi = m * EPM + u;
+                for (int vi = 16 * m / NM; vi < 16 * (m + 1) / NM; ++vi) {   // P is packed pair by pair as it is formed
                     pv[vi & 1] = element(may_diag, s, vi, sacc, sl2, keep, pm);
                     if (vi & 1) {
                         pw[vi >> 1] = pack2bf(pv[0], pv[1]);
@@ -1957,8 +1964,8 @@ static inline int group_shift(int Hq, int Hkv) {
 #ifndef DSA_TILE_WAVES_128
 #define DSA_TILE_WAVES_128 8
 #endif
-template <int D> constexpr int tile_waves() { return D == 128 ? DSA_TILE_WAVES_128 : 4; }
-static inline int tile_waves_of(int D) { return D == 128 ? DSA_TILE_WAVES_128 : 4; }
+template <int D> constexpr int tile_waves() { return (D == 128 || D == 96) ? DSA_TILE_WAVES_128 : 4; }
+static inline int tile_waves_of(int D) { return (D == 128 || D == 96) ? DSA_TILE_WAVES_128 : 4; }
 template <int D, bool HAS_IDX, int GS>
 static hipError_t launch_fwd_i(dim3 grid, hipStream_t stream, const void *q, const void *k, const void *v,
                          const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T, int Hq, int Hkv, float sl2,
@@ -2021,12 +2028,24 @@ static hipError_t launch_dkv_i(dim3 grid, hipStream_t stream, const void *dout, 
     }                                                                                     \
     if (launch_status != hipSuccess) return launch_status;
 
+// the same with head_dim 96 (dense only: no selection bitmap), for the three attention kernels
+#define TILE_SWITCH_96(FN, ...)                                                           \
+    hipError_t launch_status = hipSuccess;                                                \
+    switch (D) {                                                                          \
+        case 64: if (bitmap) { GS_SWITCH(FN, 64, true, __VA_ARGS__) } else { GS_SWITCH(FN, 64, false, __VA_ARGS__) } break;    \
+        case 96: if (bitmap) return hipErrorInvalidValue; GS_SWITCH(FN, 96, false, __VA_ARGS__) break;                         \
+        case 128: if (bitmap) { GS_SWITCH(FN, 128, true, __VA_ARGS__) } else { GS_SWITCH(FN, 128, false, __VA_ARGS__) } break; \
+        case 256: if (bitmap) { GS_SWITCH(FN, 256, true, __VA_ARGS__) } else { GS_SWITCH(FN, 256, false, __VA_ARGS__) } break; \
+        default: return hipErrorInvalidValue;                                             \
+    }                                                                                     \
+    if (launch_status != hipSuccess) return launch_status;
+
 extern "C" hipError_t dsa_launch_tile_fwd(const void *q, const void *k, const void *v, const uint32_t *bitmap, int ldw,
                                           const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale,
                                           int pos_split, int causal, void *out, float *lse, hipStream_t stream) {
     const int gs = group_shift(Hq, Hkv);
     const dim3 grid((unsigned)(((int64_t)T / ((32 * tile_waves_of(D)) >> gs) + N + 1) * Hkv));
-    TILE_SWITCH(launch_fwd_i, grid, stream, q, k, v, bitmap, ldw, cu, N, T, Hq, Hkv, scale * LOG2E_F, pos_split, causal, out, lse)
+    TILE_SWITCH_96(launch_fwd_i, grid, stream, q, k, v, bitmap, ldw, cu, N, T, Hq, Hkv, scale * LOG2E_F, pos_split, causal, out, lse)
     return hipGetLastError();
 }
 template <int D, bool HAS_IDX, int GS>
@@ -2093,7 +2112,7 @@ extern "C" hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const 
                                          int pos_split, int causal, void *dq, hipStream_t stream) {
     const int gs = group_shift(Hq, Hkv);
     const dim3 grid((unsigned)(((int64_t)T / ((32 * tile_waves_of(D)) >> gs) + N + 1) * Hkv));
-    TILE_SWITCH(launch_dq_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, pos_split, causal, dq)
+    TILE_SWITCH_96(launch_dq_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, pos_split, causal, dq)
     return hipGetLastError();
 }
 // bytes of fp32 partial sums a launch of T tokens may use for key-tile walks in pieces (0: launches of this size are
@@ -2129,7 +2148,7 @@ extern "C" hipError_t dsa_launch_tile_dkv(const void *dout, const void *q, const
         order = nullptr;                                 // one segment: its tiles are in order already
     }
     if (!pieces) partial = nullptr;
-    TILE_SWITCH(launch_dkv_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, causal, order, partial, dk, dv)
+    TILE_SWITCH_96(launch_dkv_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, causal, order, partial, dk, dv)
     if (pieces)
         hipLaunchKernelGGL(dsa_dkv_pieces_reduce_kernel, dim3(tiles_ub, Hkv, DSA_PIECES_Z), dim3(256), 0, stream, order,
                            order_entries_cap(T), partial, cu, N, Hkv, D, 32 >> gs, bitmap ? ldw * 32 : 0x7fffffff, scale,

@@ -57,6 +57,7 @@ def _check_cu(cu_seqlens: torch.Tensor, T: int, max_seqlen: Optional[int] = None
 
 
 _KERNEL_HEAD_DIMS = (64, 128, 256)                   # head_dim instantiations of the tile and gather kernels
+_KERNEL_HEAD_DIMS_DENSE = (64, 96, 128, 256)         # without a key selection the tile kernels also come at head_dim 96
 
 
 def _check_qkv(q, k, v):
@@ -451,7 +452,8 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, in
                 idx, n = index_topk(indexer_q, indexer_k, indexer_w, cu, int(max_seqlen), int(top_k), index_scale)
     elif return_indices or return_scores:
         raise ValueError("return_indices / return_scores need the indexer inputs")
-    d_kernel = next((d for d in _KERNEL_HEAD_DIMS if d >= D), None)
+    dims = _KERNEL_HEAD_DIMS if sparse else _KERNEL_HEAD_DIMS_DENSE
+    d_kernel = next((d for d in dims if d >= D), None)
     if d_kernel is None:
         raise ValueError(f"head_dim {D} is beyond the kernels' largest ({_KERNEL_HEAD_DIMS[-1]})")
     if d_kernel != D:
