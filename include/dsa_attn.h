@@ -129,6 +129,8 @@ size_t dsa_indexer_bwd_workspace_bytes(int T, int Di, int max_seqlen);
  * q head h reads kv head h / (Hq/Hkv) (models/qwen3/model.py:125-129).  softmax in fp32.
  * causal == 0 (only with idx == NULL) attends every key of the own segment: the vision towers' call,
  * varlen_attn(..., window_size=(-1,-1)) (models/qwen3_vl/model.py:423-428, models/qwen3_5/model.py:388-393).
+ * head_dim D: 64, 128 or 256; with idx == NULL also 96 (forward and backward), which the 72-wide heads of the
+ * 1152 / 16 vision towers are padded to.
  */
 int dsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
                  const int32_t *cu_seqlens, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
