@@ -199,6 +199,22 @@ int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k, const voi
                        void *dq, void *dk, void *dv, void *ws, size_t ws_bytes, int parts, void *stream);
 
 /*
+ * dsa_attn_bwd for a caller that kept the forward's workspace (an autograd node: torch's varlen_attn saves its
+ * tensors between forward and backward the same way, torch/nn/attention/varlen.py:206-214).  `fwd_ws` is the
+ * workspace a dsa_attn_fwd call with the same idx, n, cu_seqlens and max_seqlen filled (the inverted selection
+ * bitmap; ignored when idx == NULL); it is only read.  `scratch` holds dsa_attn_bwd_scratch_bytes() bytes that
+ * nothing outlives: delta, the launch order of the key tiles and - only for launches of at most 1024 key-tile
+ * workgroups, which may be cut into pieces - fp32 partial sums (at most 128 MiB).  So between forward and backward
+ * a layer holds the bitmap alone.  Refused (DSA_ERR_ARG) while the tile crossover is 0: that forward builds no bitmap.
+ */
+size_t dsa_attn_bwd_scratch_bytes(int T, int N, int Hq, int Hkv, int D);
+int dsa_attn_bwd_saved_bitmap(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                              const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu_seqlens, int T,
+                              int N, int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen,
+                              int causal, void *dq, void *dk, void *dv, const void *fwd_ws, size_t fwd_ws_bytes,
+                              void *scratch, size_t scratch_bytes, void *stream);
+
+/*
  * Dense causal / non-causal packed attention, the operator the reference itself calls
  * (torch.nn.attention.varlen.varlen_attn: train/model_attention.py:123-132, models/qwen3_vl/model.py:41-46,
  * models/qwen3_5/model.py:93-98).  Same as dsa_attn_fwd / dsa_attn_bwd with idx == n == NULL and K == 0;

@@ -27,6 +27,7 @@ Pinning status (what independent check fixes each function; see tests/test_oracl
 * ``selected_scores``        - a gather of the pinned ``indexer_scores_segment``; checked entry by entry in Python.
 * ``indexer_kl``             - ``torch.nn.functional.kl_div`` (library routine) on rows without padding, and
   ``softmax - mass`` for its gradient.
+* ``sparse_attention_key_rows`` - autograd of ``sparse_attention`` (dk, dv of every key row of a small packed batch).
 * ``attention_mass``         - pure-Python loop on a tiny case; rows sum to one; with one kv head the
   mass-weighted sum of the selected value rows equals the head mean of ``sparse_attention``'s output.
 
@@ -334,6 +335,57 @@ def sparse_attention_grads(q, k, v, idx, n, cu_seqlens, dout, softmax_scale: Opt
     out = sparse_attention(qf, kf, vf, idx, n, cu_seqlens, softmax_scale)
     dq, dk, dv = torch.autograd.grad(out, (qf, kf, vf), dout.float())
     return out.detach(), dq, dk, dv
+
+
+def sparse_attention_key_rows(q, k, v, dout, idx, n, keys, softmax_scale: Optional[float] = None, batch: int = 32):
+    """dK and dV of the key rows ``keys`` only -> (dk (len(keys),Hkv,D), dv (len(keys),Hkv,D)), fp32.
+
+    Key-stationary restatement of the D4 gradients, written from the formulas and not through autograd: the queries
+    that selected key ``s`` are looked up in ``idx``; each of them is attended over its own selected keys (a gather, as
+    in ``sparse_attention_rows``) for its softmax and for ``delta = sum_j p_j dP_j``; then
+        dV[s] = sum_t sum_h p[t,h,s] dO[t,h]          dK[s] = scale * sum_t sum_h p[t,h,s] (dP[t,h,s] - delta[t,h]) q[t,h]
+    over the heads ``h`` of the key's kv head.  Costs n[t] keys per contributing query whatever the segment length, so
+    single key rows of a very long sequence can be checked.  Pinned against autograd of ``sparse_attention``.
+    """
+    T, Hq, D = q.shape
+    Hkv = k.shape[1]
+    G = Hq // Hkv
+    scale = softmax_scale if softmax_scale is not None else D ** -0.5
+    keys = [int(s) for s in keys]
+    key_t = torch.tensor(keys, dtype=idx.dtype)
+    hit = torch.zeros(T, dtype=torch.bool)
+    for c0 in range(0, T, 8192):                                        # which queries selected any of the keys
+        hit[c0:c0 + 8192] = torch.isin(idx[c0:c0 + 8192], key_t).any(dim=1)
+    rows = torch.nonzero(hit).flatten()
+    dk = torch.zeros(len(keys), Hkv, D)
+    dv = torch.zeros(len(keys), Hkv, D)
+    kh, vh = k.transpose(0, 1).contiguous(), v.transpose(0, 1).contiguous()        # (Hkv,T,D): one gather per kv head
+    for b0 in range(0, rows.numel(), batch):
+        r = rows[b0:b0 + batch]
+        R = r.numel()
+        sel = idx[r].long()                                             # (R,K), -1 padded
+        ok = sel >= 0
+        safe = sel.clamp(min=0).flatten()
+        qr = q[r].float().view(R, Hkv, G, D)
+        gr = dout[r].float().view(R, Hkv, G, D)
+        at = sel[:, :, None] == torch.tensor(keys)[None, None, :]       # (R,K,len(keys)): at most one slot per (row, key)
+        has = at.any(dim=1)                                             # (R,len(keys))
+        slot = at.float().argmax(dim=1)                                 # (R,len(keys)): the slot, 0 where absent
+        for h in range(Hkv):
+            kg = kh[h][safe].float().view(R, -1, D)                     # (R,K,D)
+            vg = vh[h][safe].float().view(R, -1, D)
+            logits = torch.bmm(qr[:, h], kg.transpose(1, 2)) * scale    # (R,G,K)
+            logits = logits.masked_fill(~ok[:, None, :], float("-inf"))
+            p = torch.softmax(logits, dim=-1)
+            dP = torch.bmm(gr[:, h], vg.transpose(1, 2))
+            delta = (p * dP).sum(-1, keepdim=True)
+            dS = p * (dP - delta)
+            pick = slot[:, None, :].expand(R, G, len(keys))
+            w_p = p.gather(2, pick) * has[:, None, :]                   # (R,G,len(keys)): p[t,h,s], 0 where t did not select s
+            w_s = dS.gather(2, pick) * has[:, None, :]
+            dv[:, h] += torch.einsum("rgj,rgd->jd", w_p, gr[:, h])
+            dk[:, h] += torch.einsum("rgj,rgd->jd", w_s, qr[:, h]) * scale
+    return dk, dv
 
 
 # ----------------------------------------------------------------------------------------------

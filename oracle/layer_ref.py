@@ -59,7 +59,7 @@ def qwen3_5_attention(x, wq, wk, wv, wo, qn_w, kn_w, cos, sin, cu_seqlens, head_
 
 
 def dsa_layer(x, wq, wk, wv, wo, qn_w, kn_w, cos, sin, cu_seqlens, head_dim, wiq, wik, wiw, index_heads, index_dim, idx, n,
-              eps=1e-6, gated=False, index_scale=None):
+              eps=1e-6, gated=False, index_scale=None, round_indexer_to_bf16=False):
     """(layer output, indexer KL loss) for the selection ``idx, n``: attention over the selected keys, and
     mean_t KL(attention mass of the selected keys || softmax of the indexer's scores of the selected keys).  The mass is
     detached and the indexer reads a detached input, as in the layer under test."""
@@ -74,6 +74,11 @@ def dsa_layer(x, wq, wk, wv, wo, qn_w, kn_w, cos, sin, cu_seqlens, head_dim, wiq
     iq = F.linear(h, wiq.float()).view(T, index_heads, index_dim)
     ik = F.linear(h, wik.float())
     iw = F.linear(h, wiw.float())
+    if round_indexer_to_bf16:
+        # The layer under test hands the indexer kernels bf16 projections.  The indexer's gradient passes the gate
+        # [q_idx.k_idx > 0], a step function: to compare gradients the checker must open the same gates, i.e. see the
+        # same rounded values (straight-through: the rounding itself passes the gradient unchanged).
+        iq, ik, iw = (t + (t.to(torch.bfloat16).float() - t).detach() for t in (iq, ik, iw))
     mass = R.attention_mass(q.detach(), k.detach(), idx, n, cu_seqlens)
     sel = R.selected_scores(iq, ik, iw, idx, n, cu_seqlens, index_scale)
     return y, R.indexer_kl(sel, mass, n).mean(), (iq, ik, iw)

@@ -133,3 +133,13 @@ def test_integration_stub_matches_the_header():
         depth -= ch in ")]"
         nargs += ch == "," and depth == 0
     assert nargs == len(stub) == 21
+
+
+def test_integration_notes_name_every_exported_symbol():
+    doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    named = set(re.findall(r"`(dsa_[a-z0-9_]+)`", doc))
+    missing = [name for name in _lib.EXPORTS if name not in named]
+    assert not missing, missing
+    unknown = [name for name in named if name.startswith("dsa_") and name not in _lib.EXPORTS
+               and not name.startswith(("dsa_attn.h", "dsa_varlen_attn", "dsa_ref"))]
+    assert not unknown, unknown

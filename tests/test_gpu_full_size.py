@@ -113,7 +113,7 @@ def test_long_single_sequence_by_invariants_and_sampled_rows():
     """C4 as benchmarked (one causal sequence of 131 072 tokens, top-k 2048): the chunked score/select loop over 64
     chunks, the gather kernels at long range, bitmap rows of 4096 words.  Checked by statements that hold at any size
     (as for the headline configuration), and on sampled query rows against the oracle: selection bit-exact on the
-    GPU's own scores of that row, out and dq within tolerance."""
+    GPU's own scores of that row, out and dq of sampled query rows and dk, dv of sampled key rows within tolerance."""
     _log("C4 full size")
     w = W.C4
     lib = _lib.load()
@@ -168,6 +168,13 @@ def test_long_single_sequence_by_invariants_and_sampled_rows():
     e1 = assert_close_bf16(out[rows], ref.detach(), "out (sampled rows)")
     e2 = assert_close_bf16(dq[rows], qc.grad[rows], "dq (sampled rows)")
     _log(f"  C4 sampled rows: out ({e1[0]:.2e},{e1[1]:.6f}) dq ({e2[0]:.2e},{e2[1]:.6f})")
+    # dk and dv of sampled key rows (first key tile, around top_k, around the select cache and the tile/gather crossover,
+    # the last tile): every query that selected the key is looked up in idx and attended over its own keys by the oracle
+    keys = [17, K, 8192, 16 * K, 100003, T - 70, T - 1]
+    want_dk, want_dv = R.sparse_attention_key_rows(t["q"].cpu(), t["k"].cpu(), t["v"].cpu(), t["dout"].cpu(), idx_c, n_c, keys)
+    e3 = assert_close_bf16(dk[keys], want_dk, "dk (sampled key rows)")
+    e4 = assert_close_bf16(dv[keys], want_dv, "dv (sampled key rows)")
+    _log(f"  C4 sampled key rows: dk ({e3[0]:.2e},{e3[1]:.6f}) dv ({e4[0]:.2e},{e4[1]:.6f})")
     # a second run is bit-identical
     q2, k2, v2 = (t[x].clone().requires_grad_(True) for x in ("q", "k", "v"))
     out2, idx2, _ = ops.dsa_varlen_attn(q2, k2, v2, cu, w.max_seqlen, indexer_q=t["q_idx"], indexer_k=t["k_idx"],

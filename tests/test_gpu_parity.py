@@ -512,6 +512,40 @@ def test_argument_errors_cross_the_boundary_as_exceptions(monkeypatch):
                        torch.zeros(8, 2, dtype=torch.bfloat16, device=DEV), cu, 8, 2)
 
 
+def test_debug_switch_checks_the_segment_table_before_any_launch(monkeypatch):
+    """DSA_DEBUG_META=1 copies cu_seqlens to the host and refuses a table that does not end at T, that decreases, or
+    whose longest segment exceeds max_seqlen (the kernels would clip such a segment without a word).  Without the
+    switch nothing is copied and the same calls go through."""
+    q = torch.zeros(64, 4, 64, dtype=torch.bfloat16, device=DEV)
+    k = torch.zeros(64, 2, 64, dtype=torch.bfloat16, device=DEV)
+    qi = torch.zeros(64, 2, 32, dtype=torch.bfloat16, device=DEV)
+    ki = torch.zeros(64, 32, dtype=torch.bfloat16, device=DEV)
+    wi = torch.zeros(64, 2, dtype=torch.bfloat16, device=DEV)
+    good = torch.tensor([0, 40, 64], dtype=torch.int32, device=DEV)
+    short = torch.tensor([0, 40, 60], dtype=torch.int32, device=DEV)
+    back = torch.tensor([0, 50, 40, 64], dtype=torch.int32, device=DEV)
+    monkeypatch.setenv("DSA_DEBUG_META", "1")
+    launched = []
+    real = ops._lib.load
+
+    def counting():
+        launched.append(1)
+        return real()
+
+    monkeypatch.setattr(ops._lib, "load", counting)
+    for cu, bound, what in ((short, 64, "end at T"), (back, 64, "non-decreasing"), (good, 32, "below the longest segment")):
+        with pytest.raises(ValueError, match=what):
+            ops.dsa_varlen_attn(q, k, k, cu, bound)
+        with pytest.raises(ValueError, match=what):
+            ops.dsa_varlen_attn(q, k, k, cu, bound, indexer_q=qi, indexer_k=ki, indexer_w=wi, top_k=8)
+    with pytest.raises(ValueError, match="below the longest segment"):
+        ops.index_topk(qi, ki, wi, good, 39, 8)
+    assert not launched                                          # every refusal came before the library was touched
+    assert ops.dsa_varlen_attn(q, k, k, good, 40).shape == q.shape and launched
+    monkeypatch.delenv("DSA_DEBUG_META")
+    assert ops.dsa_varlen_attn(q, k, k, good, 64).shape == q.shape
+
+
 # ------------------------------------------------------------------------------------------ golden fixtures
 def _golden(name):
     import os

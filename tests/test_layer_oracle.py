@@ -150,3 +150,54 @@ def test_installer_replaces_the_hf_forwards_and_masks_and_can_be_undone():
         for owner, attr, old in reversed(undo):
             setattr(owner, attr, old)
     assert mods["transformers.models.qwen3.modeling_qwen3"].Qwen3Attention.forward is not M.qwen3vl_forward
+
+
+def test_installer_patches_nothing_when_a_target_is_missing(monkeypatch):
+    """A transformers build without one of the four models must leave the others as they were."""
+    import importlib
+
+    import vlm_training_amd.model_attention as MA
+    qwen3 = importlib.import_module("transformers.models.qwen3.modeling_qwen3")
+    before = qwen3.Qwen3Attention.forward
+    real_import = importlib.import_module
+
+    def failing(name, *a, **k):
+        if name.endswith("modeling_qwen3_5"):
+            raise ImportError("no qwen3_5 in this build")
+        return real_import(name, *a, **k)
+
+    monkeypatch.setattr(importlib, "import_module", failing)
+    with pytest.raises(ImportError):
+        MA.replace_attention_qwenvl()
+    assert qwen3.Qwen3Attention.forward is before and qwen3.create_causal_mask is not MA.return_mask
+
+
+# ------------------------------------------------------------------------------------------ longest segment
+def test_longest_segment_follows_the_tensor_not_its_address():
+    """train/model_attention.py:118-121 always uses the true maximum.  A new offsets tensor that lands on a freed
+    tensor's address (what the caching allocator does every step) must get its own bound; views of one tensor share
+    one read; an in-place write invalidates it."""
+    from vlm_training_amd.model_attention import _BOUND_ATTR, longest_segment
+    import numpy as np
+    buf = np.array([0, 100, 260, 300], dtype=np.int32)                   # one block of memory, two tensors in turn
+    a = torch.from_numpy(buf)
+    ptr = a.data_ptr()
+    assert longest_segment(a) == 160
+    del a
+    buf[1] = 200                                                         # "the next step's offsets" at the same address
+    b = torch.from_numpy(buf)
+    assert b.data_ptr() == ptr and b._version == 0 and b.numel() == 4    # what an address-keyed cache cannot tell apart
+    assert longest_segment(b) == 200
+    del b
+    c = torch.tensor([0, 7, 9, 30], dtype=torch.int32)
+    assert longest_segment(c) == 21 and getattr(c, _BOUND_ATTR)[3] == 21
+    masked = c.unsqueeze_(0)                                            # what return_mask does: same object, version + 1
+    assert masked is c and longest_segment(c.reshape(-1)) == 21 and longest_segment(c.squeeze()) == 21
+    c[0, 1] = 1                                                          # in-place writes bump the version
+    c[0, 2] = 2                                                          # [0,1,2,30] -> 28
+    assert longest_segment(c.reshape(-1)) == 28
+    assert longest_segment(torch.tensor([0], dtype=torch.int32)) == 1
+    assert longest_segment(torch.tensor([0, 0, 0], dtype=torch.int32)) == 1
+    # two separately built tensors with equal contents never share an entry
+    d, e = torch.tensor([0, 4, 6], dtype=torch.int32), torch.tensor([0, 4, 6], dtype=torch.int32)
+    assert longest_segment(d) == 4 and not hasattr(e, _BOUND_ATTR) and longest_segment(e) == 4

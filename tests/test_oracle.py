@@ -235,6 +235,24 @@ def test_row_wise_gather_form_matches_bruteforce_and_the_masked_form():
     assert torch.allclose(q1.grad, q2.grad, atol=1e-5)
 
 
+def test_key_row_gradients_match_autograd_of_the_masked_form():
+    """sparse_attention_key_rows (dk, dv of single key rows from the formulas) against autograd of sparse_attention:
+    every key row of a packed batch, including keys nobody selected (zero rows), and batches smaller than the
+    contributor count."""
+    for seed, top_k in ((26, 4), (27, 1), (28, 50)):
+        t = _toy(seed=seed)
+        _, idx, n = R.dsa_varlen_attn_ref(t["q"], t["k"], t["v"], t["cu"], t["q_idx"], t["k_idx"], t["w"], top_k,
+                                          return_indices=True)
+        g = rnd(t["cu"][-1], 4, 8, seed=seed + 50)
+        _, _, dk, dv = R.sparse_attention_grads(t["q"], t["k"], t["v"], idx, n, t["cu"], g)
+        keys = list(range(t["cu"][-1]))
+        got_dk, got_dv = R.sparse_attention_key_rows(t["q"], t["k"], t["v"], g, idx, n, keys, batch=5)
+        assert torch.allclose(got_dk, dk, atol=1e-5) and torch.allclose(got_dv, dv, atol=1e-5)
+        some = [36, 0, 12]
+        got_dk, got_dv = R.sparse_attention_key_rows(t["q"], t["k"], t["v"], g, idx, n, some)
+        assert torch.allclose(got_dk, dk[some], atol=1e-5) and torch.allclose(got_dv, dv[some], atol=1e-5)
+
+
 def test_k_at_least_longest_segment_equals_dense():
     t = _toy(seed=30)
     dense = R.dense_varlen_causal(t["q"], t["k"], t["v"], t["cu"])

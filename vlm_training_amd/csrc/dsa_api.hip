@@ -1,5 +1,6 @@
 // C ABI of the library (declared in include/dsa_attn.h): argument checks, workspace layout, launches.
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <mutex>
 #include <stdarg.h>
 #include <stdio.h>
@@ -250,18 +251,18 @@ static inline int bitmap_ldw(int max_seqlen) { return (max_seqlen + 31) / 32; }
 // Query rows whose position in their segment is below top_k * crossover are handled by the tile
 // kernels (their selection covers more than 1/crossover of the causal window), the rest by the
 // gather kernels.  Process-wide tuning knob; 0 = gather only, a huge value = tile only.
-static int g_tile_crossover = 16;
+static std::atomic<int> g_tile_crossover{16};          // read on every launch, possibly from several host threads
 extern "C" int dsa_set_tile_crossover(int crossover) {
     if (crossover < 0) return fail(DSA_ERR_ARG, "crossover=%d must be >= 0", crossover);
-    g_tile_crossover = crossover;
+    g_tile_crossover.store(crossover, std::memory_order_relaxed);
     return DSA_OK;
 }
-extern "C" int dsa_get_tile_crossover(void) { return g_tile_crossover; }
+extern "C" int dsa_get_tile_crossover(void) { return g_tile_crossover.load(std::memory_order_relaxed); }
 
 // first query position handled by the gather kernels (multiple of 128, the coarsest tile block)
 static int pos_split_for(const int32_t *idx, int K) {
     if (!idx) return INT32_MAX;                       // dense causal: tiles everywhere
-    const int64_t p = (int64_t)K * g_tile_crossover;
+    const int64_t p = (int64_t)K * g_tile_crossover.load(std::memory_order_relaxed);
     if (p >= INT32_MAX - 256) return INT32_MAX;
     return (int)((p + 255) / 256 * 256);          // a multiple of every tile kernel's query block
 }
@@ -380,27 +381,14 @@ extern "C" size_t dsa_attn_bwd_bitmap_offset(int T, int Hq) {
     return align_up((size_t)T * Hq * 4, 256);
 }
 
-extern "C" int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k, const void *v, const void *out,
-                                  const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu, int T,
-                                  int N, int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen,
-                                  int causal, void *dq, void *dk, void *dv, void *ws, size_t ws_bytes, int parts,
-                                  void *stream) {
-    if (int rc = check_attn(T, N, cu, Hq, Hkv, D, K, dtype, idx, n)) return rc;
-    if (!causal && idx) return fail(DSA_ERR_ARG, "a key selection (idx) implies causal attention");
-    if (!dout || !q || !k || !v || !out || !lse || !dq || !dk || !dv) return fail(DSA_ERR_ARG, "null tensor pointer");
-    if (max_seqlen < 1 || max_seqlen > (T > 0 ? T : 1)) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
-    if (T == 0) return DSA_OK;
-    const size_t need = dsa_attn_bwd_workspace_bytes(T, Hq, max_seqlen, idx != nullptr);
-    if (!ws || ws_bytes < need) return fail(DSA_ERR_WORKSPACE, "backward workspace: have %zu bytes, need %zu", ws_bytes, need);
+// the backward proper: every buffer named, so that the two entry points below differ only in where the buffers live
+static int attn_bwd_run(const void *dout, const void *q, const void *k, const void *v, const void *out, const float *lse,
+                        const int32_t *idx, const int32_t *n, const int32_t *cu, int T, int N, int Hq, int Hkv, int D, int K,
+                        float softmax_scale, int max_seqlen, int causal, void *dq, void *dk, void *dv, float *delta,
+                        uint32_t *bitmap, float *partial, size_t partial_bytes, int32_t *order, int parts, hipStream_t st) {
     const int ldw = bitmap_ldw(max_seqlen);
     if (idx && (size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);
-    float *delta = (float *)ws;
-    uint32_t *bitmap = idx ? (uint32_t *)((char *)ws + dsa_attn_bwd_bitmap_offset(T, Hq)) : nullptr;
-    int32_t *order = (int32_t *)((char *)ws + need - align_up(dsa_tile_order_bytes(T), 256));
-    const size_t partial_bytes = dsa_tile_dkv_partial_bytes(T);
-    float *partial = partial_bytes ? (float *)((char *)order - align_up(partial_bytes, 256)) : nullptr;
     const int split = pos_split_for(idx, K);
-    hipStream_t st = (hipStream_t)stream;
     hipError_t e = hipSuccess;
     if (parts & DSA_BWD_DELTA) {
         e = dsa_launch_delta(dout, out, T, Hq, D, delta, st);
@@ -426,6 +414,71 @@ extern "C" int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k
         if (e != hipSuccess) return hip_fail(e, "tile dkv launch");
     }
     return DSA_OK;
+}
+
+static int check_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out, const float *lse,
+                     const int32_t *idx, const int32_t *n, const int32_t *cu, int T, int N, int Hq, int Hkv, int D, int K,
+                     int dtype, int max_seqlen, int causal, const void *dq, const void *dk, const void *dv) {
+    if (int rc = check_attn(T, N, cu, Hq, Hkv, D, K, dtype, idx, n)) return rc;
+    if (!causal && idx) return fail(DSA_ERR_ARG, "a key selection (idx) implies causal attention");
+    if (!dout || !q || !k || !v || !out || !lse || !dq || !dk || !dv) return fail(DSA_ERR_ARG, "null tensor pointer");
+    if (max_seqlen < 1 || max_seqlen > (T > 0 ? T : 1)) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
+    return DSA_OK;
+}
+
+extern "C" int dsa_attn_bwd_parts(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                                  const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu, int T,
+                                  int N, int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen,
+                                  int causal, void *dq, void *dk, void *dv, void *ws, size_t ws_bytes, int parts,
+                                  void *stream) {
+    if (int rc = check_bwd(dout, q, k, v, out, lse, idx, n, cu, T, N, Hq, Hkv, D, K, dtype, max_seqlen, causal, dq, dk, dv)) return rc;
+    if (T == 0) return DSA_OK;
+    const size_t need = dsa_attn_bwd_workspace_bytes(T, Hq, max_seqlen, idx != nullptr);
+    if (!ws || ws_bytes < need) return fail(DSA_ERR_WORKSPACE, "backward workspace: have %zu bytes, need %zu", ws_bytes, need);
+    float *delta = (float *)ws;
+    uint32_t *bitmap = idx ? (uint32_t *)((char *)ws + dsa_attn_bwd_bitmap_offset(T, Hq)) : nullptr;
+    int32_t *order = (int32_t *)((char *)ws + need - align_up(dsa_tile_order_bytes(T), 256));
+    const size_t partial_bytes = dsa_tile_dkv_partial_bytes(T);
+    float *partial = partial_bytes ? (float *)((char *)order - align_up(partial_bytes, 256)) : nullptr;
+    return attn_bwd_run(dout, q, k, v, out, lse, idx, n, cu, T, N, Hq, Hkv, D, K, softmax_scale, max_seqlen, causal, dq, dk, dv,
+                        delta, bitmap, partial, partial_bytes, order, parts, (hipStream_t)stream);
+}
+
+// Scratch of the backward that nothing outlives: delta, the launch order of the key tiles and - only for launches small
+// enough to be cut into pieces (at most 1024 workgroups before the cut) - the fp32 partial sums of those pieces.
+static size_t bwd_partial_bytes_for(int T, int N, int Hkv, int D) {
+    const int64_t wg_per_tile = (int64_t)Hkv * (D > 128 ? 2 : 1);
+    if (((int64_t)T / 128 + N) * wg_per_tile > 4 * 256) return 0;
+    return dsa_tile_dkv_partial_bytes(T);
+}
+extern "C" size_t dsa_attn_bwd_scratch_bytes(int T, int N, int Hq, int Hkv, int D) {
+    if (T <= 0 || N < 0 || Hq <= 0 || Hkv <= 0) return 0;
+    return align_up((size_t)T * Hq * 4, 256) + align_up(bwd_partial_bytes_for(T, N, Hkv, D), 256) +
+           align_up(dsa_tile_order_bytes(T), 256);
+}
+
+extern "C" int dsa_attn_bwd_saved_bitmap(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                                         const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu, int T,
+                                         int N, int Hq, int Hkv, int D, int K, float softmax_scale, int dtype,
+                                         int max_seqlen, int causal, void *dq, void *dk, void *dv, const void *fwd_ws,
+                                         size_t fwd_ws_bytes, void *scratch, size_t scratch_bytes, void *stream) {
+    if (int rc = check_bwd(dout, q, k, v, out, lse, idx, n, cu, T, N, Hq, Hkv, D, K, dtype, max_seqlen, causal, dq, dk, dv)) return rc;
+    if (T == 0) return DSA_OK;
+    if (idx) {
+        if (pos_split_for(idx, K) <= 0) return fail(DSA_ERR_ARG, "with the tile crossover at 0 the forward builds no bitmap: use dsa_attn_bwd");
+        const size_t have = dsa_attn_fwd_workspace_bytes(T, max_seqlen, 1);
+        if (!fwd_ws || fwd_ws_bytes < have) return fail(DSA_ERR_WORKSPACE, "forward workspace (selection bitmap): have %zu bytes, need %zu", fwd_ws_bytes, have);
+    }
+    const size_t need = dsa_attn_bwd_scratch_bytes(T, N, Hq, Hkv, D);
+    if (!scratch || scratch_bytes < need) return fail(DSA_ERR_WORKSPACE, "backward scratch: have %zu bytes, need %zu", scratch_bytes, need);
+    float *delta = (float *)scratch;
+    const size_t partial_bytes = bwd_partial_bytes_for(T, N, Hkv, D);
+    float *partial = partial_bytes ? (float *)((char *)scratch + align_up((size_t)T * Hq * 4, 256)) : nullptr;
+    int32_t *order = (int32_t *)((char *)scratch + need - align_up(dsa_tile_order_bytes(T), 256));
+    // the kernels only read the bitmap; the forward's workspace is not written here
+    uint32_t *bitmap = idx ? const_cast<uint32_t *>((const uint32_t *)fwd_ws) : nullptr;
+    return attn_bwd_run(dout, q, k, v, out, lse, idx, n, cu, T, N, Hq, Hkv, D, K, softmax_scale, max_seqlen, causal, dq, dk, dv,
+                        delta, bitmap, partial, partial_bytes, order, DSA_BWD_ALL & ~DSA_BWD_BITMAP, (hipStream_t)stream);
 }
 
 extern "C" int dsa_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,

@@ -29,11 +29,17 @@ def varlen_attn(query, key, value, cu_seq_q, cu_seq_k, max_q, max_k, is_causal=N
     unknown = set(dsa) - set(_DSA_KEYS)
     if unknown:
         raise TypeError(f"unexpected arguments {sorted(unknown)}")
-    # self-attention only: both offsets must be the same tensor, or two views of the same memory.  (Comparing the
-    # contents of two distinct tensors would copy from the device and stall the stream once per layer.)
+    # self-attention only.  The same tensor, or two views of the same memory, is the usual call and costs nothing to
+    # check; two separately built tensors (a clone, a .to()) are compared by content, which copies from the device once
+    # - torch's own routine accepts them (models/qwen3_vl/model.py:41-46 passes one tensor twice) - and cannot be
+    # done while a stream is being captured.
     if cu_seq_q is not cu_seq_k and not (cu_seq_q.data_ptr() == cu_seq_k.data_ptr() and cu_seq_q.shape == cu_seq_k.shape
                                          and cu_seq_q.stride() == cu_seq_k.stride()):
-        raise ValueError("self-attention only: pass the same cu_seqlens tensor as cu_seq_q and cu_seq_k")
+        if cu_seq_q.is_cuda and torch.cuda.is_current_stream_capturing():
+            raise ValueError("self-attention only: pass the same cu_seqlens tensor as cu_seq_q and cu_seq_k "
+                             "(two tensors cannot be compared during stream capture)")
+        if cu_seq_q.shape != cu_seq_k.shape or not torch.equal(cu_seq_q, cu_seq_k.to(cu_seq_q.device)):
+            raise ValueError("self-attention only: cu_seq_q and cu_seq_k must hold the same offsets")
     if max_q != max_k:
         raise ValueError("self-attention only: max_q and max_k must agree")
     if window_size is not None:
@@ -65,25 +71,33 @@ def _hf_indexer_to_packed(x):
     return x if x is None or x.dim() < 3 or x.shape[0] != 1 else x.squeeze(0)
 
 
-_BOUND_CACHE = {}                     # (data_ptr, version, numel, device) of a cu_seqlens tensor -> its longest segment
+_BOUND_ATTR = "_dsa_longest_segment"      # (version, storage offset, numel, bound), kept on the tensor that owns the memory
 
 
 def longest_segment(cu_seqlens) -> int:
     """Longest segment of a packed row, read back from the device once per ``cu_seqlens`` tensor: every layer of a
-    step hands over the same tensor, so the copy (and its stall) is paid once per batch instead of once per layer as
-    in the reference (train/model_attention.py:120-121).  While a stream is being captured nothing may be copied to
-    the host: the packed length, an upper bound, is returned instead."""
-    if torch.cuda.is_current_stream_capturing():
+    step hands over the same tensor (or a view of it), so the copy (and its stall) is paid once per batch instead of
+    once per layer as in the reference (train/model_attention.py:120-121).
+
+    The value is kept as an attribute of the tensor *object* that owns the memory (the view's base), together with
+    that tensor's version counter: it dies with the tensor, an in-place write invalidates it, and a new tensor that
+    happens to get a freed tensor's address starts without it.  (An address is no identity: the caching allocator
+    hands the same block to every step's offsets.)  While a stream is being captured nothing may be copied to the
+    host: None is returned, which the operator reads as the packed length, an upper bound."""
+    if cu_seqlens.is_cuda and torch.cuda.is_current_stream_capturing():
         return None
-    key = (cu_seqlens.data_ptr(), cu_seqlens._version, cu_seqlens.numel(), str(cu_seqlens.device))
-    hit = _BOUND_CACHE.get(key)
-    if hit is None:
-        if len(_BOUND_CACHE) > 64:
-            _BOUND_CACHE.clear()
-        flat = cu_seqlens.reshape(-1)
-        hit = max(int((flat[1:] - flat[:-1]).max()), 1) if flat.numel() > 1 else 1
-        _BOUND_CACHE[key] = hit
-    return hit
+    owner = cu_seqlens._base if cu_seqlens._base is not None else cu_seqlens
+    key = (owner._version, cu_seqlens.storage_offset(), cu_seqlens.numel())
+    hit = getattr(owner, _BOUND_ATTR, None)
+    if hit is not None and hit[:3] == key:
+        return hit[3]
+    flat = cu_seqlens.reshape(-1)
+    bound = max(int((flat[1:] - flat[:-1]).max()), 1) if flat.numel() > 1 else 1
+    try:
+        setattr(owner, _BOUND_ATTR, key + (bound,))
+    except AttributeError:               # a tensor subclass with __slots__: no cache, one copy per call
+        pass
+    return bound
 
 
 def varlen_attention_forward(query, key, value, attention_mask, max_seqlen=None, **dsa):
@@ -181,12 +195,16 @@ def replace_attention_qwenvl():
         ("transformers.models.qwen3_vl_moe.modeling_qwen3_vl_moe", "Qwen3VLMoeTextAttention", qwen3vl_forward),
         ("transformers.models.qwen3_5.modeling_qwen3_5", "Qwen3_5Attention", qwen3_5_forward),
     )
-    undo = []
+    # resolve every target before touching any: a transformers build without one of the models then fails with
+    # nothing patched
+    resolved = []
     for mod_name, cls_name, fwd in targets:
         mod = importlib.import_module(mod_name)
-        cls = getattr(mod, cls_name)
+        resolved.append((mod, getattr(mod, cls_name), fwd, mod.create_causal_mask))
+    undo = []
+    for mod, cls, fwd, mask_fn in resolved:
         undo.append((cls, "forward", cls.forward))
         cls.forward = fwd
-        undo.append((mod, "create_causal_mask", mod.create_causal_mask))
+        undo.append((mod, "create_causal_mask", mask_fn))
         mod.create_causal_mask = return_mask
     return undo

@@ -310,6 +310,26 @@ def attn_bwd(dout, q, k, v, out, lse, idx, n, cu_seqlens, max_seqlen: int, softm
     return (dq, dk, dv) if buffers is None else (dq, dk, dv, ws)
 
 
+def attn_bwd_saved_bitmap(dout, q, k, v, out, lse, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float, fwd_ws,
+                          causal: bool = True):
+    """Stage D4 reading the selection bitmap out of the forward's workspace ``fwd_ws`` (None for dense attention); the
+    scratch it allocates lives for the call only."""
+    T, Hq, Hkv, D = _check_qkv(q, k, v)
+    cu = _check_cu(cu_seqlens, T)
+    K = idx.shape[1] if idx is not None else 0
+    lib = _lib.load()
+    N = cu.numel() - 1
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    sc_bytes = lib.dsa_attn_bwd_scratch_bytes(T, N, Hq, Hkv, D)
+    scratch = torch.empty((max(sc_bytes, 4),), dtype=torch.uint8, device=q.device)
+    rc = lib.dsa_attn_bwd_saved_bitmap(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(idx), _ptr(n),
+                                       _ptr(cu), T, N, Hq, Hkv, D, K, softmax_scale, _lib.DSA_DTYPE_BF16, max_seqlen,
+                                       1 if causal else 0, _ptr(dq), _ptr(dk), _ptr(dv), _ptr(fwd_ws),
+                                       0 if fwd_ws is None else fwd_ws.numel(), _ptr(scratch), sc_bytes, _stream(q.device))
+    _lib.check(rc, "dsa_attn_bwd_saved_bitmap")
+    return dq, dk, dv
+
+
 # ------------------------------------------------------------------------------------------------
 # the operator
 # ------------------------------------------------------------------------------------------------
@@ -351,18 +371,15 @@ class _DsaVarlenAttn(torch.autograd.Function):
             qb, kb, vb = _split_stack(q, 0), _split_stack(k, 1), _split_stack(v, 0)
         else:
             qb, kb, vb = _as_bf16(q), _as_bf16(k), _as_bf16(v)
-        bwd_ws = None
+        fwd_ws = None
         lib = _lib.load()
         if idx is not None and lib.dsa_get_tile_crossover() > 0:     # (crossover 0: the forward builds no bitmap)
-            # one workspace for forward and backward: the bitmap the forward builds stays where the backward reads it
-            T, Hq = qb.shape[0], qb.shape[1]
-            bwd_ws = torch.empty((max(lib.dsa_attn_bwd_workspace_bytes(T, Hq, int(max_seqlen), 1), 4),), dtype=torch.uint8,
-                                 device=qb.device)
-            fwd_ws = bwd_ws[lib.dsa_attn_bwd_bitmap_offset(T, Hq):]
-            out, lse = attn_fwd(qb, kb, vb, idx, n, cu_seqlens, int(max_seqlen), softmax_scale, causal, ws=fwd_ws)
-        else:
-            out, lse = attn_fwd(qb, kb, vb, idx, n, cu_seqlens, int(max_seqlen), softmax_scale, causal)
-        ctx.bwd_ws = bwd_ws
+            # the selection bitmap the forward builds is kept for the backward; nothing else is held in between
+            # (delta, the key-tile order and the partial sums of cut walks are allocated when the backward runs)
+            fwd_ws = torch.empty((max(lib.dsa_attn_fwd_workspace_bytes(qb.shape[0], int(max_seqlen), 1), 4),),
+                                 dtype=torch.uint8, device=qb.device)
+        out, lse = attn_fwd(qb, kb, vb, idx, n, cu_seqlens, int(max_seqlen), softmax_scale, causal, ws=fwd_ws)
+        ctx.fwd_ws = fwd_ws
         ctx.causal = bool(causal)
         ctx.save_for_backward(qb, kb, vb, out, lse, cu_seqlens, *(() if idx is None else (idx, n)))
         ctx.has_idx = idx is not None
@@ -392,11 +409,10 @@ class _DsaVarlenAttn(torch.autograd.Function):
             db = _split_stack(dout.float(), 1)
         else:
             db = _as_bf16(dout)
-        if ctx.bwd_ws is not None:                       # the forward left the selection bitmap in the workspace
-            bufs = (torch.empty_like(qb), torch.empty_like(kb), torch.empty_like(vb), ctx.bwd_ws)
-            dq, dk, dv, _ = attn_bwd(db, qb, kb, vb, out, lse, idx, n, cu, ctx.max_seqlen, ctx.softmax_scale,
-                                     parts=_lib.DSA_BWD_ALL & ~_lib.DSA_BWD_BITMAP, buffers=bufs, causal=ctx.causal)
-            ctx.bwd_ws = None
+        if ctx.fwd_ws is not None or idx is None:        # the forward's bitmap is read where it lies
+            dq, dk, dv = attn_bwd_saved_bitmap(db, qb, kb, vb, out, lse, idx, n, cu, ctx.max_seqlen, ctx.softmax_scale,
+                                               ctx.fwd_ws, causal=ctx.causal)
+            ctx.fwd_ws = None
         else:
             dq, dk, dv = attn_bwd(db, qb, kb, vb, out, lse, idx, n, cu, ctx.max_seqlen, ctx.softmax_scale,
                                   causal=ctx.causal)
