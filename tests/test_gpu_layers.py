@@ -135,7 +135,7 @@ def test_dsa_layers_match_the_oracle_output_loss_and_every_gradient(kind, top_k)
         if wr.grad.abs().max() > 0:
             # the oracle rounds the indexer's projections to bf16 as the device does (round_indexer_to_bf16), so that both
             # open the same ReLU gates [q_idx.k_idx > 0]; what is left is the bf16 arithmetic of the kernels
-            res.append(_close(p.grad, wr.grad, f"d{name}", rel=4e-2, min_cos=0.999))
+            res.append(_close(p.grad, wr.grad, f"d{name}"))     # the same bar as every other tensor (observed cosine 0.99998)
     _log(f"  loss {loss.item():.5f} (oracle {ref_loss.item():.5f}) " + " ".join(f"({e:.2e},{c:.6f})" for e, c in res))
     if top_k >= 512:                                       # the whole window is selected: the dense layer, bit for bit
         dense = _make(cls, _cfg(hidden, Hq, Hkv, D), None, seed=17, param_dtype=torch.bfloat16)
@@ -369,7 +369,7 @@ def test_head_sharded_dtensor_projections_pass_through_layer_kernel_and_rewrap(k
         wraps = [(w, o) for w, o in seen if w is not None]
         assert len(wraps) == 1 and len(seen) == 2            # the plain layer's call wrapped nothing
         (w_mesh, w_place), rewrapped = wraps[0]
-        assert isinstance(rewrapped, DTensor) and rewrapped.device_mesh is mesh and w_mesh is mesh
+        assert isinstance(rewrapped, DTensor) and rewrapped.device_mesh == mesh and w_mesh == mesh
         assert tuple(rewrapped.placements) == tuple(w_place) == (Shard(1),)      # (T, heads, head_dim): sharded by head
         assert rewrapped.to_local().is_cuda
     finally:
