@@ -145,12 +145,15 @@ size_t dsa_attn_fwd_workspace_bytes(int T, int max_seqlen, int has_idx);
  * over sel(t) sums to one, so a row sums to one: it is the target distribution of the KL loss that
  * trains a DSA indexer (the selection itself passes no gradient).  No reference counterpart - the
  * reference holds no indexer; it would be called beside the attention call of a layer in its training
- * step (train/train_qwen.py:534-548).  fp32 out, deterministic.  ws: dsa_attn_mass_workspace_bytes().
+ * step (train/train_qwen.py:534-548).  fp32 out, deterministic.  ws: dsa_attn_mass_workspace_bytes() for the
+ * same geometry: the selection bitmap and one (T,K) fp32 table per group of kv heads - a workgroup takes the kv
+ * heads of its group in turn and sums in place; one to Hkv groups, as many as fill the chip (two at 32 768 tokens
+ * with 8 kv heads: 0.5 GiB; none when one group takes every kv head).
  */
 int dsa_attn_mass(const void *q, const void *k, const float *lse, const int32_t *idx, const int32_t *n,
                   const int32_t *cu_seqlens, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
                   int dtype, int max_seqlen, float *mass, void *ws, size_t ws_bytes, void *stream);
-size_t dsa_attn_mass_workspace_bytes(int T, int Hkv, int K, int max_seqlen);
+size_t dsa_attn_mass_workspace_bytes(int T, int N, int Hq, int Hkv, int D, int K, int max_seqlen);
 
 /*
  * Tuning knob (process-wide, no reference counterpart): query rows whose position in their segment is

@@ -41,7 +41,7 @@ _SIGNATURES = {
     "dsa_attn_fwd_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "dsa_attn_mass": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                               c_int, c_float, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
-    "dsa_attn_mass_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "dsa_attn_mass_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
     "dsa_set_tile_crossover": (c_int, [c_int]),
     "dsa_get_tile_crossover": (c_int, []),
     "dsa_attn_bwd_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),

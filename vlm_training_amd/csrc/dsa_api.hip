@@ -1,5 +1,6 @@
 // C ABI of the library (declared in include/dsa_attn.h): argument checks, workspace layout, launches.
 #include <hip/hip_runtime.h>
+#include <algorithm>
 #include <atomic>
 #include <mutex>
 #include <stdarg.h>
@@ -48,6 +49,7 @@ hipError_t dsa_launch_tile_dkv(const void *dout, const void *q, const void *k, c
                                size_t partial_bytes, void *dk, void *dv, hipStream_t stream);
 size_t dsa_tile_order_bytes(int T);
 size_t dsa_tile_dkv_partial_bytes(int T);
+int dsa_mass_groups(int Hq, int Hkv, int D);
 }
 
 extern "C" {
@@ -306,9 +308,11 @@ extern "C" int dsa_attn_fwd(const void *q, const void *k, const void *v, const i
 }
 
 // ---- attention mass of the selected keys (training target of the indexer) ---------------------------
-extern "C" size_t dsa_attn_mass_workspace_bytes(int T, int Hkv, int K, int max_seqlen) {
-    if (T <= 0 || Hkv <= 0 || K <= 0) return 0;
-    return align_up((size_t)T * bitmap_ldw(max_seqlen) * 4, 256) + align_up((size_t)Hkv * T * K * 4, 256);
+// bitmap + one (T,K) fp32 table per group of kv heads (none when one group takes all kv heads)
+extern "C" size_t dsa_attn_mass_workspace_bytes(int T, int N, int Hq, int Hkv, int D, int K, int max_seqlen) {
+    if (T <= 0 || N < 0 || Hkv <= 0 || Hq < Hkv || K <= 0) return 0;
+    const int g = dsa_mass_groups(Hq, Hkv, D);
+    return align_up((size_t)T * bitmap_ldw(max_seqlen) * 4, 256) + (g > 1 ? align_up((size_t)g * T * K * 4, 256) : 0);
 }
 
 extern "C" int dsa_attn_mass(const void *q, const void *k, const float *lse, const int32_t *idx, const int32_t *n,
@@ -318,7 +322,7 @@ extern "C" int dsa_attn_mass(const void *q, const void *k, const float *lse, con
     if (!q || !k || !lse || !idx || !n || !mass) return fail(DSA_ERR_ARG, "null tensor pointer");
     if (max_seqlen < 1 || max_seqlen > (T > 0 ? T : 1)) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
     if (T == 0) return DSA_OK;
-    const size_t need = dsa_attn_mass_workspace_bytes(T, Hkv, K, max_seqlen);
+    const size_t need = dsa_attn_mass_workspace_bytes(T, N, Hq, Hkv, D, K, max_seqlen);
     if (!ws || ws_bytes < need) return fail(DSA_ERR_WORKSPACE, "mass workspace: have %zu bytes, need %zu", ws_bytes, need);
     const int ldw = bitmap_ldw(max_seqlen);
     if ((size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);

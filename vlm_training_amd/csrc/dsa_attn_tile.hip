@@ -152,6 +152,55 @@ __device__ __forceinline__ bool locate_block(const int32_t *cu, int N, int slot,
     return false;
 }
 
+// The same hand-out, heaviest block first over the whole batch: slot 0 takes the last block of the longest segment,
+// then every block with the next lower index in segment order, and so on - a block's walk grows with its index, so
+// long walks start first wherever their segment lies in the batch (with the segment-by-segment order the long
+// walks of a late segment start late and the launch ends on them).  For up to 64 segments (their lengths live in
+// one wave's lanes); larger batches fall back to the segment-by-segment order.
+__device__ __forceinline__ int wave_sum_i(int x) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off, 64);
+    return x;
+}
+__device__ __forceinline__ bool locate_block_heaviest_first(const int32_t *cu, int N, int slot, int blk, int &s0, int &L,
+                                                            int &b) {
+    if (N > 64) return locate_block(cu, N, slot, blk, true, s0, L, b);
+    const int lane = threadIdx.x & 63;
+    const int seg = min(lane, N - 1);
+    const int lo = cu[seg], len = cu[seg + 1] - lo;
+    const int nb = lane < N ? (len + blk - 1) / blk : 0;
+    int most = nb;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) most = max(most, __shfl_xor(most, off, 64));
+    // blocks with index >= x over all segments
+    auto count_ge = [&](int x) { return wave_sum_i(max(nb - x, 0)); };
+    if (slot >= count_ge(0)) return false;
+    int lo_b = 0, hi_b = most;                           // count_ge(lo_b) > slot >= count_ge(hi_b)
+    while (hi_b - lo_b > 1) {
+        const int mid = (lo_b + hi_b) >> 1;
+        if (count_ge(mid) > slot) lo_b = mid; else hi_b = mid;
+    }
+    b = lo_b;
+    const int rank = slot - count_ge(b + 1);             // among the segments that have a block b, in segment order
+    const uint64_t has = __builtin_amdgcn_ballot_w64(nb > b);
+    // the rank-th set bit of `has`
+    const int below = (int)__popcll(has & ((1ull << lane) - 1ull));
+    const uint64_t me = __builtin_amdgcn_ballot_w64(nb > b && below == rank);
+    const int w = (int)__builtin_ctzll(me);
+    s0 = __builtin_amdgcn_readlane(lo, w);
+    L = __builtin_amdgcn_readlane(len, w);
+    return true;
+}
+
+// Query blocks are handed out heaviest first: over the whole batch for launches of a few rounds of workgroups (they
+// would otherwise end on the long walks of a late segment: forward -11 %, dQ -15 % on 8192 tokens in seven
+// segments), segment by segment for larger ones, where the blocks of a segment that run side by side share their
+// K / V tiles in L2 (the batch-wide order is 2-3 % slower there).
+#define DSA_BATCH_ORDER_MAX_BLOCKS (6 * 256)
+#define LOCATE_QUERY_BLOCK(cu, N, slot, blk, s0, L, b)                                                           \
+    (gridDim.x <= DSA_BATCH_ORDER_MAX_BLOCKS ? locate_block_heaviest_first(cu, N, slot, blk, s0, L, b)          \
+                                             : locate_block(cu, N, slot, blk, true, s0, L, b))
+
 // ==================================================================================================
 // forward: query-stationary.  Workgroup = 4 waves x 32 rows = 128 rows = 128/Gp queries of one
 // segment and one kv head; loops over 32-key tiles of the causal range.
@@ -207,7 +256,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     const int G = Hq / Hkv;
     const int kvh = blockIdx.x % Hkv;
     int s0, L, blk;
-    if (!locate_block(cu, N, blockIdx.x / Hkv, QBW, true, s0, L, blk)) return;
+    if (!LOCATE_QUERY_BLOCK(cu, N, blockIdx.x / Hkv, QBW, s0, L, blk)) return;
     if (HAS_IDX) L = min(L, ldw * 32);                  // a bitmap row has ldw words whatever the caller's max_seqlen
     const int qc0 = blk * QBW;
     if (qc0 >= pos_split || qc0 >= L) return;                       // rows past the split belong to the gather kernel
@@ -328,23 +377,32 @@ __device__ __forceinline__ float group_sum(float x) {
     if (GSHIFT >= 4) x += dpp_f<0x140>(x);              // row_mirror: the other half row's total
     return x;
 }
-template <int D, int GSHIFT, int NW>
-__global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_tile_mass_kernel(
+// The heads of a query meet in one workgroup: a wave's 32 rows are (query, head of one kv group) pairs as in the
+// forward, and the workgroup takes the HPG kv heads of its group one after the other *inside* each key tile - all
+// their K tiles are staged together, all their q rows stay in registers (one wave per SIMD, so a wave may hold
+// 512) - and adds their probabilities up in registers.  A slot of the result is therefore written once, by one
+// lane, with the finished sum: no table per kv head, nothing read back.  Only a batch with more kv heads than a
+// workgroup can hold (HPG * D/4 <= 256 registers of q rows) is cut into groups with one table each.
+template <int D> constexpr int mass_heads_max() { return 1024 / D; }      // 16 / 8 / 4 kv heads at head_dim 64 / 128 / 256
+template <int D, int HPG> constexpr size_t mass_lds_bytes() { return (size_t)HPG * tile_bytes<D>(); }
+template <int D, int GSHIFT, int HPG>
+__global__ __launch_bounds__(256, 1) void dsa_tile_mass_kernel(
     const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const float *__restrict__ lse,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
-    float scale_log2, int K, float *__restrict__ partial) {
-    constexpr int KS = D / 16, CPR = D / 8, TILE_B = tile_bytes<D>(), LOADS = 32 * CPR / (NW * 64);
-    constexpr int NBUF = 2, NT = NW * 64, Gp = 1 << GSHIFT, QBW = (NW * 32) >> GSHIFT;
-    static_assert(LOADS >= 1, "tile must give every thread a chunk");
-    __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][TILE_B];
+    float scale_log2, int K, int ngroups, float final_mul, float *__restrict__ table) {
+    constexpr int KS = D / 16, CPR = D / 8, TILE_B = tile_bytes<D>(), NT = 256;
+    constexpr int Gp = 1 << GSHIFT, QBW = (4 * 32) >> GSHIFT;
+    constexpr int CH = 32 * HPG * CPR, LOADS = CH / NT;  // 16-byte chunks of one key tile of all HPG heads; per thread
+    static_assert(CH % NT == 0 && LOADS >= 1, "every thread stages the same number of chunks");
+    extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];   // [HPG][TILE_B]
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
     LaneOffsets<D> lo;
     lo.init(lane);
     const int G = Hq / Hkv;
-    const int kvh = blockIdx.x % Hkv;
+    const int grp = blockIdx.x % ngroups, kvh0 = grp * HPG;
     int s0, L, blk;
-    if (!locate_block(cu, N, blockIdx.x / Hkv, QBW, true, s0, L, blk)) return;
+    if (!locate_block_heaviest_first(cu, N, blockIdx.x / ngroups, QBW, s0, L, blk)) return;
     L = min(L, ldw * 32);                               // a bitmap row has ldw words whatever the caller's max_seqlen
     const int qc0 = blk * QBW;
     if (qc0 >= L) return;
@@ -352,69 +410,95 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     const int r = wv * 32 + j;
     const int qcol = qc0 + (r >> GSHIFT), head = r & (Gp - 1);
     const bool row_ok = qcol < L && head < G;
-    const int t = s0 + min(qcol, L - 1), hq = kvh * G + min(head, G - 1);
-    u32x4 kst[2][LOADS];
-#define MASS_LOAD(SET, TILE)                                                                        \
-    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
-        const int c = i * NT + tid;                                                                \
-        const int row = c / CPR, ch = c % CPR;                                                     \
-        kst[SET][i] = *reinterpret_cast<const u32x4 *>(                                            \
-            k + ((int64_t)(s0 + min((TILE) * 32 + row, L - 1)) * Hkv + kvh) * D + ch * 8);         \
-    }
-    MASS_LOAD(0, 0)
-    bf16x8 qB[KS];
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-        qB[ks] = row_ok ? load_bf16x8(q + ((int64_t)t * Hq + hq) * D + 16 * ks + 8 * h) : zero_bf16x8();
-    // padding rows (head >= G, query past the segment) get lse = +inf: their P is exp2(-inf) = 0 in the head sums.
-    // Keys that are not selected need no masking: their sums are never stored.
-    const float lse_row = lse[(int64_t)hq * T + t];
-    const float lse2 = row_ok ? lse_row * LOG2E_F : INFINITY;
+    const int t = s0 + min(qcol, L - 1);
     const int ntiles = min(qc0 + QBW - 1, L - 1) / 32 + 1;
     const uint32_t *wrow = bitmap + (int64_t)t * ldw;
-    uint32_t word_next = wrow[0];
-    int seen = 0;                                        // selected keys of this row in the tiles already walked
-    float *prow = partial + ((int64_t)kvh * T + t) * K;
-
-#define MASS_STORE(SET, BUF, TILE)                                                                  \
+    float *prow = table + ((int64_t)grp * T + t) * K;
+    if (ngroups == 1) {
+        // the table is the result itself: slots past a row's selection (rows shorter than K keys) are zero
+        for (int qq = 0; qq < QBW && qc0 + qq < L; ++qq) {
+            float *zr = table + (int64_t)(s0 + qc0 + qq) * K;
+            for (int jj = qc0 + qq + 1 + tid; jj < K; jj += NT) zr[jj] = 0.f;
+        }
+    }
+    u32x4 kst[LOADS];
+    // one key row of the group's kv heads is contiguous in memory (HPG * D elements); kv heads past the last one
+    // (a short last group) read the last head again and count for nothing (lse = +inf below)
+#define MASS_LOAD(TILE)                                                                             \
     _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
         const int c = i * NT + tid;                                                                \
-        const int row = c / CPR, ch = c % CPR;                                                     \
-        *reinterpret_cast<u32x4 *>(&lds[BUF][tile_off<D>(row, ch)]) = kst[SET][i];                 \
+        const int row = c / (HPG * CPR), hh = (c / CPR) % HPG, ch = c % CPR;                       \
+        kst[i] = *reinterpret_cast<const u32x4 *>(                                                 \
+            k + ((int64_t)(s0 + min((TILE) * 32 + row, L - 1)) * Hkv + min(kvh0 + hh, Hkv - 1)) * D + ch * 8); \
     }
-#define MASS_COMPUTE(TILE, BUF)                                                                     \
-    {                                                                                              \
-        const unsigned char *kt = lds[BUF];                                                        \
-        /* padding lanes of a query (head >= G) compute nothing but take their share of the stores */ \
-        const uint32_t word_full = qcol < L ? word_next : 0u;                                      \
-        word_next = wrow[min((TILE) + 1, ntiles - 1)];                                             \
-        f32x16 sacc = zero16();                                                                    \
-        {                                                                                          \
-            bf16x8 ka[KS];                                                                         \
-            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) ka[ks] = lo.rowop(kt, ks);           \
-            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) sacc = mfma32(ka[ks], qB[ks], sacc); \
-            sched_reads_ahead<KS, 4, 1>();                                                         \
-        }                                                                                          \
-        float p[16];                                                                               \
-        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) p[vi] = fast_exp2(fmaf(sacc[vi], scale_log2, -lse2)); \
-        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) p[vi] = group_sum<GSHIFT>(p[vi]);        \
-        /* the lanes of a query share the stores: lane `head` writes the elements vi = u*Gp + head */ \
-        _Pragma("unroll") for (int u = 0; u < 16 / Gp; ++u) {                                      \
-            float val = p[u * Gp];                                                                 \
-            _Pragma("unroll") for (int g = 1; g < Gp; ++g) val = head == g ? p[u * Gp + g] : val;  \
-            const int vi = u * Gp + head;                                                          \
-            const int bit = 8 * (vi >> 2) + (vi & 3) + 4 * h;    /* the key's column in the tile */ \
-            if ((word_full >> bit) & 1u) prow[seen + __popc(word_full & ((1u << bit) - 1u))] = val; \
-        }                                                                                          \
-        seen += __popc(word_full);                                                                 \
+#define MASS_STORE()                                                                                \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                            \
+        const int c = i * NT + tid;                                                                \
+        const int row = c / (HPG * CPR), hh = (c / CPR) % HPG, ch = c % CPR;                       \
+        *reinterpret_cast<u32x4 *>(&dyn_lds[hh * TILE_B + tile_off<D>(row, ch)]) = kst[i];         \
     }
-    TILE_PIPELINE(ntiles, MASS_LOAD, MASS_STORE, MASS_COMPUTE)
+    MASS_LOAD(0)
+    bf16x8 qB[HPG][KS];
+    float lse2[HPG];
+#pragma unroll
+    for (int hh = 0; hh < HPG; ++hh) {
+        const int kvh = min(kvh0 + hh, Hkv - 1);
+        const int hq = kvh * G + min(head, G - 1);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+            qB[hh][ks] = row_ok ? load_bf16x8(q + ((int64_t)t * Hq + hq) * D + 16 * ks + 8 * h) : zero_bf16x8();
+        // padding rows (head >= G, query past the segment, kv head past the last) get lse = +inf: their P is
+        // exp2(-inf) = 0 in the sums.  Keys that are not selected need no masking: their sums are never stored.
+        const float lse_row = lse[(int64_t)hq * T + t];
+        lse2[hh] = (row_ok && kvh0 + hh < Hkv) ? lse_row * LOG2E_F : INFINITY;
+    }
+    uint32_t word_next = qcol < L ? wrow[0] : 0u;
+    int seen = 0;                                        // selected keys of this row in the tiles already walked
+    MASS_STORE()
+    __syncthreads();
+    for (int it = 0; it < ntiles; ++it) {
+        MASS_LOAD(min(it + 1, ntiles - 1))               // lands during this tile's matrix work
+        const uint32_t word_full = word_next;
+        { const uint32_t wl = wrow[min(it + 1, ntiles - 1)]; word_next = qcol < L ? wl : 0u; }
+        float p[16];
+#pragma unroll
+        for (int vi = 0; vi < 16; ++vi) p[vi] = 0.f;
+#pragma unroll
+        for (int hh = 0; hh < HPG; ++hh) {
+            // (issuing the matrix work of head hh+1 between the exponentials of head hh in a hand-fixed order
+            // measured no faster than what the scheduler makes of this loop)
+            const unsigned char *kt = dyn_lds + hh * TILE_B;
+            f32x16 sacc = zero16();
+            bf16x8 ka[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) ka[ks] = lo.rowop(kt, ks);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) sacc = mfma32(ka[ks], qB[hh][ks], sacc);
+#pragma unroll
+            for (int vi = 0; vi < 16; ++vi) p[vi] += fast_exp2(fmaf(sacc[vi], scale_log2, -lse2[hh]));
+        }
+#pragma unroll
+        for (int vi = 0; vi < 16; ++vi) p[vi] = group_sum<GSHIFT>(p[vi]);
+        // the lanes of a query share the stores: lane `head` writes the elements vi = u*Gp + head
+#pragma unroll
+        for (int u = 0; u < 16 / Gp; ++u) {
+            float val = p[u * Gp];
+#pragma unroll
+            for (int g = 1; g < Gp; ++g) val = head == g ? p[u * Gp + g] : val;
+            const int vi = u * Gp + head;
+            const int bit = 8 * (vi >> 2) + (vi & 3) + 4 * h;    // the key's column in the tile
+            if ((word_full >> bit) & 1u) prow[seen + __popc(word_full & ((1u << bit) - 1u))] = val * final_mul;
+        }
+        seen += __popc(word_full);
+        __syncthreads();                                 // every wave is done with this tile's K
+        MASS_STORE()
+        __syncthreads();
+    }
 #undef MASS_LOAD
 #undef MASS_STORE
-#undef MASS_COMPUTE
 }
 
-// mass[t,j] = inv_hq * sum over kv heads of partial[kvh][t][j] for j < n[t], else 0.  One workgroup per query row
+// mass[t,j] = inv_hq * sum over the tables of partial[g][t][j] for j < n[t], else 0.  One workgroup per query row
 // and blockIdx.y-th part of it, four columns per thread (16-byte accesses when K is a multiple of four).
 __global__ __launch_bounds__(256) void dsa_mass_reduce_kernel(const float *__restrict__ partial,
                                                                const int32_t *__restrict__ nsel, int T, int K, int Hkv,
@@ -474,7 +558,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     LaneOffsets<D> lo;
     lo.init(lane);
     int s0, L, blk;
-    if (!locate_block(cu, N, blockIdx.x, QBW, true, s0, L, blk)) return;
+    if (!LOCATE_QUERY_BLOCK(cu, N, blockIdx.x, QBW, s0, L, blk)) return;
     L = min(L, ldw * 32);
     const int qc0 = blk * QBW;
     if (qc0 >= L) return;
@@ -761,7 +845,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     const int G = Hq / Hkv;
     const int kvh = blockIdx.x % Hkv;
     int s0, L, blk;
-    if (!locate_block(cu, N, blockIdx.x / Hkv, QBW, true, s0, L, blk)) return;
+    if (!LOCATE_QUERY_BLOCK(cu, N, blockIdx.x / Hkv, QBW, s0, L, blk)) return;
     if (HAS_IDX) L = min(L, ldw * 32);                  // a bitmap row has ldw words whatever the caller's max_seqlen
     const int qc0 = blk * QBW;
     if (qc0 >= pos_split || qc0 >= L) return;
@@ -2048,26 +2132,65 @@ extern "C" hipError_t dsa_launch_tile_fwd(const void *q, const void *k, const vo
     TILE_SWITCH_96(launch_fwd_i, grid, stream, q, k, v, bitmap, ldw, cu, N, T, Hq, Hkv, scale * LOG2E_F, pos_split, causal, out, lse)
     return hipGetLastError();
 }
+// kv heads a workgroup of the attention-mass kernel takes (a power of two, at most what its registers hold; with
+// one query head per kv head a lane also holds all sixteen sums of a tile to itself, which costs the top size)
+template <int D>
+static int mass_hpg(int Hq, int Hkv) {
+    const int most = Hq == Hkv ? mass_heads_max<D>() / 2 : mass_heads_max<D>();
+    int hpg = 1;
+    while (hpg * 2 <= most && hpg < Hkv) hpg *= 2;
+    return hpg;
+}
+extern "C" int dsa_mass_groups(int Hq, int Hkv, int D) {
+    const int hpg = D == 64 ? mass_hpg<64>(Hq, Hkv) : D == 128 ? mass_hpg<128>(Hq, Hkv) : mass_hpg<256>(Hq, Hkv);
+    return (Hkv + hpg - 1) / hpg;
+}
+template <int D, int GS, int HPG>
+static hipError_t launch_mass_h(dim3 grid, hipStream_t stream, const void *q, const void *k, const float *lse,
+                                const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T, int Hq, int Hkv, float sl2,
+                                int K, int ngroups, float final_mul, float *table) {
+    if constexpr (HPG > mass_heads_max<D>()) {
+        return hipErrorInvalidValue;
+    } else {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&dsa_tile_mass_kernel<D, GS, HPG>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)mass_lds_bytes<D, HPG>());
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL((dsa_tile_mass_kernel<D, GS, HPG>), grid, dim3(256), (mass_lds_bytes<D, HPG>()), stream,
+                           (const bf16_t *)q, (const bf16_t *)k, lse, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, K, ngroups, final_mul,
+                           table);
+        return hipSuccess;
+    }
+}
 template <int D, bool HAS_IDX, int GS>
 static hipError_t launch_mass_i(dim3 grid, hipStream_t stream, const void *q, const void *k, const float *lse,
                           const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T, int Hq, int Hkv, float sl2,
-                          int K, float *partial) {
-    hipLaunchKernelGGL((dsa_tile_mass_kernel<D, GS, tile_waves<D>()>), grid, dim3(64 * tile_waves<D>()), 0, stream,
-                       (const bf16_t *)q, (const bf16_t *)k, lse, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, K, partial);
-    return hipSuccess;
+                          int K, int ngroups, float final_mul, float *table) {
+    switch (mass_hpg<D>(Hq, Hkv)) {
+        case 1: return launch_mass_h<D, GS, 1>(grid, stream, q, k, lse, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, K, ngroups, final_mul, table);
+        case 2: return launch_mass_h<D, GS, 2>(grid, stream, q, k, lse, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, K, ngroups, final_mul, table);
+        case 4: return launch_mass_h<D, GS, 4>(grid, stream, q, k, lse, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, K, ngroups, final_mul, table);
+        case 8: return launch_mass_h<D, GS, 8>(grid, stream, q, k, lse, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, K, ngroups, final_mul, table);
+        default: return launch_mass_h<D, GS, 16>(grid, stream, q, k, lse, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, K, ngroups, final_mul, table);
+    }
 }
-// attention mass of the selected keys: partial (Hkv,T,K) tables, then their sum scaled by 1/Hq into mass (T,K)
+// attention mass of the selected keys: the heads of a query summed in registers, scaled by 1/Hq and written into
+// mass (T,K); batches with more kv heads than one workgroup holds leave one (T,K) table per group in `partial`,
+// which dsa_mass_reduce_kernel adds in group order
 extern "C" hipError_t dsa_launch_tile_mass(const void *q, const void *k, const float *lse, const uint32_t *bitmap,
                                            int ldw, const int32_t *n, const int32_t *cu, int N, int T, int Hq, int Hkv,
                                            int D, int K, float scale, float *partial, float *mass, hipStream_t stream) {
     const int gs = group_shift(Hq, Hkv);
-    const dim3 grid((unsigned)(((int64_t)T / ((32 * tile_waves_of(D)) >> gs) + N + 1) * Hkv));
-    TILE_SWITCH(launch_mass_i, grid, stream, q, k, lse, bitmap, ldw, cu, N, T, Hq, Hkv, scale * LOG2E_F, K, partial)
+    const int ngroups = dsa_mass_groups(Hq, Hkv, D);
+    const dim3 grid((unsigned)(((int64_t)T / ((32 * 4) >> gs) + N + 1) * ngroups));
+    const float inv_hq = 1.f / (float)Hq;
+    float *table = ngroups == 1 ? mass : partial;
+    const float final_mul = ngroups == 1 ? inv_hq : 1.f;
+    TILE_SWITCH(launch_mass_i, grid, stream, q, k, lse, bitmap, ldw, cu, N, T, Hq, Hkv, scale * LOG2E_F, K, ngroups, final_mul, table)
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    if (e != hipSuccess || ngroups == 1) return e;
     const unsigned parts = (unsigned)((K / 4 + 255) / 256 > 0 ? (K / 4 + 255) / 256 : 1);
-    hipLaunchKernelGGL(dsa_mass_reduce_kernel, dim3(T, parts < 8 ? parts : 8), dim3(256), 0, stream, partial, n, T, K, Hkv,
-                       1.f / (float)Hq, mass);
+    hipLaunchKernelGGL(dsa_mass_reduce_kernel, dim3(T, parts < 8 ? parts : 8), dim3(256), 0, stream, partial, n, T, K, ngroups,
+                       inv_hq, mass);
     return hipGetLastError();
 }
 // indexer backward: prefix table, query side (dq_idx, dw), key side (dk_idx).  D = indexer head_dim (64 or 128),

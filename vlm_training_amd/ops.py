@@ -279,7 +279,7 @@ def attn_mass(q, k, lse, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: Opt
     lib = _lib.load()
     qb, kb = _as_bf16(q), _as_bf16(k)
     mass = torch.empty((T, K), dtype=torch.float32, device=q.device)
-    ws_bytes = lib.dsa_attn_mass_workspace_bytes(T, Hkv, K, max_seqlen)
+    ws_bytes = lib.dsa_attn_mass_workspace_bytes(T, cu.numel() - 1, Hq, Hkv, D, K, max_seqlen)
     ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q.device)
     rc = lib.dsa_attn_mass(_ptr(qb), _ptr(kb), _ptr(lse.contiguous()), _ptr(idx), _ptr(n), _ptr(cu), T, cu.numel() - 1, Hq,
                            Hkv, D, K, scale, _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(mass), _ptr(ws), ws_bytes,
