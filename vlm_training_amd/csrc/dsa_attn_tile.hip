@@ -2054,7 +2054,21 @@ template <int D, bool HAS_IDX, int GS>
 static hipError_t launch_fwd_i(dim3 grid, hipStream_t stream, const void *q, const void *k, const void *v,
                          const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T, int Hq, int Hkv, float sl2,
                          int pos_split, int causal, void *out, float *lse) {
-    hipLaunchKernelGGL((dsa_tile_fwd_kernel<D, HAS_IDX, GS, tile_waves<D>()>), grid, dim3(64 * tile_waves<D>()), 0, stream, (const bf16_t *)q,
+    constexpr int NW = tile_waves<D>();
+    if constexpr (NW == 8) {
+        // A launch of a few rounds of workgroups is bound by what a workgroup pays before its first tile and after
+        // its last (memory round trips, row stores), and with eight waves only one workgroup fits a CU.  Such
+        // launches run the four-wave form, two workgroups per CU, whose fixed parts overlap (forward -9 % on 8192
+        // tokens in seven segments; the dQ kernel measured 19 % slower that way and keeps eight waves).
+        if (grid.x <= DSA_BATCH_ORDER_MAX_BLOCKS) {
+            const int Gp = 1 << GS;
+            const dim3 grid4((unsigned)(((int64_t)T / ((32 * 4) / Gp) + N + 1) * Hkv));
+            hipLaunchKernelGGL((dsa_tile_fwd_kernel<D, HAS_IDX, GS, 4>), grid4, dim3(256), 0, stream, (const bf16_t *)q,
+                               (const bf16_t *)k, (const bf16_t *)v, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, pos_split, causal, (bf16_t *)out, lse);
+            return hipSuccess;
+        }
+    }
+    hipLaunchKernelGGL((dsa_tile_fwd_kernel<D, HAS_IDX, GS, NW>), grid, dim3(64 * NW), 0, stream, (const bf16_t *)q,
                        (const bf16_t *)k, (const bf16_t *)v, bitmap, ldw, cu, N, T, Hq, Hkv, sl2, pos_split, causal, (bf16_t *)out, lse);
     return hipSuccess;
 }
