@@ -315,6 +315,13 @@ def main():
     dom = max(kern, key=lambda name: stage_ms[name])
     dom_kernel, dom_flop = kern[dom]
     achieved = dom_flop / (stage_ms[dom] * 1e-3) / 1e12
+    # what the matrix cores actually execute: the tile kernels compute every causal pair of a visited tile and mask
+    # the unselected ones, so their MFMA rate is the selected-pair rate times (executed pairs / selected pairs)
+    xq, xk = w.executed_pairs(ops._lib.load().dsa_get_tile_crossover())
+    executed_pairs = {"attn_fwd": xq, "bwd_dq": xq, "bwd_dkv": xk}
+    executed = dom_flop / S * executed_pairs[dom] / (stage_ms[dom] * 1e-3) / 1e12
+    executed_by_kernel = {kern[name][0]: kern[name][1] / S * executed_pairs[name] / (stage_ms[name] * 1e-3) / 1e12 / PEAK_MFMA_BF16_TFLOPS
+                          for name in kern}
     t_roof_ms = {
         "index_topk": max(wk["F1"] / (PEAK_MFMA_BF16_TFLOPS * 1e12), wk["B2"] / (PEAK_HBM_GBS * 1e9)) * 1e3,
         "attn_fwd": max(wk["F3"] / (PEAK_MFMA_BF16_TFLOPS * 1e12), wk["B3"] / (PEAK_HBM_GBS * 1e9)) * 1e3,
@@ -349,7 +356,10 @@ def main():
         "config": {"workload": f"{w.name}: T={w.T} packed tokens, segments={list(w.seg_lens)}, Hq/Hkv/D={w.Hq}/{w.Hkv}/{w.D}, "
                                f"indexer {w.Hi}x{w.Di}, top_k={w.top_k}, fwd+bwd"},
         "roofline": {"bound": "mfma", "kernel": dom_kernel, "achieved": achieved, "peak": PEAK_MFMA_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_BF16_TFLOPS, "traffic": traffic,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_BF16_TFLOPS,
+                     "executed": executed, "executed_frac": executed / PEAK_MFMA_BF16_TFLOPS,
+                     "executed_pairs_over_selected": executed_pairs[dom] / S, "executed_frac_by_kernel": executed_by_kernel,
+                     "traffic": traffic,
                      "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command, scaled by a 1 GiB copy (profiles/)",
                      "algorithmic_flop": dom_flop, "avg_ms": stage_ms[dom]},
         "stage_ms": stage_ms,

@@ -85,6 +85,8 @@ int dsa_index_topk(const void *q_idx, const void *k_idx, const void *w_idx, cons
  * max_seqlen > dsa_index_topk_noalloc_max_seqlen() (2 097 152) returns DSA_ERR_WORKSPACE.  The call allocates
  * nothing and frees nothing.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (two
  * streams, two threads) race and must be serialised by the caller; calls on different GPUs are independent.
+ * The first call on a device looks up the array's address on that device (hipGetSymbolAddress): make one call
+ * outside any capture before capturing a graph around it.
  */
 int dsa_index_topk_noalloc(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu_seqlens, int T,
                            int N, int Hi, int Di, int K, float scale, int dtype, int max_seqlen, int32_t *idx,

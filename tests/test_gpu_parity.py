@@ -481,6 +481,12 @@ def test_reference_named_entry_points():
                                           v.transpose(0, 1).unsqueeze(0), cu.unsqueeze(0))
     assert none is None and hf.shape == (1, 260, 8, 64)
     assert torch.equal(a, b) and torch.equal(a, c) and torch.equal(a, hf[0])
+    assert torch.equal(a, M.SelfAttention._run_varlen_attn(q, k, v, cu, 160))      # models/qwen3_5/model.py:90-98
+    # two separately built offsets tensors with equal contents are accepted (torch's routine takes any two tensors);
+    # different contents are not: this operator is self-attention
+    assert torch.equal(a, M.varlen_attn(q, k, v, cu, cu.clone(), 160, 160, is_causal=True))
+    with pytest.raises(ValueError):
+        M.varlen_attn(q, k, v, cu, torch.tensor([0, 90, 260], dtype=torch.int32, device=DEV), 160, 160, is_causal=True)
     ref = R.dense_varlen_causal(q.cpu(), k.cpu(), v.cpu(), cu.cpu())
     assert_close_bf16(a, ref, "dispatch_varlen_attention")
 

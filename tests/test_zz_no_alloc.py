@@ -65,3 +65,34 @@ def test_index_topk_without_allocation_rejects_rows_beyond_the_scratch():
     rc = lib.dsa_index_topk_noalloc(_ptr(x), _ptr(x), _ptr(x), _ptr(x), limit + 64, 1, 4, 32, 8, 1.0, 0, limit + 32, _ptr(x),
                                     _ptr(x), None)
     assert rc == -3 and b"static scratch" in lib.dsa_last_error()
+
+
+def test_index_topk_without_allocation_under_graph_capture():
+    """The callers the entry point is for: a HIP graph captured around it (after one plain call on the device, which
+    looks up the scratch address) replays to the selection of dsa_index_topk, on every replay, with eager work between
+    the replays."""
+    lib = _lib.load()
+    w = W.scaled(W.C3, (1500, 40, 700), top_k=256, name="noalloc-graph")
+    t = W.make_inputs(w, device=DEV, with_dout=False)
+    cu = t["cu_seqlens"]
+    T, N, K = w.T, len(w.seg_lens), w.top_k
+    scale = (w.Di ** -0.5) * (w.Hi ** -0.5)
+    (want_idx, want_n), _ = _both(lib, w)                       # includes the plain noalloc call that precedes a capture
+    sq, sk, sw = (t[x].clone() for x in ("q_idx", "k_idx", "w_idx"))            # static inputs of the graph
+    idx = torch.full((T, K), -7, dtype=torch.int32, device=DEV)
+    n = torch.full((T,), -7, dtype=torch.int32, device=DEV)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = lib.dsa_index_topk_noalloc(_ptr(sq), _ptr(sk), _ptr(sw), _ptr(cu), T, N, w.Hi, w.Di, K, scale, 0, w.max_seqlen,
+                                        _ptr(idx), _ptr(n), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.dsa_last_error().decode()
+    for replay in range(3):
+        sq.copy_(torch.randn_like(sq))                           # other inputs first: a replay that computes nothing must not pass
+        graph.replay()
+        torch.cuda.synchronize()
+        assert not torch.equal(idx, want_idx)
+        sq.copy_(t["q_idx"])
+        _both(lib, W.scaled(W.C2, (600, 90), top_k=64, name="noalloc-between"))  # eager work on the same scratch in between
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(idx, want_idx) and torch.equal(n, want_n), f"replay {replay}"

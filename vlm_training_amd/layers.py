@@ -23,6 +23,7 @@ import torch
 import torch.nn as nn
 
 from .dtensor_utils import _dtensor_rewrap, _dtensor_unwrap, _local
+from .model_attention import run_varlen_attn
 from .ops import dsa_varlen_attn, indexer_kl_loss
 from .prologue import qk_norm_rope, sigmoid_gate
 
@@ -180,12 +181,10 @@ class SelfAttention(nn.Module):
         self.indexer = DsaIndexer(cfg.hidden_size, dsa) if dsa is not None else None
         self.indexer_loss = None
 
-    @staticmethod
-    @torch.compiler.disable
-    def _run_varlen_attn(q, k, v, cu_seqlens, max_seqlen):
-        from .model_attention import varlen_attn
-        return varlen_attn(q, k, v, cu_seq_q=cu_seqlens, cu_seq_k=cu_seqlens, max_q=max_seqlen, max_k=max_seqlen,
-                           window_size=(-1, 0))
+    # models/qwen3_5/model.py:90-98: the reference's name for the attention call of this layer (packed (T,H,D) tensors
+    # in and out, outside any compiled graph).  The layer's own forward goes through ``attention_core``, which fuses
+    # norm and RoPE in front of the same operator; this name is kept for code that calls the attention call directly.
+    _run_varlen_attn = staticmethod(run_varlen_attn)
 
     def forward(self, x, cos, sin, cu_seqlens, max_seqlen):
         total = x.shape[1]

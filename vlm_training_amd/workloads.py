@@ -52,6 +52,15 @@ class Workload:
             S += d * (d + 1) // 2 + max(0, L - self.top_k) * self.top_k
         return P, S
 
+    def executed_pairs(self, crossover: int = 16) -> Tuple[int, int]:
+        """(query side, key side): the (query, key) pairs the tile kernels put through the matrix cores.  They walk
+        whole tiles with the selection as a mask, so every causal pair of a visited tile is computed: on the query side
+        (forward, dQ) the causal pairs of the rows below the tile/gather split (positions < top_k * crossover, rounded up
+        to 256), on the key side (dK/dV) every causal pair."""
+        split = (self.top_k * crossover + 255) // 256 * 256
+        q_side = sum(min(L, split) * (min(L, split) + 1) // 2 for L in self.seg_lens)
+        return q_side, self.pair_counts()[0]
+
     def work(self) -> Dict[str, float]:
         """Algorithmic flop / byte counts per fwd+bwd pass (bf16 element = 2 bytes)."""
         P, S = self.pair_counts()
