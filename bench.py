@@ -228,6 +228,8 @@ def main():
     ap.add_argument("--crossover", type=int, default=None,
                     help="tile/gather split (rows with pos < top_k * crossover run on the tile kernels; 0 = gather kernels only)")
     ap.add_argument("--only-step", action="store_true", help="the timed steps and the roofline line only (for profiler runs)")
+    ap.add_argument("--indexer-training", action="store_true",
+                    help="with --only-step: also run the indexer's training path (mass, selected scores, KL, indexer backward)")
     ap.add_argument("--head-shard", type=int, default=1,
                     help="measure one GPU's share of the workload with the attention heads split this many ways (the "
                          "reference's tensor parallelism); implies --only-step")
@@ -377,7 +379,8 @@ def main():
         result["adjacent_kernels"] = prologue_stage(w, dev, it)
         result["reference_operator"] = reference_operator(w, t, it)
         result["vision_tower_operator"] = vision_tower_operator(dev, it)
-        result["indexer_training"] = indexer_target_stage(w, t, it)
+    if not args.only_step or args.indexer_training:
+        result["indexer_training"] = indexer_target_stage(w, t, min(it, 5))
     if not args.no_cpu_baseline and not args.only_step:
         result["cpu_baseline"] = cpu_baseline(w, torch.get_num_threads(), sample_only=args.cpu_sample)
     print(json.dumps(result))
