@@ -144,7 +144,9 @@ def test_long_single_sequence_by_invariants_and_sampled_rows():
     want = t["dout"].float().sum(0).view(w.Hkv, G, w.D).sum(1)
     assert torch.allclose(dv.float().sum(0), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
     # sampled rows: around top_k, around the select kernel's LDS cache, around the tile/gather crossover, the end
-    rows = [0, 1, K - 1, K, K + 1, 8191, 8192, 8193, 16 * K - 1, 16 * K, 16 * K + 1, 65535, 100003, T - 2, T - 1]
+    X = lib.dsa_get_tile_crossover() * K                 # first row of the gather kernels (a multiple of 256 here)
+    assert K < X < T and X % 256 == 0
+    rows = [0, 1, K - 1, K, K + 1, 8191, 8192, 8193, X - 1, X, X + 1, 65535, 100003, T - 2, T - 1]
     scale = (w.Di ** -0.5) * (w.Hi ** -0.5)
     st = torch.cuda.current_stream().cuda_stream
     row_sc = torch.empty((1, T), dtype=torch.float32, device=DEV)
@@ -170,7 +172,7 @@ def test_long_single_sequence_by_invariants_and_sampled_rows():
     _log(f"  C4 sampled rows: out ({e1[0]:.2e},{e1[1]:.6f}) dq ({e2[0]:.2e},{e2[1]:.6f})")
     # dk and dv of sampled key rows (first key tile, around top_k, around the select cache and the tile/gather crossover,
     # the last tile): every query that selected the key is looked up in idx and attended over its own keys by the oracle
-    keys = [17, K, 8192, 16 * K, 100003, T - 70, T - 1]
+    keys = [17, K, 8192, X, 100003, T - 70, T - 1]
     want_dk, want_dv = R.sparse_attention_key_rows(t["q"].cpu(), t["k"].cpu(), t["v"].cpu(), t["dout"].cpu(), idx_c, n_c, keys)
     e3 = assert_close_bf16(dk[keys], want_dk, "dk (sampled key rows)")
     e4 = assert_close_bf16(dv[keys], want_dv, "dv (sampled key rows)")

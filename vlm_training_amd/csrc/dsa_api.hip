@@ -253,7 +253,7 @@ static inline int bitmap_ldw(int max_seqlen) { return (max_seqlen + 31) / 32; }
 // Query rows whose position in their segment is below top_k * crossover are handled by the tile
 // kernels (their selection covers more than 1/crossover of the causal window), the rest by the
 // gather kernels.  Process-wide tuning knob; 0 = gather only, a huge value = tile only.
-static std::atomic<int> g_tile_crossover{16};          // read on every launch, possibly from several host threads
+static std::atomic<int> g_tile_crossover{24};          // read on every launch, possibly from several host threads
 extern "C" int dsa_set_tile_crossover(int crossover) {
     if (crossover < 0) return fail(DSA_ERR_ARG, "crossover=%d must be >= 0", crossover);
     g_tile_crossover.store(crossover, std::memory_order_relaxed);

@@ -52,7 +52,7 @@ class Workload:
             S += d * (d + 1) // 2 + max(0, L - self.top_k) * self.top_k
         return P, S
 
-    def executed_pairs(self, crossover: int = 16) -> Tuple[int, int]:
+    def executed_pairs(self, crossover: int = 24) -> Tuple[int, int]:
         """(query side, key side): the (query, key) pairs the tile kernels put through the matrix cores.  They walk
         whole tiles with the selection as a mask, so every causal pair of a visited tile is computed: on the query side
         (forward, dQ) the causal pairs of the rows below the tile/gather split (positions < top_k * crossover, rounded up
