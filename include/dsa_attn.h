@@ -237,26 +237,29 @@ int dsa_dense_bwd(const void *dout, const void *q, const void *k, const void *v,
  *
  * dsa_qk_norm_rope_fwd stands for, in one pass over q and k (models/qwen3_vl/model.py:256-269,
  * models/qwen3_5/model.py:110-129): `q_norm(q)`, `k_norm(k)` = F.rms_norm over head_dim with weight `w`
- * (`w_offset` = 0) or `1 + w` (`w_offset` = 1, OffsetRMSNorm, models/qwen3_5/model.py:58-72), the two
+ * or `1 + w` (`norm_flags & DSA_NORM_OFFSET`: OffsetRMSNorm, models/qwen3_5/model.py:58-72), the two
  * transposes, `apply_rope(q, k, cos, sin)` (models/qwen3_vl/model.py:181-193; partial rotary width
  * R <= D: models/qwen3_5/utils.py:88-110) and the `.contiguous()` copies into (T, H, D).
  *   q_in, k_in: bf16, element (t, h, d) at  base + t*tok_stride + h*head_stride + d  (strides in elements,
  *               so the q half of Qwen3.5's interleaved [q | gate] projection can be read in place);
- *   qw, kw: fp32 (D);  cos, sin: (T, R) bf16 (cs_dtype DSA_DTYPE_BF16) or fp32 (DSA_DTYPE_FP32), R % 16 == 0;
+ *   qw, kw: (D) fp32, or bf16 with `norm_flags & DSA_NORM_WEIGHT_BF16` (read as the module holds them: no cast
+ *           kernel in front of the call);  cos, sin: (T, R) bf16 (cs_dtype DSA_DTYPE_BF16) or fp32 (DSA_DTYPE_FP32), R % 16 == 0;
  *   q_out (T,Hq,D), k_out (T,Hkv,D) bf16 contiguous;  q_rstd (T,Hq), k_rstd (T,Hkv) fp32: 1/rms of
  *   every row, kept for the backward pass.  D in {64, 128, 256}.
  * dsa_qk_norm_rope_bwd: gq, gk = gradients of q_out, k_out (same layout) -> dq_in, dk_in (strided like
  * the inputs, bf16) and dqw, dkw (D) fp32.  `ws` holds dsa_qk_norm_rope_bwd_workspace_bytes(T, D) bytes
  * of per-workgroup partial sums that are added up in a fixed order (no atomics, deterministic).
  */
+#define DSA_NORM_OFFSET 1      /* scale by 1 + w */
+#define DSA_NORM_WEIGHT_BF16 2 /* qw, kw point at bf16 */
 size_t dsa_qk_norm_rope_bwd_workspace_bytes(int T, int D);
 int dsa_qk_norm_rope_fwd(const void *q_in, int64_t q_tok_stride, int64_t q_head_stride, const void *k_in,
-                         int64_t k_tok_stride, int64_t k_head_stride, const float *qw, const float *kw, float eps,
-                         int w_offset, const void *cos, const void *sin, int cs_dtype, int R, int T, int Hq, int Hkv,
+                         int64_t k_tok_stride, int64_t k_head_stride, const void *qw, const void *kw, float eps,
+                         int norm_flags, const void *cos, const void *sin, int cs_dtype, int R, int T, int Hq, int Hkv,
                          int D, void *q_out, void *k_out, float *q_rstd, float *k_rstd, void *stream);
 int dsa_qk_norm_rope_bwd(const void *gq, const void *gk, const void *q_in, int64_t q_tok_stride, int64_t q_head_stride,
-                         const void *k_in, int64_t k_tok_stride, int64_t k_head_stride, const float *qw, const float *kw,
-                         int w_offset, const void *cos, const void *sin, int cs_dtype, int R, const float *q_rstd,
+                         const void *k_in, int64_t k_tok_stride, int64_t k_head_stride, const void *qw, const void *kw,
+                         int norm_flags, const void *cos, const void *sin, int cs_dtype, int R, const float *q_rstd,
                          const float *k_rstd, int T, int Hq, int Hkv, int D, void *dq_in, int64_t dq_tok_stride,
                          int64_t dq_head_stride, void *dk_in, int64_t dk_tok_stride, int64_t dk_head_stride, float *dqw,
                          float *dkw, void *ws, size_t ws_bytes, void *stream);

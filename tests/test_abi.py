@@ -46,7 +46,17 @@ def test_workspace_sizes_without_a_gpu():
     assert lib.dsa_attn_bwd_bitmap_offset(1000, 8) == up(1000 * 8 * 4)   # forward workspace fits behind it
     assert lib.dsa_attn_fwd_workspace_bytes(1000, 640, 0) == 0
     old = lib.dsa_get_tile_crossover()
-    assert old == 16 and lib.dsa_set_tile_crossover(-1) == -1 and lib.dsa_set_tile_crossover(3) == 0
+    # what the backward allocates when it runs: delta, the key-tile order, and partial sums only for launches small
+    # enough to be cut into pieces (at most 1024 key-tile workgroups); the bitmap stays in the forward's workspace
+    order_of = lambda T: up(((T // 128 + 4096 + 1 + 4096) * 5 + 4) * 4)
+    assert lib.dsa_attn_bwd_scratch_bytes(32768, 8, 32, 8, 128) == up(32768 * 32 * 4) + order_of(32768)
+    assert lib.dsa_attn_bwd_scratch_bytes(8192, 7, 16, 8, 128) == up(8192 * 16 * 4) + up(8192 * 16384) + order_of(8192)
+    # attention mass: the bitmap alone when one workgroup holds every kv head (8 at head_dim 128, 4 at 256), else a
+    # (T,K) table per group of kv heads
+    assert lib.dsa_attn_mass_workspace_bytes(32768, 8, 32, 8, 128, 2048, 7168) == up(32768 * 224 * 4)
+    assert lib.dsa_attn_mass_workspace_bytes(16384, 33, 16, 2, 256, 512, 1669) == up(16384 * 53 * 4)
+    assert lib.dsa_attn_mass_workspace_bytes(1000, 3, 32, 16, 128, 64, 640) == up(1000 * 20 * 4) + up(2 * 1000 * 64 * 4)
+    assert old == 24 and lib.dsa_set_tile_crossover(-1) == -1 and lib.dsa_set_tile_crossover(3) == 0
     assert lib.dsa_get_tile_crossover() == 3 and lib.dsa_set_tile_crossover(old) == 0
 
 

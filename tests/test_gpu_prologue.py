@@ -66,6 +66,11 @@ def test_qk_norm_rope_forward_and_backward(T, Hq, Hkv, D, R, offset, cs, inter):
     torch.cuda.synchronize()
     assert_close_bf16(oq, want_q, "q_out")
     assert_close_bf16(ok, want_k, "k_out")
+    # the weights are read as the module holds them: fp32 parameters with the same values give the same bits
+    with torch.no_grad():
+        oq32, ok32 = prologue.qk_norm_rope(qd.detach(), kd.detach(), qw.float().to(DEV), kw.float().to(DEV), cos.to(DEV), sin.to(DEV),
+                                           1e-6, offset)
+    assert torch.equal(oq32, oq) and torch.equal(ok32, ok)
     # against an evaluation that never rounds: the reference (and the kernel, and `want_q` above) rounds F.rms_norm's
     # result to bf16 before the rotation, so the rotated value x*cos + rot(x)*sin carries up to (|cos| + |sin|)/2 <= 0.71
     # steps of that first rounding plus half a step of the final one - two bf16 steps bound it

@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libdsa_attn.so")
 
 DSA_DTYPE_BF16 = 0
 DSA_DTYPE_FP32 = 1
+DSA_NORM_OFFSET, DSA_NORM_WEIGHT_BF16 = 1, 2                                               # norm_flags of the prologue
 DSA_BWD_DELTA, DSA_BWD_BITMAP, DSA_BWD_DQ, DSA_BWD_DKV, DSA_BWD_ALL = 1, 2, 4, 8, 15      # parts of dsa_attn_bwd_parts
 
 _SIGNATURES = {

@@ -55,12 +55,12 @@ int dsa_mass_groups(int Hq, int Hkv, int D);
 extern "C" {
 int dsa_prologue_bwd_blocks(int T);
 hipError_t dsa_launch_qk_norm_rope_fwd(const void *q_in, int64_t q_tok, int64_t q_head, const void *k_in, int64_t k_tok,
-                                       int64_t k_head, const float *qw, const float *kw, float eps, float w_offset,
+                                       int64_t k_head, const void *qw, const void *kw, int w_bf16, float eps, float w_offset,
                                        const void *cosp, const void *sinp, int cs_f32, int R, int T, int Hq, int Hkv, int D,
                                        void *q_out, void *k_out, float *q_rstd, float *k_rstd, hipStream_t stream);
 hipError_t dsa_launch_qk_norm_rope_bwd(const void *gq, const void *gk, const void *q_in, int64_t q_tok, int64_t q_head,
-                                       const void *k_in, int64_t k_tok, int64_t k_head, const float *qw, const float *kw,
-                                       float w_offset, const void *cosp, const void *sinp, int cs_f32, int R,
+                                       const void *k_in, int64_t k_tok, int64_t k_head, const void *qw, const void *kw,
+                                       int w_bf16, float w_offset, const void *cosp, const void *sinp, int cs_f32, int R,
                                        const float *q_rstd, const float *k_rstd, int T, int Hq, int Hkv, int D, void *dq_in,
                                        int64_t dq_tok, int64_t dq_head, void *dk_in, int64_t dk_tok, int64_t dk_head,
                                        float *dqw, float *dkw, float *part, hipStream_t stream);
@@ -526,22 +526,23 @@ extern "C" size_t dsa_qk_norm_rope_bwd_workspace_bytes(int T, int D) {
 }
 
 extern "C" int dsa_qk_norm_rope_fwd(const void *q_in, int64_t q_tok, int64_t q_head, const void *k_in, int64_t k_tok,
-                                    int64_t k_head, const float *qw, const float *kw, float eps, int w_offset,
+                                    int64_t k_head, const void *qw, const void *kw, float eps, int norm_flags,
                                     const void *cosp, const void *sinp, int cs_dtype, int R, int T, int Hq, int Hkv, int D,
                                     void *q_out, void *k_out, float *q_rstd, float *k_rstd, void *stream) {
     if (int rc = check_prologue(T, Hq, Hkv, D, R, cs_dtype, q_head, k_head)) return rc;
     if (!q_in || !k_in || !qw || !kw || !q_out || !k_out || !q_rstd || !k_rstd || (R > 0 && (!cosp || !sinp)))
         return fail(DSA_ERR_ARG, "null tensor pointer");
     if (q_tok % 8 || k_tok % 8) return fail(DSA_ERR_ARG, "token strides must be multiples of 8 elements");
-    hipError_t e = dsa_launch_qk_norm_rope_fwd(q_in, q_tok, q_head, k_in, k_tok, k_head, qw, kw, eps, w_offset ? 1.f : 0.f,
+    hipError_t e = dsa_launch_qk_norm_rope_fwd(q_in, q_tok, q_head, k_in, k_tok, k_head, qw, kw, (norm_flags & DSA_NORM_WEIGHT_BF16) != 0, eps,
+                                               (norm_flags & DSA_NORM_OFFSET) ? 1.f : 0.f,
                                                cosp, sinp, cs_dtype == DSA_DTYPE_FP32, R, T, Hq, Hkv, D, q_out, k_out, q_rstd,
                                                k_rstd, (hipStream_t)stream);
     return e == hipSuccess ? DSA_OK : hip_fail(e, "qk_norm_rope forward launch");
 }
 
 extern "C" int dsa_qk_norm_rope_bwd(const void *gq, const void *gk, const void *q_in, int64_t q_tok, int64_t q_head,
-                                    const void *k_in, int64_t k_tok, int64_t k_head, const float *qw, const float *kw,
-                                    int w_offset, const void *cosp, const void *sinp, int cs_dtype, int R,
+                                    const void *k_in, int64_t k_tok, int64_t k_head, const void *qw, const void *kw,
+                                    int norm_flags, const void *cosp, const void *sinp, int cs_dtype, int R,
                                     const float *q_rstd, const float *k_rstd, int T, int Hq, int Hkv, int D, void *dq_in,
                                     int64_t dq_tok, int64_t dq_head, void *dk_in, int64_t dk_tok, int64_t dk_head,
                                     float *dqw, float *dkw, void *ws, size_t ws_bytes, void *stream) {
@@ -553,7 +554,8 @@ extern "C" int dsa_qk_norm_rope_bwd(const void *gq, const void *gk, const void *
         return fail(DSA_ERR_ARG, "strides must be multiples of 8 elements");
     const size_t need = dsa_qk_norm_rope_bwd_workspace_bytes(T, D);
     if (need && (!ws || ws_bytes < need)) return fail(DSA_ERR_WORKSPACE, "prologue backward workspace: have %zu bytes, need %zu", ws_bytes, need);
-    hipError_t e = dsa_launch_qk_norm_rope_bwd(gq, gk, q_in, q_tok, q_head, k_in, k_tok, k_head, qw, kw, w_offset ? 1.f : 0.f,
+    hipError_t e = dsa_launch_qk_norm_rope_bwd(gq, gk, q_in, q_tok, q_head, k_in, k_tok, k_head, qw, kw, (norm_flags & DSA_NORM_WEIGHT_BF16) != 0,
+                                               (norm_flags & DSA_NORM_OFFSET) ? 1.f : 0.f,
                                                cosp, sinp, cs_dtype == DSA_DTYPE_FP32, R, q_rstd, k_rstd, T, Hq, Hkv, D, dq_in,
                                                dq_tok, dq_head, dk_in, dk_tok, dk_head, dqw, dkw, (float *)ws,
                                                (hipStream_t)stream);

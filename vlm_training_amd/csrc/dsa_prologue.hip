@@ -52,10 +52,15 @@ __device__ __forceinline__ float row_sum(float x) {
     return x;
 }
 
+// a norm weight as the module holds it: fp32 (the trainer's master parameters under autocast) or bf16
+__device__ __forceinline__ float norm_weight(const void *w, int w_bf16, int d) {
+    return w_bf16 ? (float)reinterpret_cast<const bf16_t *>(w)[d] : reinterpret_cast<const float *>(w)[d];
+}
+
 template <int D, bool CS_F32>
 __global__ __launch_bounds__(256) void dsa_qk_norm_rope_fwd_kernel(
     const bf16_t *__restrict__ q_in, int64_t q_tok, int64_t q_head, const bf16_t *__restrict__ k_in, int64_t k_tok,
-    int64_t k_head, const float *__restrict__ qw, const float *__restrict__ kw, float eps, float w_offset,
+    int64_t k_head, const void *__restrict__ qw, const void *__restrict__ kw, int w_bf16, float eps, float w_offset,
     const void *__restrict__ cosp, const void *__restrict__ sinp, int R, int T, int Hq, int Hkv,
     bf16_t *__restrict__ q_out, bf16_t *__restrict__ k_out, float *__restrict__ q_rstd, float *__restrict__ k_rstd) {
     constexpr int LPR = D / 8, RPW = 64 / LPR;           // lanes per row, rows per wave and step
@@ -65,7 +70,7 @@ __global__ __launch_bounds__(256) void dsa_qk_norm_rope_fwd_kernel(
     const bool low = d0 < R / 2, rot = d0 < R;
     f32x8 wq, wk;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { wq[i] = qw[d0 + i] + w_offset; wk[i] = kw[d0 + i] + w_offset; }
+    for (int i = 0; i < 8; ++i) { wq[i] = norm_weight(qw, w_bf16, d0 + i) + w_offset; wk[i] = norm_weight(kw, w_bf16, d0 + i) + w_offset; }
     for (int64_t t = (int64_t)blockIdx.x * 4 + wv; t < T; t += (int64_t)gridDim.x * 4) {
         f32x8 c, s;
         load_cs<CS_F32>(cosp, t, R, d0, c, 1.f);
@@ -105,8 +110,8 @@ __global__ __launch_bounds__(256) void dsa_qk_norm_rope_fwd_kernel(
 template <int D, bool CS_F32>
 __global__ __launch_bounds__(256) void dsa_qk_norm_rope_bwd_kernel(
     const bf16_t *__restrict__ gq, const bf16_t *__restrict__ gk, const bf16_t *__restrict__ q_in, int64_t q_tok,
-    int64_t q_head, const bf16_t *__restrict__ k_in, int64_t k_tok, int64_t k_head, const float *__restrict__ qw,
-    const float *__restrict__ kw, float w_offset, const void *__restrict__ cosp, const void *__restrict__ sinp, int R,
+    int64_t q_head, const bf16_t *__restrict__ k_in, int64_t k_tok, int64_t k_head, const void *__restrict__ qw,
+    const void *__restrict__ kw, int w_bf16, float w_offset, const void *__restrict__ cosp, const void *__restrict__ sinp, int R,
     const float *__restrict__ q_rstd, const float *__restrict__ k_rstd, int T, int Hq, int Hkv,
     bf16_t *__restrict__ dq_in, int64_t dq_tok, int64_t dq_head, bf16_t *__restrict__ dk_in, int64_t dk_tok,
     int64_t dk_head, float *__restrict__ part) {
@@ -118,7 +123,7 @@ __global__ __launch_bounds__(256) void dsa_qk_norm_rope_bwd_kernel(
     const bool low = d0 < R / 2, rot = d0 < R;
     f32x8 wq, wk, aq, ak;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { wq[i] = qw[d0 + i] + w_offset; wk[i] = kw[d0 + i] + w_offset; aq[i] = 0.f; ak[i] = 0.f; }
+    for (int i = 0; i < 8; ++i) { wq[i] = norm_weight(qw, w_bf16, d0 + i) + w_offset; wk[i] = norm_weight(kw, w_bf16, d0 + i) + w_offset; aq[i] = 0.f; ak[i] = 0.f; }
     for (int64_t t = (int64_t)blockIdx.x * 4 + wv; t < T; t += (int64_t)gridDim.x * 4) {
         f32x8 c, s;
         load_cs<CS_F32>(cosp, t, R, d0, c, 1.f);
@@ -260,20 +265,20 @@ extern "C" int dsa_prologue_bwd_blocks(int T) { return prologue_blocks(T); }
     }
 
 extern "C" hipError_t dsa_launch_qk_norm_rope_fwd(const void *q_in, int64_t q_tok, int64_t q_head, const void *k_in,
-                                                  int64_t k_tok, int64_t k_head, const float *qw, const float *kw, float eps,
+                                                  int64_t k_tok, int64_t k_head, const void *qw, const void *kw, int w_bf16, float eps,
                                                   float w_offset, const void *cosp, const void *sinp, int cs_f32, int R, int T,
                                                   int Hq, int Hkv, int D, void *q_out, void *k_out, float *q_rstd,
                                                   float *k_rstd, hipStream_t stream) {
     if (T == 0) return hipSuccess;
     PROLOGUE_SWITCH(dsa_qk_norm_rope_fwd_kernel, dim3(prologue_blocks(T)), dim3(256), 0, stream, (const bf16_t *)q_in, q_tok,
-                    q_head, (const bf16_t *)k_in, k_tok, k_head, qw, kw, eps, w_offset, cosp, sinp, R, T, Hq, Hkv,
+                    q_head, (const bf16_t *)k_in, k_tok, k_head, qw, kw, w_bf16, eps, w_offset, cosp, sinp, R, T, Hq, Hkv,
                     (bf16_t *)q_out, (bf16_t *)k_out, q_rstd, k_rstd)
     return hipGetLastError();
 }
 
 extern "C" hipError_t dsa_launch_qk_norm_rope_bwd(const void *gq, const void *gk, const void *q_in, int64_t q_tok,
                                                   int64_t q_head, const void *k_in, int64_t k_tok, int64_t k_head,
-                                                  const float *qw, const float *kw, float w_offset, const void *cosp,
+                                                  const void *qw, const void *kw, int w_bf16, float w_offset, const void *cosp,
                                                   const void *sinp, int cs_f32, int R, const float *q_rstd,
                                                   const float *k_rstd, int T, int Hq, int Hkv, int D, void *dq_in,
                                                   int64_t dq_tok, int64_t dq_head, void *dk_in, int64_t dk_tok,
@@ -281,7 +286,7 @@ extern "C" hipError_t dsa_launch_qk_norm_rope_bwd(const void *gq, const void *gk
     const int nb = prologue_blocks(T);
     if (T > 0) {
         PROLOGUE_SWITCH(dsa_qk_norm_rope_bwd_kernel, dim3(nb), dim3(256), 0, stream, (const bf16_t *)gq, (const bf16_t *)gk,
-                        (const bf16_t *)q_in, q_tok, q_head, (const bf16_t *)k_in, k_tok, k_head, qw, kw, w_offset, cosp, sinp,
+                        (const bf16_t *)q_in, q_tok, q_head, (const bf16_t *)k_in, k_tok, k_head, qw, kw, w_bf16, w_offset, cosp, sinp,
                         R, q_rstd, k_rstd, T, Hq, Hkv, (bf16_t *)dq_in, dq_tok, dq_head, (bf16_t *)dk_in, dk_tok, dk_head, part)
     }
     hipLaunchKernelGGL(dsa_norm_weight_reduce_kernel, dim3(2 * D / 64), dim3(1024), 0, stream, part, T > 0 ? nb : 0, D, dqw,

@@ -48,25 +48,30 @@ class _QkNormRope(torch.autograd.Function):
         (qt, qh), (kt, kh) = _thd_strides(q, "q"), _thd_strides(k, "k")
         cos, sin, cs_code = _cs(cos, sin, T)
         R = cos.shape[1]
-        qw, kw = q_weight.detach().float().contiguous(), k_weight.detach().float().contiguous()
+        # the weights go in as the module holds them (fp32 master parameters, or bf16): a cast in front of the call would
+        # be two more kernels per layer
+        qw, kw = q_weight.detach().contiguous(), k_weight.detach().contiguous()
+        if qw.dtype != kw.dtype or qw.dtype not in (torch.float32, torch.bfloat16):
+            qw, kw = qw.float(), kw.float()
         if qw.numel() != D or kw.numel() != D:
             raise ValueError("norm weights must have head_dim elements")
+        flags = (_lib.DSA_NORM_OFFSET if offset else 0) | (_lib.DSA_NORM_WEIGHT_BF16 if qw.dtype == torch.bfloat16 else 0)
         q_out = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=q.device)
         k_out = torch.empty((T, Hkv, D), dtype=torch.bfloat16, device=q.device)
         q_rstd = torch.empty((T, Hq), dtype=torch.float32, device=q.device)
         k_rstd = torch.empty((T, Hkv), dtype=torch.float32, device=q.device)
         rc = _lib.load().dsa_qk_norm_rope_fwd(_ptr(q), qt, qh, _ptr(k), kt, kh, _ptr(qw), _ptr(kw), float(eps),
-                                              1 if offset else 0, _ptr(cos), _ptr(sin), cs_code, R, T, Hq, Hkv, D,
+                                              flags, _ptr(cos), _ptr(sin), cs_code, R, T, Hq, Hkv, D,
                                               _ptr(q_out), _ptr(k_out), _ptr(q_rstd), _ptr(k_rstd), _stream(q.device))
         _lib.check(rc, "dsa_qk_norm_rope_fwd")
         ctx.save_for_backward(q, k, qw, kw, cos, sin, q_rstd, k_rstd)
-        ctx.meta = (cs_code, R, bool(offset), q_weight.dtype, k_weight.dtype)
+        ctx.meta = (cs_code, R, flags, q_weight.dtype, k_weight.dtype)
         return q_out, k_out
 
     @staticmethod
     def backward(ctx, gq, gk):
         q, k, qw, kw, cos, sin, q_rstd, k_rstd = ctx.saved_tensors
-        cs_code, R, offset, qw_dtype, kw_dtype = ctx.meta
+        cs_code, R, flags, qw_dtype, kw_dtype = ctx.meta
         T, Hq, D = q.shape
         Hkv = k.shape[1]
         gq, gk = gq.contiguous().to(torch.bfloat16), gk.contiguous().to(torch.bfloat16)
@@ -78,7 +83,7 @@ class _QkNormRope(torch.autograd.Function):
         ws_bytes = lib.dsa_qk_norm_rope_bwd_workspace_bytes(T, D)
         ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q.device)
         rc = lib.dsa_qk_norm_rope_bwd(_ptr(gq), _ptr(gk), _ptr(q), q.stride(0), q.stride(1), _ptr(k), k.stride(0),
-                                      k.stride(1), _ptr(qw), _ptr(kw), 1 if offset else 0, _ptr(cos), _ptr(sin), cs_code,
+                                      k.stride(1), _ptr(qw), _ptr(kw), flags, _ptr(cos), _ptr(sin), cs_code,
                                       R, _ptr(q_rstd), _ptr(k_rstd), T, Hq, Hkv, D, _ptr(dq), Hq * D, D, _ptr(dk), Hkv * D,
                                       D, _ptr(dqw), _ptr(dkw), _ptr(ws), ws_bytes, _stream(q.device))
         _lib.check(rc, "dsa_qk_norm_rope_bwd")
