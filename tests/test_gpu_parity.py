@@ -187,10 +187,12 @@ def test_sparse_path_odd_head_groups(Hq, Hkv, D):
         ops.set_tile_crossover(old)
 
 
-@pytest.mark.parametrize("n_short", [300, 4500])
+@pytest.mark.parametrize("n_short", [63, 64, 65, 300, 4500])
 def test_many_segments_in_every_launch_order_of_the_key_tiles(n_short):
     """dK/dV lists its key tiles longest walk first; 300 segments go through the order table, 4500 are more than
-    it holds (plain order).  Lengths 0-3 with two long segments between them."""
+    it holds (plain order).  The query-side kernels hand their blocks out heaviest first over the whole batch for up to
+    64 segments (a wave holds the lengths in its lanes) and segment by segment beyond: 63, 64 and 65 segments sit on
+    both sides of that.  Lengths 0-3 with two long segments between them."""
     _log(f"many segments {n_short}")
     g = torch.Generator().manual_seed(23 + n_short)
     lens = torch.randint(0, 4, (n_short,), generator=g).tolist()
