@@ -376,3 +376,36 @@ def test_head_sharded_dtensor_projections_pass_through_layer_kernel_and_rewrap(k
         _restore(undo)
         if created:
             dist.destroy_process_group()
+
+
+@pytest.mark.parametrize("sparse", [False, True])
+def test_layer_under_activation_checkpointing_recomputes_to_the_same_bits(sparse):
+    """train/infra.py:187-195 wraps every block in torch's checkpoint wrapper: the forward runs a second time inside the
+    backward.  The operator keeps no state between calls and is deterministic, so a checkpointed layer must give the
+    output and the gradients of the plain one bit for bit (the selection included: it is recomputed, not saved)."""
+    _log(f"activation checkpointing, sparse={sparse}")
+    from torch.utils.checkpoint import checkpoint
+    hidden, Hq, Hkv, D = 256, 8, 2, 128
+    dsa = DsaConfig(index_heads=8, index_dim=64, top_k=64) if sparse else None
+    m = _make(Qwen3VLTextAttention, _cfg(hidden, Hq, Hkv, D), dsa, seed=41, param_dtype=torch.bfloat16)
+    if sparse:
+        for p in m.indexer.parameters():                   # the indexer's own loss is not what is checked here
+            p.requires_grad_(False)
+    cu = [0, 300, 700, 1024]
+    T = cu[-1]
+    g = torch.Generator().manual_seed(42)
+    x_cpu = torch.randn(1, T, hidden, generator=g).bfloat16()
+    gy = torch.randn(1, T, hidden, generator=g).bfloat16().to(DEV)
+    cos, sin = (t.to(DEV).to(torch.bfloat16) for t in _tables(T, D, torch.float32))
+    cu_d = torch.tensor(cu, dtype=torch.int32, device=DEV)
+    results = []
+    for wrapped in (False, True):
+        for p in m.parameters():
+            p.grad = None
+        x = x_cpu.to(DEV).requires_grad_(True)
+        y = checkpoint(m, x, cos, sin, cu_d, 512, use_reentrant=False) if wrapped else m(x, cos, sin, cu_d, 512)
+        y.backward(gy)
+        results.append([y.detach().clone(), x.grad.clone()] + [p.grad.clone() for p in m.parameters() if p.grad is not None])
+    assert len(results[0]) == len(results[1]) >= 8
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
