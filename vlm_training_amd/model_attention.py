@@ -74,6 +74,7 @@ def _hf_indexer_to_packed(x):
 _BOUND_ATTR = "_dsa_longest_segment"      # (version, storage offset, numel, bound), kept on the tensor that owns the memory
 
 
+@torch.compiler.disable                 # reads a value back from the device and writes an attribute: never part of a traced graph
 def longest_segment(cu_seqlens) -> int:
     """Longest segment of a packed row, read back from the device once per ``cu_seqlens`` tensor: every layer of a
     step hands over the same tensor (or a view of it), so the copy (and its stall) is paid once per batch instead of
