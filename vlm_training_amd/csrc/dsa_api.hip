@@ -42,7 +42,8 @@ hipError_t dsa_launch_tile_fwd(const void *q, const void *k, const void *v, cons
                                int causal, void *out, float *lse, hipStream_t stream);
 hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const void *k, const void *v, const float *lse,
                               const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T,
-                              int Hq, int Hkv, int D, float scale, int pos_split, int causal, void *dq, hipStream_t stream);
+                              int Hq, int Hkv, int D, float scale, int pos_split, int causal, void *dq, const void *out_for_delta,
+                              float *delta_out, hipStream_t stream);
 hipError_t dsa_launch_tile_dkv(const void *dout, const void *q, const void *k, const void *v, const float *lse,
                                const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N, int T,
                                int Hq, int Hkv, int D, float scale, int causal, int32_t *order, float *partial,
@@ -394,7 +395,10 @@ static int attn_bwd_run(const void *dout, const void *q, const void *k, const vo
     if (idx && (size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);
     const int split = pos_split_for(idx, K);
     hipError_t e = hipSuccess;
-    if (parts & DSA_BWD_DELTA) {
+    // delta = rowsum(dO * O): a pass of its own, unless the tile dQ kernel of the same call owns every query row
+    // (no row beyond the tile/gather split) - then that kernel forms it from the dO rows it loads anyway
+    const bool fuse_delta = (parts & DSA_BWD_DELTA) && (parts & DSA_BWD_DQ) && split > 0 && max_seqlen <= split;
+    if ((parts & DSA_BWD_DELTA) && !fuse_delta) {
         e = dsa_launch_delta(dout, out, T, Hq, D, delta, st);
         if (e != hipSuccess) return hip_fail(e, "delta launch");
     }
@@ -404,7 +408,8 @@ static int attn_bwd_run(const void *dout, const void *q, const void *k, const vo
     }
     if (parts & DSA_BWD_DQ) {
         if (split > 0) {
-            e = dsa_launch_tile_dq(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, split, causal, dq, st);
+            e = dsa_launch_tile_dq(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, split, causal, dq,
+                                   fuse_delta ? out : nullptr, delta, st);
             if (e != hipSuccess) return hip_fail(e, "tile dq launch");
         }
         if (max_seqlen > split) {

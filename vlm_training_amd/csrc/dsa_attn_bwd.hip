@@ -12,7 +12,8 @@
 #include "dsa_common.h"
 
 // ------------------------------------------------------------------------------------------------
-// delta: 16 lanes per (t,h) row
+// delta: 16 lanes per (t,h) row; lane i sums the 8-element chunks i, i+16, ... in one chain, then a butterfly over the 16
+// lanes (dsa_tile_dq_kernel reproduces this order when it forms delta itself)
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void dsa_bwd_delta_kernel(const bf16_t *__restrict__ dout,
                                                             const bf16_t *__restrict__ out, int T, int Hq, int D,
@@ -22,9 +23,7 @@ __global__ __launch_bounds__(256) void dsa_bwd_delta_kernel(const bf16_t *__rest
     float acc = 0.f;
     if (row < (int64_t)T * Hq) {
         for (int c = sub * 8; c < D; c += 128) {
-            const bf16x8 a = load_bf16x8(dout + row * D + c), b = load_bf16x8(out + row * D + c);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) acc += (float)a[e] * (float)b[e];
+            acc = dot8_chain(load_bf16x8(dout + row * D + c), load_bf16x8(out + row * D + c), acc);
         }
     }
 #pragma unroll

@@ -860,9 +860,10 @@ __global__ __launch_bounds__(64) void dsa_bitmap_prefix_kernel(const uint32_t *_
 template <int D, bool HAS_IDX, int GSHIFT, int NW>
 __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_tile_dq_kernel(
     const bf16_t *__restrict__ dout, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
-    const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
+    const bf16_t *__restrict__ v, const float *__restrict__ lse, const float *delta,
     const uint32_t *__restrict__ bitmap, int ldw, const int32_t *__restrict__ cu, int N, int T, int Hq, int Hkv,
-    float scale, int pos_split, int causal, bf16_t *__restrict__ dq) {
+    float scale, int pos_split, int causal, bf16_t *__restrict__ dq, const bf16_t *__restrict__ out_for_delta,
+    float *delta_out) {
     constexpr int KS = D / 16, DT = D / 32, CPR = D / 8, TILE_B = tile_bytes<D>();
     constexpr int NBUF = (D > 128) ? 1 : 2;
     constexpr int NT = NW * 64, Gp = 1 << GSHIFT, QBW = (NW * 32) >> GSHIFT;
@@ -906,7 +907,32 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     // the two accumulators of a tile start from -lse/scale and -delta of the lane's row, so that S - lse/scale and
     // dP - delta come out of the MFMAs (one multiply per element instead of a multiply-add and a subtraction)
     const float neg_lse = -lse[(int64_t)hq * T + t] / scale;
-    const float neg_dlt = -delta[(int64_t)hq * T + t];
+    // delta = rowsum(dO * O) of the lane's row: read, or - when every query row of the launch belongs to this kernel -
+    // formed here from the dO row the lane already holds and written out for the key-side pass (one launch and one
+    // pass over dO and O less)
+    float dlt;
+    if (out_for_delta) {                                 // (kernel argument: the same for every wave)
+        // the order of dsa_bwd_delta_kernel, so that both give the same bits: chain j of this lane covers the 8-element
+        // chunks 2*ks+h with ks = j, j+8, ... (that kernel's lane 2*j+h), then its butterfly over 16 lanes - the three
+        // steps between lanes of one parity here, the last one across the lane pair
+        float p[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            p[j] = 0.f;
+#pragma unroll
+            for (int ks = j; ks < KS; ks += 8) {
+                const int64_t off = ((int64_t)t * Hq + hq) * D + 16 * ks + 8 * h;
+                const bf16x8 o8 = row_ok ? load_bf16x8(out_for_delta + off) : zero_bf16x8();
+                p[j] = dot8_chain(doB[ks], o8, p[j]);
+            }
+        }
+        const float part = ((p[0] + p[4]) + (p[2] + p[6])) + ((p[1] + p[5]) + (p[3] + p[7]));
+        dlt = half_sum_f(part);
+        if (row_ok && h == 0) delta_out[(int64_t)hq * T + t] = dlt;
+    } else {
+        dlt = delta[(int64_t)hq * T + t];
+    }
+    const float neg_dlt = -dlt;
     const int ntiles = (causal ? min(qc0 + QBW - 1, L - 1) : L - 1) / 32 + 1;
     const int klim = causal ? qcol : L - 1;             // last key column this row may attend (dense mode)
     const uint32_t *wrow = bitmap + (int64_t)t * ldw;
@@ -2106,10 +2132,11 @@ static hipError_t launch_fwd_i(dim3 grid, hipStream_t stream, const void *q, con
 template <int D, bool HAS_IDX, int GS>
 static hipError_t launch_dq_i(dim3 grid, hipStream_t stream, const void *dout, const void *q, const void *k, const void *v,
                         const float *lse, const float *delta, const uint32_t *bitmap, int ldw, const int32_t *cu, int N,
-                        int T, int Hq, int Hkv, float scale, int pos_split, int causal, void *dq) {
+                        int T, int Hq, int Hkv, float scale, int pos_split, int causal, void *dq, const void *out_for_delta,
+                        float *delta_out) {
     hipLaunchKernelGGL((dsa_tile_dq_kernel<D, HAS_IDX, GS, tile_waves<D>()>), grid, dim3(64 * tile_waves<D>()), 0, stream, (const bf16_t *)dout,
                        (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv,
-                       scale, pos_split, causal, (bf16_t *)dq);
+                       scale, pos_split, causal, (bf16_t *)dq, (const bf16_t *)out_for_delta, delta_out);
     return hipSuccess;
 }
 template <int D, bool HAS_IDX, int GS>
@@ -2277,10 +2304,12 @@ extern "C" hipError_t dsa_launch_indexer_bwd(const void *q_idx, const void *k_id
 extern "C" hipError_t dsa_launch_tile_dq(const void *dout, const void *q, const void *k, const void *v,
                                          const float *lse, const float *delta, const uint32_t *bitmap, int ldw,
                                          const int32_t *cu, int N, int T, int Hq, int Hkv, int D, float scale,
-                                         int pos_split, int causal, void *dq, hipStream_t stream) {
+                                         int pos_split, int causal, void *dq, const void *out_for_delta, float *delta_out,
+                                         hipStream_t stream) {
+    // out_for_delta != null: the kernel forms delta = rowsum(dO * O) of its rows itself and writes it to delta_out
     const int gs = group_shift(Hq, Hkv);
     const dim3 grid((unsigned)(((int64_t)T / ((32 * tile_waves_of(D)) >> gs) + N + 1) * Hkv));
-    TILE_SWITCH_96(launch_dq_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, pos_split, causal, dq)
+    TILE_SWITCH_96(launch_dq_i, grid, stream, dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, scale, pos_split, causal, dq, out_for_delta, delta_out)
     return hipGetLastError();
 }
 // bytes of fp32 partial sums a launch of T tokens may use for key-tile walks in pieces (0: launches of this size are

@@ -36,6 +36,18 @@ __device__ __forceinline__ bf16x8 load_bf16x8(const bf16_t *p) {   // 16-byte al
 }
 
 // two fp32 -> packed bf16 pair, round-to-nearest-even (one v_cvt_pk_bf16_f32 on gfx950)
+// acc + sum_e a[e] * b[e] over 8 bf16 pairs, one fused multiply-add per element in element order.  Every kernel that forms
+// delta = rowsum(dO * O) goes through this one chain, so that they agree to the bit.
+__device__ __forceinline__ float dot8_chain(bf16x8 a, bf16x8 b, float acc) {
+    const u32x4 x = __builtin_bit_cast(u32x4, a), y = __builtin_bit_cast(u32x4, b);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        acc = __builtin_fmaf(__uint_as_float(x[e] << 16), __uint_as_float(y[e] << 16), acc);
+        acc = __builtin_fmaf(__uint_as_float(x[e] & 0xffff0000u), __uint_as_float(y[e] & 0xffff0000u), acc);
+    }
+    return acc;
+}
+
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pack2bf(float lo, float hi) {
