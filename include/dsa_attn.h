@@ -282,6 +282,12 @@ int dsa_sigmoid_gate_bwd(const void *gy, const void *x, const void *gate, int64_
  */
 int dsa_split_bf16_stack(const float *x, int64_t rows, int D, int order, void *y, void *stream);
 int dsa_split_bf16_combine(const void *y, int64_t rows, int D, int part, float *out, void *stream);
+/* The three operands of one attention call in one launch: q (rows_q, D) with order 0, k (rows_kv, D) with order 1 and
+ * v (rows_kv, D) with order 0; and the way back for the three gradients: dq part 2, dk part 1, dv part 2. */
+int dsa_split_bf16_stack_qkv(const float *q, const float *k, const float *v, int64_t rows_q, int64_t rows_kv, int D,
+                             void *yq, void *yk, void *yv, void *stream);
+int dsa_split_bf16_combine_qkv(const void *yq, const void *yk, const void *yv, int64_t rows_q, int64_t rows_kv, int D,
+                               float *dq, float *dk, float *dv, void *stream);
 
 #ifdef __cplusplus
 }

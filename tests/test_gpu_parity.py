@@ -136,6 +136,29 @@ def test_c1_toy_fp32_full():
     _run_case(W.C1)
 
 
+def test_fp32_carrier_of_three_operands_equals_the_single_operand_launches():
+    """q, k, v split into stacked bf16 parts by one launch, and the three gradients combined by one: bit-identical to
+    the launches that take one operand each, and hi + lo gives the fp32 value back to 2^-16 relative."""
+    _log("fp32 carrier, three operands")
+    g = torch.Generator(device=DEV).manual_seed(5)
+    T, Hq, Hkv, D = 333, 6, 2, 20
+    q = torch.randn(T, Hq, D, device=DEV, generator=g)
+    k = torch.randn(T, Hkv, D, device=DEV, generator=g)
+    v = torch.randn(T, Hkv, D, device=DEV, generator=g)
+    yq, yk, yv = ops._split_stack_qkv(q, k, v)
+    assert torch.equal(yq, ops._split_stack(q, 0)) and torch.equal(yk, ops._split_stack(k, 1))
+    assert torch.equal(yv, ops._split_stack(v, 0))
+    back = yq[..., :D].float() + yq[..., D:2 * D].float()
+    assert (back - q).abs().max() <= 2.0 ** -16 * q.abs().max()
+    gq, gk, gv = (torch.randn(y.shape, device=DEV, generator=g).bfloat16() for y in (yq, yk, yv))
+    dq, dk, dv = ops._split_combine_qkv(gq, gk, gv)
+    assert torch.equal(dq, ops._split_combine(gq, 2)) and torch.equal(dk, ops._split_combine(gk, 1))
+    assert torch.equal(dv, ops._split_combine(gv, 2))
+    assert torch.equal(dq, gq[..., :D].float() + gq[..., 2 * D:3 * D].float())
+    e = ops._split_stack_qkv(q[:0], k[:0], v[:0])
+    assert [x.shape[0] for x in e] == [0, 0, 0]
+
+
 @pytest.mark.parametrize("name,segs,K", [
     ("C2", (700, 333, 40, 0, 515, 204), 256),
     ("C3", (1100, 64, 600, 284), 512),

@@ -69,6 +69,10 @@ hipError_t dsa_launch_sigmoid_gate_fwd(const void *x, const void *gate, int64_t 
                                        int64_t rows, void *y, hipStream_t stream);
 hipError_t dsa_launch_split_stack(const float *x, int64_t rows, int D, int order, void *y, hipStream_t stream);
 hipError_t dsa_launch_split_combine(const void *y, int64_t rows, int D, int part, float *out, hipStream_t stream);
+hipError_t dsa_launch_split_stack_qkv(const float *q, const float *k, const float *v, int64_t rows_q, int64_t rows_kv, int D, void *yq,
+                                      void *yk, void *yv, hipStream_t stream);
+hipError_t dsa_launch_split_combine_qkv(const void *yq, const void *yk, const void *yv, int64_t rows_q, int64_t rows_kv, int D,
+                                        float *dq, float *dk, float *dv, hipStream_t stream);
 hipError_t dsa_launch_sigmoid_gate_bwd(const void *gy, const void *x, const void *gate, int64_t gate_tok, int64_t gate_head,
                                        int D, int H, int64_t rows, void *dx, void *dgate, int64_t dgate_tok,
                                        int64_t dgate_head, hipStream_t stream);
@@ -597,5 +601,19 @@ extern "C" int dsa_split_bf16_combine(const void *y, int64_t rows, int D, int pa
     if (rows < 0 || D < 4 || D % 4 || part < 1 || part > 3) return fail(DSA_ERR_ARG, "rows=%lld D=%d part=%d", (long long)rows, D, part);
     if (rows > 0 && (!y || !out)) return fail(DSA_ERR_ARG, "null tensor pointer");
     hipError_t e = dsa_launch_split_combine(y, rows, D, part, out, (hipStream_t)stream);
+    return e == hipSuccess ? DSA_OK : hip_fail(e, "split/combine launch");
+}
+extern "C" int dsa_split_bf16_stack_qkv(const float *q, const float *k, const float *v, int64_t rows_q, int64_t rows_kv, int D,
+                                        void *yq, void *yk, void *yv, void *stream) {
+    if (rows_q < 0 || rows_kv < 0 || D < 4 || D % 4) return fail(DSA_ERR_ARG, "rows_q=%lld rows_kv=%lld D=%d", (long long)rows_q, (long long)rows_kv, D);
+    if ((rows_q > 0 && (!q || !yq)) || (rows_kv > 0 && (!k || !v || !yk || !yv))) return fail(DSA_ERR_ARG, "null tensor pointer");
+    hipError_t e = dsa_launch_split_stack_qkv(q, k, v, rows_q, rows_kv, D, yq, yk, yv, (hipStream_t)stream);
+    return e == hipSuccess ? DSA_OK : hip_fail(e, "split/stack launch");
+}
+extern "C" int dsa_split_bf16_combine_qkv(const void *yq, const void *yk, const void *yv, int64_t rows_q, int64_t rows_kv, int D,
+                                          float *dq, float *dk, float *dv, void *stream) {
+    if (rows_q < 0 || rows_kv < 0 || D < 4 || D % 4) return fail(DSA_ERR_ARG, "rows_q=%lld rows_kv=%lld D=%d", (long long)rows_q, (long long)rows_kv, D);
+    if ((rows_q > 0 && (!yq || !dq)) || (rows_kv > 0 && (!yk || !yv || !dk || !dv))) return fail(DSA_ERR_ARG, "null tensor pointer");
+    hipError_t e = dsa_launch_split_combine_qkv(yq, yk, yv, rows_q, rows_kv, D, dq, dk, dv, (hipStream_t)stream);
     return e == hipSuccess ? DSA_OK : hip_fail(e, "split/combine launch");
 }

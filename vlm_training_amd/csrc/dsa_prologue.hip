@@ -321,37 +321,62 @@ extern "C" hipError_t dsa_launch_sigmoid_gate_bwd(const void *gy, const void *x,
 //   order 0: [hi, lo, hi, 0]  (q, v)        order 1: [hi, hi, lo, 0]  (k, dO)
 // and the way back, out[r, :] = y[r, 0:D] + y[r, part*D:(part+1)*D] in fp32.  One thread per 4 elements.
 // ---------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void split_stack4(const float *__restrict__ x, int64_t i, int D, int order, bf16_t *__restrict__ y) {
+    const int64_t r = i / (D / 4);
+    const int c = (int)(i % (D / 4)) * 4;
+    const f32x4 v = *reinterpret_cast<const f32x4 *>(x + r * D + c);
+    const uint32_t h0 = pack2bf(v[0], v[1]), h1 = pack2bf(v[2], v[3]);
+    const uint32_t l0 = pack2bf(v[0] - __uint_as_float(h0 << 16), v[1] - __uint_as_float(h0 & 0xffff0000u));
+    const uint32_t l1 = pack2bf(v[2] - __uint_as_float(h1 << 16), v[3] - __uint_as_float(h1 & 0xffff0000u));
+    bf16_t *o = y + r * 4 * D + c;
+    const u32x2 hi = {h0, h1}, lo = {l0, l1}, z = {0u, 0u};
+    *reinterpret_cast<u32x2 *>(o) = hi;
+    *reinterpret_cast<u32x2 *>(o + D) = order ? hi : lo;
+    *reinterpret_cast<u32x2 *>(o + 2 * D) = order ? lo : hi;
+    *reinterpret_cast<u32x2 *>(o + 3 * D) = z;
+}
+__device__ __forceinline__ void split_combine4(const bf16_t *__restrict__ y, int64_t i, int D, int part, float *__restrict__ out) {
+    const int64_t r = i / (D / 4);
+    const int c = (int)(i % (D / 4)) * 4;
+    const u32x2 a = *reinterpret_cast<const u32x2 *>(y + r * 4 * D + c);
+    const u32x2 b = *reinterpret_cast<const u32x2 *>(y + r * 4 * D + part * D + c);
+    const f32x4 o = {__uint_as_float(a[0] << 16) + __uint_as_float(b[0] << 16),
+                     __uint_as_float(a[0] & 0xffff0000u) + __uint_as_float(b[0] & 0xffff0000u),
+                     __uint_as_float(a[1] << 16) + __uint_as_float(b[1] << 16),
+                     __uint_as_float(a[1] & 0xffff0000u) + __uint_as_float(b[1] & 0xffff0000u)};
+    *reinterpret_cast<f32x4 *>(out + r * D + c) = o;
+}
 __global__ __launch_bounds__(256) void dsa_split_stack_kernel(const float *__restrict__ x, int64_t rows, int D, int order,
                                                                bf16_t *__restrict__ y) {
     const int64_t n4 = rows * (D / 4);
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
-        const int64_t r = i / (D / 4);
-        const int c = (int)(i % (D / 4)) * 4;
-        const f32x4 v = *reinterpret_cast<const f32x4 *>(x + r * D + c);
-        const uint32_t h0 = pack2bf(v[0], v[1]), h1 = pack2bf(v[2], v[3]);
-        const uint32_t l0 = pack2bf(v[0] - __uint_as_float(h0 << 16), v[1] - __uint_as_float(h0 & 0xffff0000u));
-        const uint32_t l1 = pack2bf(v[2] - __uint_as_float(h1 << 16), v[3] - __uint_as_float(h1 & 0xffff0000u));
-        bf16_t *o = y + r * 4 * D + c;
-        const u32x2 hi = {h0, h1}, lo = {l0, l1}, z = {0u, 0u};
-        *reinterpret_cast<u32x2 *>(o) = hi;
-        *reinterpret_cast<u32x2 *>(o + D) = order ? hi : lo;
-        *reinterpret_cast<u32x2 *>(o + 2 * D) = order ? lo : hi;
-        *reinterpret_cast<u32x2 *>(o + 3 * D) = z;
-    }
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) split_stack4(x, i, D, order, y);
 }
 __global__ __launch_bounds__(256) void dsa_split_combine_kernel(const bf16_t *__restrict__ y, int64_t rows, int D, int part,
                                                                  float *__restrict__ out) {
     const int64_t n4 = rows * (D / 4);
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
-        const int64_t r = i / (D / 4);
-        const int c = (int)(i % (D / 4)) * 4;
-        const u32x2 a = *reinterpret_cast<const u32x2 *>(y + r * 4 * D + c);
-        const u32x2 b = *reinterpret_cast<const u32x2 *>(y + r * 4 * D + part * D + c);
-        const f32x4 o = {__uint_as_float(a[0] << 16) + __uint_as_float(b[0] << 16),
-                         __uint_as_float(a[0] & 0xffff0000u) + __uint_as_float(b[0] & 0xffff0000u),
-                         __uint_as_float(a[1] << 16) + __uint_as_float(b[1] << 16),
-                         __uint_as_float(a[1] & 0xffff0000u) + __uint_as_float(b[1] & 0xffff0000u)};
-        *reinterpret_cast<f32x4 *>(out + r * D + c) = o;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) split_combine4(y, i, D, part, out);
+}
+// the three operands of one attention call in one launch: q-shaped (rows_q) first, then the two kv-shaped ones
+__global__ __launch_bounds__(256) void dsa_split_stack_qkv_kernel(const float *__restrict__ q, const float *__restrict__ k,
+                                                                   const float *__restrict__ v, int64_t rows_q, int64_t rows_kv,
+                                                                   int D, bf16_t *__restrict__ yq, bf16_t *__restrict__ yk,
+                                                                   bf16_t *__restrict__ yv) {
+    const int64_t nq = rows_q * (D / 4), nkv = rows_kv * (D / 4);
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nq + 2 * nkv; i += (int64_t)gridDim.x * 256) {
+        if (i < nq) split_stack4(q, i, D, 0, yq);
+        else if (i < nq + nkv) split_stack4(k, i - nq, D, 1, yk);
+        else split_stack4(v, i - nq - nkv, D, 0, yv);
+    }
+}
+__global__ __launch_bounds__(256) void dsa_split_combine_qkv_kernel(const bf16_t *__restrict__ yq, const bf16_t *__restrict__ yk,
+                                                                     const bf16_t *__restrict__ yv, int64_t rows_q,
+                                                                     int64_t rows_kv, int D, float *__restrict__ dq,
+                                                                     float *__restrict__ dk, float *__restrict__ dv) {
+    const int64_t nq = rows_q * (D / 4), nkv = rows_kv * (D / 4);
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nq + 2 * nkv; i += (int64_t)gridDim.x * 256) {
+        if (i < nq) split_combine4(yq, i, D, 2, dq);
+        else if (i < nq + nkv) split_combine4(yk, i - nq, D, 1, dk);
+        else split_combine4(yv, i - nq - nkv, D, 2, dv);
     }
 }
 extern "C" hipError_t dsa_launch_split_stack(const float *x, int64_t rows, int D, int order, void *y, hipStream_t stream) {
@@ -366,5 +391,23 @@ extern "C" hipError_t dsa_launch_split_combine(const void *y, int64_t rows, int 
     if (n4 == 0) return hipSuccess;
     const int nb = (int)((n4 + 255) / 256 > 8192 ? 8192 : (n4 + 255) / 256);
     hipLaunchKernelGGL(dsa_split_combine_kernel, dim3(nb), dim3(256), 0, stream, (const bf16_t *)y, rows, D, part, out);
+    return hipGetLastError();
+}
+extern "C" hipError_t dsa_launch_split_stack_qkv(const float *q, const float *k, const float *v, int64_t rows_q, int64_t rows_kv,
+                                                 int D, void *yq, void *yk, void *yv, hipStream_t stream) {
+    const int64_t n4 = (rows_q + 2 * rows_kv) * (D / 4);
+    if (n4 == 0) return hipSuccess;
+    const int nb = (int)((n4 + 255) / 256 > 8192 ? 8192 : (n4 + 255) / 256);
+    hipLaunchKernelGGL(dsa_split_stack_qkv_kernel, dim3(nb), dim3(256), 0, stream, q, k, v, rows_q, rows_kv, D, (bf16_t *)yq,
+                       (bf16_t *)yk, (bf16_t *)yv);
+    return hipGetLastError();
+}
+extern "C" hipError_t dsa_launch_split_combine_qkv(const void *yq, const void *yk, const void *yv, int64_t rows_q, int64_t rows_kv,
+                                                   int D, float *dq, float *dk, float *dv, hipStream_t stream) {
+    const int64_t n4 = (rows_q + 2 * rows_kv) * (D / 4);
+    if (n4 == 0) return hipSuccess;
+    const int nb = (int)((n4 + 255) / 256 > 8192 ? 8192 : (n4 + 255) / 256);
+    hipLaunchKernelGGL(dsa_split_combine_qkv_kernel, dim3(nb), dim3(256), 0, stream, (const bf16_t *)yq, (const bf16_t *)yk,
+                       (const bf16_t *)yv, rows_q, rows_kv, D, dq, dk, dv);
     return hipGetLastError();
 }

@@ -353,6 +353,30 @@ def _split_combine(y: torch.Tensor, part: int) -> torch.Tensor:
     return out
 
 
+def _split_stack_qkv(q, k, v):
+    """The three operands of one call in one launch: q and v with order 0, k with order 1."""
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    (T, Hq, D), Hkv = q.shape, k.shape[1]
+    yq = torch.empty((T, Hq, 4 * D), dtype=torch.bfloat16, device=q.device)
+    ykv = torch.empty((2, T, Hkv, 4 * D), dtype=torch.bfloat16, device=q.device)
+    rc = _lib.load().dsa_split_bf16_stack_qkv(_ptr(q), _ptr(k), _ptr(v), T * Hq, T * Hkv, D, _ptr(yq), _ptr(ykv[0]),
+                                              _ptr(ykv[1]), _stream(q.device))
+    _lib.check(rc, "dsa_split_bf16_stack_qkv")
+    return yq, ykv[0], ykv[1]
+
+
+def _split_combine_qkv(dq, dk, dv):
+    """The three gradients back to fp32 in one launch: dq and dv with part 2, dk with part 1."""
+    (T, Hq, D4), Hkv = dq.shape, dk.shape[1]
+    D = D4 // 4
+    oq = torch.empty((T, Hq, D), dtype=torch.float32, device=dq.device)
+    okv = torch.empty((2, T, Hkv, D), dtype=torch.float32, device=dq.device)
+    rc = _lib.load().dsa_split_bf16_combine_qkv(_ptr(dq), _ptr(dk), _ptr(dv), T * Hq, T * Hkv, D, _ptr(oq), _ptr(okv[0]),
+                                                _ptr(okv[1]), _stream(dq.device))
+    _lib.check(rc, "dsa_split_bf16_combine_qkv")
+    return oq, okv[0], okv[1]
+
+
 class _DsaVarlenAttn(torch.autograd.Function):
     """bf16 inputs go to the kernels as they are.  fp32 inputs with 4*D <= 256 are carried as split-bf16
     operands (x = hi + lo) stacked along head_dim, which keeps near-fp32 logits on the bf16 MFMA path:
@@ -368,7 +392,7 @@ class _DsaVarlenAttn(torch.autograd.Function):
         D = q.shape[-1]
         split = in_dtype == torch.float32 and 4 * D <= 256
         if split:
-            qb, kb, vb = _split_stack(q, 0), _split_stack(k, 1), _split_stack(v, 0)
+            qb, kb, vb = _split_stack_qkv(q, k, v)
         else:
             qb, kb, vb = _as_bf16(q), _as_bf16(k), _as_bf16(v)
         fwd_ws = None
@@ -417,7 +441,7 @@ class _DsaVarlenAttn(torch.autograd.Function):
             dq, dk, dv = attn_bwd(db, qb, kb, vb, out, lse, idx, n, cu, ctx.max_seqlen, ctx.softmax_scale,
                                   causal=ctx.causal)
         if ctx.split:
-            dq, dk, dv = _split_combine(dq, 2), _split_combine(dk, 1), _split_combine(dv, 2)
+            dq, dk, dv = _split_combine_qkv(dq, dk, dv)
         elif ctx.in_dtype != torch.bfloat16:
             dq, dk, dv = dq.to(ctx.in_dtype), dk.to(ctx.in_dtype), dv.to(ctx.in_dtype)
         return dq, dk, dv, None, None, None, None, None, None, None
