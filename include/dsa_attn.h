@@ -167,6 +167,20 @@ size_t dsa_attn_mass_workspace_bytes(int T, int N, int Hq, int Hkv, int D, int K
 int dsa_set_tile_crossover(int crossover);
 int dsa_get_tile_crossover(void);
 
+/*
+ * Tuning knob (process-wide, no reference counterpart): the backward's query-side pass (dQ) and key-side pass (dK/dV)
+ * read the same inputs and write different outputs.  1 (default): when the key-side launch has at most 1536
+ * workgroups - a short batch, or one GPU's share of head-sharded attention, which ends on its longest walks with most
+ * CUs idle - and T * max_seqlen * Hq * D is at least 6e10 (below that the fork and join cost what the overlap gains)
+ * the query side runs on a second stream of the library's own (default priority, one per device, created
+ * on the first such call outside a capture) between a fork and a join event on the caller's stream, so that to the
+ * caller the whole call is still ordered on the stream it passed; under stream capture the second stream joins the
+ * capture through those events.  0: never (one stream).  2: for every launch size.  Results are the same bits in all
+ * modes.
+ */
+int dsa_set_bwd_overlap(int mode);
+int dsa_get_bwd_overlap(void);
+
 /* Bytes of workspace dsa_attn_bwd needs: softmax row terms, the inverted selection bitmap, the launch order of the
  * dK/dV key tiles (about 128 KiB + T/8 bytes) and, up to 131072 tokens, fp32 partial sums for key-tile walks that a
  * small launch cuts into pieces (16 KiB per token, at most 128 MiB). */

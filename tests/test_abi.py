@@ -58,6 +58,8 @@ def test_workspace_sizes_without_a_gpu():
     assert lib.dsa_attn_mass_workspace_bytes(1000, 3, 32, 16, 128, 64, 640) == up(1000 * 20 * 4) + up(2 * 1000 * 64 * 4)
     assert old == 24 and lib.dsa_set_tile_crossover(-1) == -1 and lib.dsa_set_tile_crossover(3) == 0
     assert lib.dsa_get_tile_crossover() == 3 and lib.dsa_set_tile_crossover(old) == 0
+    assert lib.dsa_get_bwd_overlap() == 1 and lib.dsa_set_bwd_overlap(3) == -1 and lib.dsa_set_bwd_overlap(0) == 0
+    assert lib.dsa_get_bwd_overlap() == 0 and lib.dsa_set_bwd_overlap(1) == 0
 
 
 def test_argument_errors_are_reported_not_thrown():

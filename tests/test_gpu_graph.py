@@ -1,6 +1,8 @@
 """The operator under HIP graph capture: a captured forward+backward, replayed with eager work between the replays,
-gives on every replay what the eager call gives.  (The library launches kernels on the caller's stream and nothing
-else: no allocation, no memset node, no synchronisation of its own.)"""
+gives on every replay what the eager call gives.  (The library launches kernels and nothing else: no allocation, no
+memset node, no synchronisation of its own.  With the backward's passes side by side - forced here, the launch being
+too small for the default to choose it - the query-side pass is forked onto the library's second stream and joined
+again, and the captured graph holds that fork and join too.)"""
 import pytest
 import torch
 
@@ -14,9 +16,16 @@ def _log(msg):
     print(f"[graph] {msg}", flush=True)
 
 
+@pytest.fixture(params=[1, 2], ids=["one-stream", "two-streams"])
+def overlap(request):
+    old = ops.set_bwd_overlap(request.param)
+    yield request.param
+    ops.set_bwd_overlap(old)
+
+
 @pytest.mark.parametrize("sparse", [True, False])
-def test_captured_step_replays_to_the_eager_result(sparse):
-    _log(f"capture sparse={sparse}")
+def test_captured_step_replays_to_the_eager_result(sparse, overlap):
+    _log(f"capture sparse={sparse} overlap={overlap}")
     w = W.scaled(W.C3, (700, 130, 260), top_k=128, name="graph")
     t = W.make_inputs(w, device=DEV)
     cu, msl = t["cu_seqlens"], w.max_seqlen

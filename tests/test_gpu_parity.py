@@ -491,6 +491,37 @@ def test_backward_is_deterministic_and_unselected_keys_get_zero():
     assert (grads[0][1][~used] == 0).all() and (grads[0][2][~used] == 0).all()
 
 
+@pytest.mark.parametrize("sparse", [True, False])
+def test_backward_passes_side_by_side_give_the_same_bits(sparse):
+    """dQ on the library's second stream beside dK/dV (modes 1 and 2) against one pass after the other (mode 0), with
+    eager work queued right behind the call on the caller's stream, which must wait for both passes."""
+    _log(f"bwd overlap sparse={sparse}")
+    w = W.scaled(W.C2, (900, 77, 410, 1300), top_k=128, name="overlap")
+    t = W.make_inputs(w, device=DEV)
+    cu, msl, scale = t["cu_seqlens"], w.max_seqlen, w.D ** -0.5
+    idx, n = ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k) if sparse else (None, None)
+    out, lse = ops.attn_fwd(t["q"], t["k"], t["v"], idx, n, cu, msl, scale)
+    old = ops.set_bwd_overlap(0)
+    try:
+        res = {}
+        for mode in (0, 1, 2, 0, 2):
+            ops.set_bwd_overlap(mode)
+            for stream in (torch.cuda.current_stream(), torch.cuda.Stream()):
+                stream.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(stream):
+                    dq, dk, dv = ops.attn_bwd(t["dout"], t["q"], t["k"], t["v"], out, lse, idx, n, cu, msl, scale)
+                    sums = dq.float().sum() + dk.float().sum() + dv.float().sum()     # queued behind the call
+                torch.cuda.current_stream().wait_stream(stream)
+                got = (dq, dk, dv, sums)
+                if not res:
+                    res = got
+                for a, b in zip(res, got):
+                    assert torch.equal(a, b), f"mode {mode}"
+    finally:
+        ops.set_bwd_overlap(old)
+    assert old == 1
+
+
 def test_reference_named_entry_points():
     _log("entry points")
     import vlm_training_amd as M

@@ -45,6 +45,8 @@ _SIGNATURES = {
     "dsa_attn_mass_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
     "dsa_set_tile_crossover": (c_int, [c_int]),
     "dsa_get_tile_crossover": (c_int, []),
+    "dsa_set_bwd_overlap": (c_int, [c_int]),
+    "dsa_get_bwd_overlap": (c_int, []),
     "dsa_attn_bwd_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "dsa_attn_bwd_bitmap_offset": (c_size_t, [c_int, c_int]),
     "dsa_attn_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,

@@ -390,6 +390,53 @@ extern "C" size_t dsa_attn_bwd_bitmap_offset(int T, int Hq) {
     return align_up((size_t)T * Hq * 4, 256);
 }
 
+// ---- the query-side and the key-side pass of one backward side by side ----
+// Both read the same inputs and write different outputs, and a launch of few workgroups ends on its longest walks with
+// most CUs idle: the query side then runs on a second stream of the library's own (default priority, one per device,
+// made on first use outside any capture) between a fork and a join event, so that to the caller everything still
+// happens on the stream it passed.  A stream under capture takes the second one into the capture through the events.
+// mode 1 runs the passes side by side for key-side launches of at most this many workgroups (larger ones fill the GPU
+// alone) whose work bound T * max_seqlen * Hq * D reaches the second figure (about 0.4 ms of backward: below it the
+// fork, the join and the delta pass that the query side otherwise absorbs cost what the overlap gains)
+#define DSA_BWD_OVERLAP_MAX_WG (6 * 256)
+#define DSA_BWD_OVERLAP_MIN_WORK 6.0e10
+struct OverlapCtx {
+    hipStream_t aux = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
+    bool failed = false;
+};
+static OverlapCtx g_overlap[DSA_MAX_DEVICES];
+static std::mutex g_overlap_mu;                          // held from fork to join: the events are shared by every caller
+static std::atomic<int> g_bwd_overlap{1};               // 0 never, 1 launches of few workgroups, 2 always
+extern "C" int dsa_set_bwd_overlap(int mode) {
+    if (mode < 0 || mode > 2) return fail(DSA_ERR_ARG, "bwd overlap mode=%d outside [0,2]", mode);
+    g_bwd_overlap.store(mode, std::memory_order_relaxed);
+    return DSA_OK;
+}
+extern "C" int dsa_get_bwd_overlap(void) { return g_bwd_overlap.load(std::memory_order_relaxed); }
+// null when the second stream is not to be had (then the passes run one after the other); call with g_overlap_mu held
+static OverlapCtx *overlap_ctx(hipStream_t main_stream) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= DSA_MAX_DEVICES) return nullptr;
+    OverlapCtx &c = g_overlap[dev];
+    if (c.aux) return &c;
+    if (c.failed) return nullptr;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (main_stream && (hipStreamIsCapturing(main_stream, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone)) {
+        (void)hipGetLastError();
+        return nullptr;                                  // nothing is created while a capture runs
+    }
+    if (hipStreamCreateWithFlags(&c.aux, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&c.fork, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&c.join, hipEventDisableTiming) != hipSuccess) {
+        (void)hipGetLastError();
+        c.aux = nullptr;
+        c.failed = true;
+        return nullptr;
+    }
+    return &c;
+}
+
 // the backward proper: every buffer named, so that the two entry points below differ only in where the buffers live
 static int attn_bwd_run(const void *dout, const void *q, const void *k, const void *v, const void *out, const float *lse,
                         const int32_t *idx, const int32_t *n, const int32_t *cu, int T, int N, int Hq, int Hkv, int D, int K,
@@ -399,9 +446,23 @@ static int attn_bwd_run(const void *dout, const void *q, const void *k, const vo
     if (idx && (size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);
     const int split = pos_split_for(idx, K);
     hipError_t e = hipSuccess;
+    // the two passes side by side on two streams: launches of few workgroups only (larger ones fill the GPU alone)
+    std::unique_lock<std::mutex> ov_lock;
+    OverlapCtx *ov = nullptr;
+    const int ov_mode = g_bwd_overlap.load(std::memory_order_relaxed);
+    if ((parts & DSA_BWD_DQ) && (parts & DSA_BWD_DKV) && ov_mode > 0) {
+        const int64_t dkv_wg = ((int64_t)T / 128 + N) * Hkv * (D > 128 ? 2 : 1);
+        const double work = (double)T * max_seqlen * Hq * D;
+        if (ov_mode == 2 || (dkv_wg <= DSA_BWD_OVERLAP_MAX_WG && work >= DSA_BWD_OVERLAP_MIN_WORK)) {
+            ov_lock = std::unique_lock<std::mutex>(g_overlap_mu);
+            ov = overlap_ctx(st);
+            if (!ov) ov_lock.unlock();
+        }
+    }
     // delta = rowsum(dO * O): a pass of its own, unless the tile dQ kernel of the same call owns every query row
-    // (no row beyond the tile/gather split) - then that kernel forms it from the dO rows it loads anyway
-    const bool fuse_delta = (parts & DSA_BWD_DELTA) && (parts & DSA_BWD_DQ) && split > 0 && max_seqlen <= split;
+    // (no row beyond the tile/gather split) - then that kernel forms it from the dO rows it loads anyway - and the
+    // key side, which reads every delta, runs after it
+    const bool fuse_delta = (parts & DSA_BWD_DELTA) && (parts & DSA_BWD_DQ) && split > 0 && max_seqlen <= split && !ov;
     if ((parts & DSA_BWD_DELTA) && !fuse_delta) {
         e = dsa_launch_delta(dout, out, T, Hq, D, delta, st);
         if (e != hipSuccess) return hip_fail(e, "delta launch");
@@ -410,23 +471,36 @@ static int attn_bwd_run(const void *dout, const void *q, const void *k, const vo
         e = dsa_launch_bitmap(idx, n, cu, N, T, K, ldw, bitmap, st);
         if (e != hipSuccess) return hip_fail(e, "bitmap launch");
     }
+    hipStream_t sq = st;
+    if (ov) {
+        e = hipEventRecord(ov->fork, st);
+        if (e == hipSuccess) e = hipStreamWaitEvent(ov->aux, ov->fork, 0);
+        if (e != hipSuccess) return hip_fail(e, "fork to the second stream");
+        sq = ov->aux;
+    }
+    int rc = DSA_OK;
     if (parts & DSA_BWD_DQ) {
         if (split > 0) {
             e = dsa_launch_tile_dq(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, split, causal, dq,
-                                   fuse_delta ? out : nullptr, delta, st);
-            if (e != hipSuccess) return hip_fail(e, "tile dq launch");
+                                   fuse_delta ? out : nullptr, delta, sq);
+            if (e != hipSuccess) rc = hip_fail(e, "tile dq launch");
         }
-        if (max_seqlen > split) {
-            e = dsa_launch_gather_dq(dout, q, k, v, lse, delta, idx, n, cu, N, T, Hq, Hkv, D, K, softmax_scale, split, dq, st);
-            if (e != hipSuccess) return hip_fail(e, "gather dq launch");
+        if (rc == DSA_OK && max_seqlen > split) {
+            e = dsa_launch_gather_dq(dout, q, k, v, lse, delta, idx, n, cu, N, T, Hq, Hkv, D, K, softmax_scale, split, dq, sq);
+            if (e != hipSuccess) rc = hip_fail(e, "gather dq launch");
         }
     }
-    if (parts & DSA_BWD_DKV) {
+    if (rc == DSA_OK && (parts & DSA_BWD_DKV)) {
         e = dsa_launch_tile_dkv(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, causal, order, partial,
                                 partial_bytes, dk, dv, st);
-        if (e != hipSuccess) return hip_fail(e, "tile dkv launch");
+        if (e != hipSuccess) rc = hip_fail(e, "tile dkv launch");
     }
-    return DSA_OK;
+    if (ov) {                                            // joined also after a failed launch: the caller's stream stays whole
+        e = hipEventRecord(ov->join, ov->aux);
+        if (e == hipSuccess) e = hipStreamWaitEvent(st, ov->join, 0);
+        if (e != hipSuccess && rc == DSA_OK) rc = hip_fail(e, "join of the second stream");
+    }
+    return rc;
 }
 
 static int check_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out, const float *lse,

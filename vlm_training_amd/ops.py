@@ -243,6 +243,16 @@ def set_tile_crossover(crossover: int) -> int:
     return old
 
 
+def set_bwd_overlap(mode: int) -> int:
+    """0: the backward's passes run one after the other on the caller's stream; 1 (default): launches of few
+    workgroups run dQ beside dK/dV on a second stream of the library's own; 2: every launch does.  Same bits in every
+    mode.  Returns the previous mode."""
+    lib = _lib.load()
+    old = lib.dsa_get_bwd_overlap()
+    _lib.check(lib.dsa_set_bwd_overlap(int(mode)), "dsa_set_bwd_overlap")
+    return old
+
+
 def attn_fwd(q, k, v, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float, causal: bool = True, ws=None):
     """Stage D3.  ``ws`` (optional, uint8) is used as the workspace instead of a fresh allocation; the
     autograd wrapper passes the tail of the backward workspace so that the selection bitmap is built once."""
