@@ -479,7 +479,13 @@ static int attn_bwd_run(const void *dout, const void *q, const void *k, const vo
         sq = ov->aux;
     }
     int rc = DSA_OK;
-    if (parts & DSA_BWD_DQ) {
+    // (side by side, the key side is issued first: it is the longer pass and starts with its longest walks)
+    if (ov) {
+        e = dsa_launch_tile_dkv(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, causal, order, partial,
+                                partial_bytes, dk, dv, st);
+        if (e != hipSuccess) rc = hip_fail(e, "tile dkv launch");
+    }
+    if (rc == DSA_OK && (parts & DSA_BWD_DQ)) {
         if (split > 0) {
             e = dsa_launch_tile_dq(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, split, causal, dq,
                                    fuse_delta ? out : nullptr, delta, sq);
@@ -490,7 +496,7 @@ static int attn_bwd_run(const void *dout, const void *q, const void *k, const vo
             if (e != hipSuccess) rc = hip_fail(e, "gather dq launch");
         }
     }
-    if (rc == DSA_OK && (parts & DSA_BWD_DKV)) {
+    if (rc == DSA_OK && !ov && (parts & DSA_BWD_DKV)) {
         e = dsa_launch_tile_dkv(dout, q, k, v, lse, delta, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, causal, order, partial,
                                 partial_bytes, dk, dv, st);
         if (e != hipSuccess) rc = hip_fail(e, "tile dkv launch");
