@@ -16,7 +16,8 @@
  *     n (T) int32: how many are valid.  idx == NULL and n == NULL select every causal key of the
  *     token's own segment (the reference's dense causal semantics);
  *   - lse (Hq,T) fp32 natural-log softmax normaliser (what the flash kernel behind varlen_attn saves);
- *   - stream is a hipStream_t passed as void*; all work is enqueued on it, nothing synchronises;
+ *   - stream is a hipStream_t passed as void*; all work is ordered on it, nothing synchronises (the backward may run
+ *     one of its passes on a second stream between a fork and a join event on this one: dsa_set_bwd_overlap);
  *   - every entry returns 0 on success or a negative dsa_status; dsa_last_error() gives the text
  *     (thread-local).  No exception crosses the boundary.
  */
@@ -137,6 +138,23 @@ size_t dsa_indexer_bwd_workspace_bytes(int T, int Di, int max_seqlen);
 int dsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
                  const int32_t *cu_seqlens, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
                  int dtype, int max_seqlen, int causal, void *out, float *lse, void *ws, size_t ws_bytes, void *stream);
+
+/*
+ * The selection bitmap without a pass over the finished list (no reference counterpart).  dsa_index_topk_bitmap is
+ * dsa_index_topk (sel_scores == NULL) or dsa_index_topk_scores (sel_scores != NULL) whose top-k kernel also leaves,
+ * in `bitmap`, what dsa_attn_fwd would build from idx/n in its workspace (same layout and size:
+ * dsa_attn_fwd_workspace_bytes(T, max_seqlen, 1)) - the ballots of its compaction are those words already.
+ * dsa_attn_fwd_saved_bitmap is dsa_attn_fwd reading such a bitmap (made with the same idx, n, cu_seqlens and
+ * max_seqlen by dsa_index_topk_bitmap or by an earlier dsa_attn_fwd) instead of building it; the same buffer then
+ * serves dsa_attn_bwd_saved_bitmap.  With the tile crossover at 0 no kernel reads the bitmap.
+ */
+int dsa_index_topk_bitmap(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu_seqlens, int T, int N,
+                          int Hi, int Di, int K, float scale, int dtype, int max_seqlen, int32_t *idx, int32_t *n,
+                          float *sel_scores, void *bitmap, size_t bitmap_bytes, void *ws, size_t ws_bytes, void *stream);
+int dsa_attn_fwd_saved_bitmap(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
+                              const int32_t *cu_seqlens, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
+                              int dtype, int max_seqlen, int causal, void *out, float *lse, const void *bitmap,
+                              size_t bitmap_bytes, void *stream);
 
 /* Bytes of workspace dsa_attn_fwd needs (the inverted selection bitmap; 0 without idx). */
 size_t dsa_attn_fwd_workspace_bytes(int T, int max_seqlen, int has_idx);

@@ -491,6 +491,38 @@ def test_backward_is_deterministic_and_unselected_keys_get_zero():
     assert (grads[0][1][~used] == 0).all() and (grads[0][2][~used] == 0).all()
 
 
+@pytest.mark.parametrize("segs,K", [
+    ((700, 333, 40, 0, 515, 204), 256),       # rows inside and beyond top_k, an empty segment
+    ((9000, 100), 512),                       # rows beyond the LDS cache of the selection kernel
+    ((65,), 64), ((1100, 64, 600, 284), 2048),  # one key more than top_k; top_k above every row
+])
+def test_bitmap_left_by_the_selection_kernel_equals_the_one_built_from_the_list(segs, K):
+    """index_topk(..., bitmap=) writes, from the ballots of its compaction, the words the forward builds from idx/n:
+    every byte of the rows equal (also the zero words behind a row's window, over a buffer that held other bytes), same
+    idx/n/scores as without it, and a forward and backward that read it give the bits of the ones that build their own;
+    for the exact longest segment and for the bound T (odd word counts per row)."""
+    _log(f"bitmap from top-k segs={segs} K={K}")
+    w = W.scaled(W.C2, segs, top_k=K, name="bm")
+    t = W.make_inputs(w, device=DEV)
+    cu, scale, lib = t["cu_seqlens"], w.D ** -0.5, ops._lib.load()
+    for ms in (w.max_seqlen, w.T):
+        nbytes, used = lib.dsa_attn_fwd_workspace_bytes(w.T, ms, 1), w.T * ((ms + 31) // 32) * 4
+        a = torch.full((nbytes,), 0xAB, dtype=torch.uint8, device=DEV)
+        b = torch.full((nbytes,), 0xCD, dtype=torch.uint8, device=DEV)
+        idx, n, sel = ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, ms, K, return_scores=True, bitmap=a)
+        idx2, n2, sel2 = ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, ms, K, return_scores=True)
+        assert torch.equal(idx, idx2) and torch.equal(n, n2) and torch.equal(sel, sel2)
+        a2 = torch.full((nbytes,), 0x17, dtype=torch.uint8, device=DEV)
+        idx3, n3 = ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, ms, K, bitmap=a2)
+        assert torch.equal(idx, idx3) and torch.equal(n, n3)
+        out, lse = ops.attn_fwd(t["q"], t["k"], t["v"], idx, n, cu, ms, scale, ws=b)
+        assert torch.equal(a[:used], b[:used]) and torch.equal(a2[:used], b[:used])
+        out2, lse2 = ops.attn_fwd(t["q"], t["k"], t["v"], idx, n, cu, ms, scale, ws=a, bitmap_ready=True)
+        assert torch.equal(out, out2) and torch.equal(lse, lse2) and torch.equal(a[:used], b[:used])
+    with pytest.raises(RuntimeError, match="selection bitmap"):
+        ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, w.max_seqlen, K, bitmap=a[:8])
+
+
 @pytest.mark.parametrize("sparse", [True, False])
 def test_backward_passes_side_by_side_give_the_same_bits(sparse):
     """dQ on the library's second stream beside dK/dV (modes 1 and 2) against one pass after the other (mode 0), with

@@ -11,7 +11,7 @@
 
 extern "C" {
 hipError_t dsa_launch_topk(const float *scores, int64_t ld, int row_begin, int row_end, const int32_t *cu, int N,
-                           int K, int max_row, int32_t *idx, int32_t *n, hipStream_t stream);
+                           int K, int max_row, int32_t *idx, int32_t *n, uint32_t *bitmap, int ldw, hipStream_t stream);
 hipError_t dsa_launch_gather_scores(const float *scores, int64_t ld, int row_begin, int row_end, const int32_t *cu, int N,
                                     int K, const int32_t *idx, const int32_t *n, float *sel, hipStream_t stream);
 hipError_t dsa_launch_indexer_kl(const float *sel, const float *mass, const int32_t *n, int T, int K, float grad_scale,
@@ -124,7 +124,7 @@ extern "C" int dsa_topk_from_scores(const float *scores, int64_t ld, int row_beg
     if (!scores || !idx || !n) return fail(DSA_ERR_ARG, "null tensor pointer");
     if (K < 1) return fail(DSA_ERR_ARG, "top_k=%d must be >= 1", K);
     if (row_begin < 0 || row_end > T || row_begin > row_end) return fail(DSA_ERR_ARG, "bad row range [%d,%d)", row_begin, row_end);
-    hipError_t e = dsa_launch_topk(scores, ld, row_begin, row_end, cu, N, K, (int)ld, idx, n, (hipStream_t)stream);
+    hipError_t e = dsa_launch_topk(scores, ld, row_begin, row_end, cu, N, K, (int)ld, idx, n, nullptr, 0, (hipStream_t)stream);
     return e == hipSuccess ? DSA_OK : hip_fail(e, "top-k launch");
 }
 
@@ -138,11 +138,13 @@ extern "C" size_t dsa_index_topk_workspace_bytes(int T, int max_seqlen, int K) {
     return align_up(rows, 4) * row_bytes;
 }
 
+static inline int bitmap_ldw(int max_seqlen) { return (max_seqlen + 31) / 32; }   // words of a row of the selection bitmap
+
 // sel_scores != NULL: every row is scored (also those whose whole causal window is selected) and the scores of
-// the selected keys are kept
+// the selected keys are kept; bitmap != NULL: the top-k kernel also leaves the inverted selection there
 static int index_topk_impl(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu, int T, int N,
                            int Hi, int Di, int K, float scale, int dtype, int max_seqlen, int32_t *idx, int32_t *n,
-                           float *sel_scores, void *ws, size_t ws_bytes, void *stream) {
+                           float *sel_scores, uint32_t *bitmap, void *ws, size_t ws_bytes, void *stream) {
     if (int rc = check_packed(T, N, cu)) return rc;
     if (K < 1) return fail(DSA_ERR_ARG, "top_k=%d must be >= 1", K);
     if (max_seqlen < 1 || max_seqlen > T) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
@@ -161,7 +163,8 @@ static int index_topk_impl(const void *q_idx, const void *k_idx, const void *w_i
                                         (float *)ws, ld, stream);
             if (rc) return rc;
         }
-        hipError_t e = dsa_launch_topk((const float *)ws, ld, (int)r0, r1, cu, N, K, max_seqlen, idx, n, (hipStream_t)stream);
+        hipError_t e = dsa_launch_topk((const float *)ws, ld, (int)r0, r1, cu, N, K, max_seqlen, idx, n, bitmap,
+                                       bitmap_ldw(max_seqlen), (hipStream_t)stream);
         if (e != hipSuccess) return hip_fail(e, "top-k launch");
         if (sel_scores) {
             e = dsa_launch_gather_scores((const float *)ws, ld, (int)r0, r1, cu, N, K, idx, n, sel_scores, (hipStream_t)stream);
@@ -174,16 +177,16 @@ static int index_topk_impl(const void *q_idx, const void *k_idx, const void *w_i
 extern "C" int dsa_index_topk(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu, int T, int N,
                               int Hi, int Di, int K, float scale, int dtype, int max_seqlen, int32_t *idx, int32_t *n,
                               void *ws, size_t ws_bytes, void *stream) {
-    return index_topk_impl(q_idx, k_idx, w_idx, cu, T, N, Hi, Di, K, scale, dtype, max_seqlen, idx, n, nullptr, ws, ws_bytes,
-                           stream);
+    return index_topk_impl(q_idx, k_idx, w_idx, cu, T, N, Hi, Di, K, scale, dtype, max_seqlen, idx, n, nullptr, nullptr, ws,
+                           ws_bytes, stream);
 }
 
 extern "C" int dsa_index_topk_scores(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu, int T,
                                      int N, int Hi, int Di, int K, float scale, int dtype, int max_seqlen, int32_t *idx,
                                      int32_t *n, float *sel_scores, void *ws, size_t ws_bytes, void *stream) {
     if (!sel_scores) return fail(DSA_ERR_ARG, "null output pointer");
-    return index_topk_impl(q_idx, k_idx, w_idx, cu, T, N, Hi, Di, K, scale, dtype, max_seqlen, idx, n, sel_scores, ws,
-                           ws_bytes, stream);
+    return index_topk_impl(q_idx, k_idx, w_idx, cu, T, N, Hi, Di, K, scale, dtype, max_seqlen, idx, n, sel_scores, nullptr,
+                           ws, ws_bytes, stream);
 }
 
 // ---- dsa_index_topk for callers that cannot allocate -------------------------------------------------------
@@ -227,7 +230,7 @@ extern "C" int dsa_index_topk_noalloc(const void *q_idx, const void *k_idx, cons
     if (int rc = scratch_of_current_device(&ws)) return rc;
     // nothing in the scratch has to start at zero: the indexer writes every column [0, pos] of a row before the
     // selection reads it, and rows whose whole window is selected are never read
-    return index_topk_impl(q_idx, k_idx, w_idx, cu, T, N, Hi, Di, K, scale, dtype, max_seqlen, idx, n, nullptr, ws,
+    return index_topk_impl(q_idx, k_idx, w_idx, cu, T, N, Hi, Di, K, scale, dtype, max_seqlen, idx, n, nullptr, nullptr, ws,
                            DSA_SCRATCH_BYTES, stream);
 }
 
@@ -253,8 +256,6 @@ static int check_attn(int T, int N, const int32_t *cu, int Hq, int Hkv, int D, i
     return DSA_OK;
 }
 
-static inline int bitmap_ldw(int max_seqlen) { return (max_seqlen + 31) / 32; }
-
 // Query rows whose position in their segment is below top_k * crossover are handled by the tile
 // kernels (their selection covers more than 1/crossover of the causal window), the rest by the
 // gather kernels.  Process-wide tuning knob; 0 = gather only, a huge value = tile only.
@@ -279,10 +280,10 @@ extern "C" size_t dsa_attn_fwd_workspace_bytes(int T, int max_seqlen, int has_id
     return align_up((size_t)T * bitmap_ldw(max_seqlen) * 4, 256);
 }
 
-extern "C" int dsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
-                            const int32_t *cu, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
-                            int dtype, int max_seqlen, int causal, void *out, float *lse, void *ws, size_t ws_bytes,
-                            void *stream) {
+// build_bitmap == 0: ws already holds the bitmap of idx/n (it is only read)
+static int attn_fwd_run(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n, const int32_t *cu,
+                        int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen, int causal,
+                        void *out, float *lse, void *ws, size_t ws_bytes, int build_bitmap, void *stream) {
     if (int rc = check_attn(T, N, cu, Hq, Hkv, D, K, dtype, idx, n)) return rc;
     if (!causal && idx) return fail(DSA_ERR_ARG, "a key selection (idx) implies causal attention");
     if (!q || !k || !v || !out || !lse) return fail(DSA_ERR_ARG, "null tensor pointer");
@@ -299,8 +300,10 @@ extern "C" int dsa_attn_fwd(const void *q, const void *k, const void *v, const i
             if (!ws || ws_bytes < need) return fail(DSA_ERR_WORKSPACE, "forward workspace: have %zu bytes, need %zu", ws_bytes, need);
             if ((size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);
             bitmap = (uint32_t *)ws;
-            e = dsa_launch_bitmap(idx, n, cu, N, T, K, ldw, bitmap, st);
-            if (e != hipSuccess) return hip_fail(e, "bitmap launch");
+            if (build_bitmap) {
+                e = dsa_launch_bitmap(idx, n, cu, N, T, K, ldw, bitmap, st);
+                if (e != hipSuccess) return hip_fail(e, "bitmap launch");
+            }
         }
         e = dsa_launch_tile_fwd(q, k, v, bitmap, ldw, cu, N, T, Hq, Hkv, D, softmax_scale, split, causal, out, lse, st);
         if (e != hipSuccess) return hip_fail(e, "tile forward launch");
@@ -310,6 +313,35 @@ extern "C" int dsa_attn_fwd(const void *q, const void *k, const void *v, const i
         if (e != hipSuccess) return hip_fail(e, "gather forward launch");
     }
     return DSA_OK;
+}
+
+extern "C" int dsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
+                            const int32_t *cu, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
+                            int dtype, int max_seqlen, int causal, void *out, float *lse, void *ws, size_t ws_bytes,
+                            void *stream) {
+    return attn_fwd_run(q, k, v, idx, n, cu, T, N, Hq, Hkv, D, K, softmax_scale, dtype, max_seqlen, causal, out, lse, ws, ws_bytes,
+                        1, stream);
+}
+
+extern "C" int dsa_attn_fwd_saved_bitmap(const void *q, const void *k, const void *v, const int32_t *idx, const int32_t *n,
+                                         const int32_t *cu, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
+                                         int dtype, int max_seqlen, int causal, void *out, float *lse, const void *bitmap,
+                                         size_t bitmap_bytes, void *stream) {
+    if (!idx) return fail(DSA_ERR_ARG, "a saved bitmap belongs to a selection: idx is null");
+    return attn_fwd_run(q, k, v, idx, n, cu, T, N, Hq, Hkv, D, K, softmax_scale, dtype, max_seqlen, causal, out, lse,
+                        const_cast<void *>(bitmap), bitmap_bytes, 0, stream);
+}
+
+extern "C" int dsa_index_topk_bitmap(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu, int T, int N,
+                                     int Hi, int Di, int K, float scale, int dtype, int max_seqlen, int32_t *idx, int32_t *n,
+                                     float *sel_scores, void *bitmap, size_t bitmap_bytes, void *ws, size_t ws_bytes,
+                                     void *stream) {
+    if (T > 0 && max_seqlen >= 1) {
+        const size_t need = dsa_attn_fwd_workspace_bytes(T, max_seqlen, 1);
+        if (!bitmap || bitmap_bytes < need) return fail(DSA_ERR_WORKSPACE, "selection bitmap: have %zu bytes, need %zu", bitmap_bytes, need);
+    }
+    return index_topk_impl(q_idx, k_idx, w_idx, cu, T, N, Hi, Di, K, scale, dtype, max_seqlen, idx, n, sel_scores,
+                           (uint32_t *)bitmap, ws, ws_bytes, stream);
 }
 
 // ---- attention mass of the selected keys (training target of the indexer) ---------------------------

@@ -10,6 +10,10 @@
 //      output offset, so the result comes out ascending and deterministic without sorting.
 //
 // Rows up to TOPK_LDS_CAP keys are read from HBM once and kept in LDS as keys.
+//
+// With a bitmap pointer the kernel also leaves the row's inverted selection (bit c of the row's ldw words = "key column c
+// of the segment is selected", what dsa_bitmap_kernel builds from the finished list): the compaction's ballots are those
+// words already, so the list need not be read back.
 #include "dsa_common.h"
 
 #define TOPK_THREADS 256
@@ -29,7 +33,8 @@ __device__ __forceinline__ uint32_t score_key(float x) {
 template <bool CACHED>
 __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
     const float *__restrict__ scores, int64_t ld, int row_begin, const int32_t *__restrict__ cu, int N, int K, int lds_keys,
-    int only, int skip_upto, int32_t *__restrict__ idx_out, int32_t *__restrict__ n_out) {
+    int only, int skip_upto, int32_t *__restrict__ idx_out, int32_t *__restrict__ n_out, uint32_t *__restrict__ bitmap,
+    int ldw) {
     __shared__ uint32_t hist[TOPK_BINS];
     __shared__ uint32_t wave_tot[4];
     __shared__ uint32_t sel_digit, sel_remaining;
@@ -47,9 +52,15 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
     if (only == 1 && nvalid > lds_keys) return;
     if (only == 2 && nvalid <= skip_upto) return;
 
+    uint32_t *brow = bitmap ? bitmap + (int64_t)t * ldw : nullptr;
     if (nvalid <= K) {
         for (int i = tid; i < K; i += TOPK_THREADS) orow[i] = (i < nvalid) ? (s0 + i) : -1;
         if (tid == 0) n_out[t] = nvalid;
+        if (brow)
+            for (int w = tid; w < ldw; w += TOPK_THREADS) {
+                const int left = nvalid - 32 * w;       // columns of this word inside the window
+                brow[w] = left >= 32 ? ~0u : (left > 0 ? (1u << left) - 1u : 0u);
+            }
         return;
     }
     const float *row = scores + (int64_t)(t - row_begin) * ld;
@@ -193,26 +204,32 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
             // count, hence the bound on the slot
             const uint32_t slot = out_pos + (uint32_t)__popcll(b_take & lt_mask);
             if (take && slot < (uint32_t)K) orow[slot] = s0 + i;
+            if (brow && lane < 2) {                     // the ballot is the two bitmap words of these 64 columns
+                const int w = ((base + u * 64) >> 5) + lane;
+                if (w < ldw) brow[w] = (uint32_t)(b_take >> (32 * lane));
+            }
             out_pos += (uint32_t)__popcll(b_take);
             eq_seen += (uint32_t)__popcll(b_eq);
         }
     }
+    if (brow)                                           // the words behind the window: the quarters end on 64 columns
+        for (int w = 2 * ((nvalid + 63) >> 6) + tid; w < ldw; w += TOPK_THREADS) brow[w] = 0u;
     if (tid == 0) n_out[t] = K;
 }
 
 extern "C" hipError_t dsa_launch_topk(const float *scores, int64_t ld, int row_begin, int row_end,
                                       const int32_t *cu, int N, int K, int max_row, int32_t *idx, int32_t *n,
-                                      hipStream_t stream) {
+                                      uint32_t *bitmap, int ldw, hipStream_t stream) {
     const int rows = row_end - row_begin;
     if (rows <= 0) return hipSuccess;
     if (max_row <= TOPK_LDS_CAP) {
         hipLaunchKernelGGL(dsa_topk_rows_kernel<true>, dim3(rows), dim3(TOPK_THREADS), (size_t)((max_row + 3) & ~3) * 4, stream,
-                           scores, ld, row_begin, cu, N, K, (max_row + 3) & ~3, 0, 0, idx, n);
+                           scores, ld, row_begin, cu, N, K, (max_row + 3) & ~3, 0, 0, idx, n, bitmap, ldw);
     } else {
         hipLaunchKernelGGL(dsa_topk_rows_kernel<true>, dim3(rows), dim3(TOPK_THREADS), (size_t)TOPK_LDS_CAP * 4, stream, scores,
-                           ld, row_begin, cu, N, K, TOPK_LDS_CAP, 1, 0, idx, n);
+                           ld, row_begin, cu, N, K, TOPK_LDS_CAP, 1, 0, idx, n, bitmap, ldw);
         hipLaunchKernelGGL(dsa_topk_rows_kernel<false>, dim3(rows), dim3(TOPK_THREADS), 16, stream, scores, ld, row_begin, cu,
-                           N, K, 0, 2, TOPK_LDS_CAP, idx, n);
+                           N, K, 0, 2, TOPK_LDS_CAP, idx, n, bitmap, ldw);
     }
     return hipGetLastError();
 }

@@ -112,9 +112,11 @@ def topk_from_scores(scores: torch.Tensor, cu_seqlens, top_k: int) -> Tuple[torc
 
 
 def index_topk(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen: int, top_k: int,
-               index_scale: Optional[float] = None, return_scores: bool = False):
+               index_scale: Optional[float] = None, return_scores: bool = False, bitmap=None):
     """Stages D1+D2: selected key rows per query, (idx (T,K) int32 ascending/-1 padded, n (T,) int32);
-    ``return_scores=True`` adds the (T,K) fp32 indexer scores of the selected keys (0 past n[t])."""
+    ``return_scores=True`` adds the (T,K) fp32 indexer scores of the selected keys (0 past n[t]).  ``bitmap`` (uint8, the
+    size of the forward's workspace) receives the inverted selection the forward would otherwise build from the list:
+    pass it on as ``attn_fwd(..., ws=bitmap, bitmap_ready=True)``."""
     _require_cuda(q_idx, k_idx, w_idx, cu_seqlens)
     if q_idx.dim() != 3 or k_idx.dim() != 2 or w_idx.dim() != 2:
         raise ValueError("indexer tensors must be q_idx (T,Hi,Di), k_idx (T,Di), w_idx (T,Hi)")
@@ -136,6 +138,13 @@ def index_topk(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen: int, top_k: int,
         # as it is in the CPU restatement of the selection
         if not (torch.isfinite(qi.float()).all() and torch.isfinite(ki.float()).all() and torch.isfinite(wi.float()).all()):
             raise ValueError("non-finite indexer inputs: their scores have no defined rank")
+    if bitmap is not None:
+        sel = torch.empty((T, top_k), dtype=torch.float32, device=q_idx.device) if return_scores else None
+        rc = lib.dsa_index_topk_bitmap(_ptr(qi), _ptr(ki), _ptr(wi), _ptr(cu), T, cu.numel() - 1, Hi, Di, top_k, scale,
+                                       _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(idx), _ptr(n), _ptr(sel), _ptr(bitmap),
+                                       bitmap.numel(), _ptr(ws), ws_bytes, _stream(q_idx.device))
+        _lib.check(rc, "dsa_index_topk_bitmap")
+        return (idx, n, sel) if return_scores else (idx, n)
     if return_scores:
         sel = torch.empty((T, top_k), dtype=torch.float32, device=q_idx.device)
         rc = lib.dsa_index_topk_scores(_ptr(qi), _ptr(ki), _ptr(wi), _ptr(cu), T, cu.numel() - 1, Hi, Di, top_k, scale,
@@ -253,9 +262,11 @@ def set_bwd_overlap(mode: int) -> int:
     return old
 
 
-def attn_fwd(q, k, v, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float, causal: bool = True, ws=None):
-    """Stage D3.  ``ws`` (optional, uint8) is used as the workspace instead of a fresh allocation; the
-    autograd wrapper passes the tail of the backward workspace so that the selection bitmap is built once."""
+def attn_fwd(q, k, v, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float, causal: bool = True, ws=None,
+             bitmap_ready: bool = False):
+    """Stage D3.  ``ws`` (optional, uint8) is used as the workspace instead of a fresh allocation: the autograd wrapper
+    keeps it for the backward, so that the selection bitmap is built once.  ``bitmap_ready``: ``ws`` already holds the
+    bitmap of this selection (``index_topk(..., bitmap=ws)``) and is only read."""
     T, Hq, Hkv, D = _check_qkv(q, k, v)
     cu = _check_cu(cu_seqlens, T)
     out = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=q.device)
@@ -267,6 +278,12 @@ def attn_fwd(q, k, v, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float,
         ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q.device)
     elif ws.numel() < ws_bytes:
         raise ValueError(f"forward workspace: have {ws.numel()} bytes, need {ws_bytes}")
+    if bitmap_ready:
+        rc = lib.dsa_attn_fwd_saved_bitmap(_ptr(q), _ptr(k), _ptr(v), _ptr(idx), _ptr(n), _ptr(cu), T, cu.numel() - 1, Hq, Hkv,
+                                           D, K, softmax_scale, _lib.DSA_DTYPE_BF16, max_seqlen, 1 if causal else 0, _ptr(out),
+                                           _ptr(lse), _ptr(ws), ws_bytes, _stream(q.device))
+        _lib.check(rc, "dsa_attn_fwd_saved_bitmap")
+        return out, lse
     rc = lib.dsa_attn_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(idx), _ptr(n), _ptr(cu), T, cu.numel() - 1, Hq, Hkv, D, K,
                           softmax_scale, _lib.DSA_DTYPE_BF16, max_seqlen, 1 if causal else 0, _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
                           _stream(q.device))
@@ -397,7 +414,7 @@ class _DsaVarlenAttn(torch.autograd.Function):
     Other dtypes / larger head_dim are rounded to bf16 once."""
 
     @staticmethod
-    def forward(ctx, q, k, v, cu_seqlens, max_seqlen, idx, n, softmax_scale, causal=True, want_mass=False):
+    def forward(ctx, q, k, v, cu_seqlens, max_seqlen, idx, n, softmax_scale, causal=True, want_mass=False, bitmap=None):
         in_dtype = q.dtype
         D = q.shape[-1]
         split = in_dtype == torch.float32 and 4 * D <= 256
@@ -407,12 +424,14 @@ class _DsaVarlenAttn(torch.autograd.Function):
             qb, kb, vb = _as_bf16(q), _as_bf16(k), _as_bf16(v)
         fwd_ws = None
         lib = _lib.load()
-        if idx is not None and lib.dsa_get_tile_crossover() > 0:     # (crossover 0: the forward builds no bitmap)
-            # the selection bitmap the forward builds is kept for the backward; nothing else is held in between
-            # (delta, the key-tile order and the partial sums of cut walks are allocated when the backward runs)
-            fwd_ws = torch.empty((max(lib.dsa_attn_fwd_workspace_bytes(qb.shape[0], int(max_seqlen), 1), 4),),
-                                 dtype=torch.uint8, device=qb.device)
-        out, lse = attn_fwd(qb, kb, vb, idx, n, cu_seqlens, int(max_seqlen), softmax_scale, causal, ws=fwd_ws)
+        if idx is not None and lib.dsa_get_tile_crossover() > 0:     # (crossover 0: no kernel reads a bitmap)
+            # the selection bitmap - left by the top-k kernel (`bitmap`), else built by the forward - is kept for the
+            # backward; nothing else is held in between (delta, the key-tile order and the partial sums of cut walks
+            # are allocated when the backward runs)
+            fwd_ws = bitmap if bitmap is not None else torch.empty(
+                (max(lib.dsa_attn_fwd_workspace_bytes(qb.shape[0], int(max_seqlen), 1), 4),), dtype=torch.uint8, device=qb.device)
+        out, lse = attn_fwd(qb, kb, vb, idx, n, cu_seqlens, int(max_seqlen), softmax_scale, causal, ws=fwd_ws,
+                            bitmap_ready=fwd_ws is not None and bitmap is not None)
         ctx.fwd_ws = fwd_ws
         ctx.causal = bool(causal)
         ctx.save_for_backward(qb, kb, vb, out, lse, cu_seqlens, *(() if idx is None else (idx, n)))
@@ -454,7 +473,7 @@ class _DsaVarlenAttn(torch.autograd.Function):
             dq, dk, dv = _split_combine_qkv(dq, dk, dv)
         elif ctx.in_dtype != torch.bfloat16:
             dq, dk, dv = dq.to(ctx.in_dtype), dk.to(ctx.in_dtype), dv.to(ctx.in_dtype)
-        return dq, dk, dv, None, None, None, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None, None, None, None
 
 
 @torch.compiler.disable                                  # a compiled caller (the reference compiles per block) breaks the graph here
@@ -486,7 +505,7 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, in
     cu = _check_cu(cu_seqlens, T, max_seqlen)
     scale = float(softmax_scale) if softmax_scale is not None else D ** -0.5
     sparse = indexer_q is not None or indexer_k is not None or indexer_w is not None
-    idx = n = None
+    idx = n = bitmap = None
     if sparse and not causal:
         raise ValueError("DSA key selection is defined for causal attention only")
     if sparse:
@@ -494,12 +513,17 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, in
             raise ValueError("DSA needs indexer_q, indexer_k, indexer_w and top_k together")
         if indexer_q.shape[0] != T:
             raise ValueError("indexer tensors must cover the same T packed tokens as q")
+        lib = _lib.load()
+        if lib.dsa_get_tile_crossover() > 0:
+            # the top-k kernel leaves the inverted selection here: forward and backward read it, nothing builds it again
+            bitmap = torch.empty((max(lib.dsa_attn_fwd_workspace_bytes(T, int(max_seqlen), 1), 4),), dtype=torch.uint8,
+                                 device=q.device)
         with torch.no_grad():
             if return_scores:
                 idx, n, sel_scores = index_topk(indexer_q, indexer_k, indexer_w, cu, int(max_seqlen), int(top_k), index_scale,
-                                                return_scores=True)
+                                                return_scores=True, bitmap=bitmap)
             else:
-                idx, n = index_topk(indexer_q, indexer_k, indexer_w, cu, int(max_seqlen), int(top_k), index_scale)
+                idx, n = index_topk(indexer_q, indexer_k, indexer_w, cu, int(max_seqlen), int(top_k), index_scale, bitmap=bitmap)
     elif return_indices or return_scores:
         raise ValueError("return_indices / return_scores need the indexer inputs")
     dims = _KERNEL_HEAD_DIMS if sparse else _KERNEL_HEAD_DIMS_DENSE
@@ -512,7 +536,7 @@ def dsa_varlen_attn(q, k, v, cu_seqlens, max_seqlen: Optional[int] = None, *, in
     if return_mass and not sparse:
         raise ValueError("return_mass needs the indexer inputs")
     out = _DsaVarlenAttn.apply(q.contiguous(), k.contiguous(), v.contiguous(), cu, int(max_seqlen), idx, n, scale,
-                               bool(causal), bool(return_mass))
+                               bool(causal), bool(return_mass), bitmap)
     mass = None
     if return_mass:
         out, mass = out
