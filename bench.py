@@ -291,18 +291,27 @@ def main():
     it = max(2, min(args.steps, 20))
     with torch.no_grad():
         qd, kd, vd = q.detach(), k.detach(), v.detach()
-        idx, n = ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k)
-        out, lse = ops.attn_fwd(qd, kd, vd, idx, n, cu, msl, scale)
+        # as the operator runs them: the selection kernel leaves the bitmap, forward and backward read it, and the
+        # query side of the backward forms delta itself where it owns every row (else the delta pass runs with it)
+        lib = ops._lib.load()
+        bm = torch.empty((max(lib.dsa_attn_fwd_workspace_bytes(w.T, msl, 1), 4),), dtype=torch.uint8, device=dev) \
+            if lib.dsa_get_tile_crossover() > 0 else None
+        idx, n = ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k, bitmap=bm)
+        out, lse = ops.attn_fwd(qd, kd, vd, idx, n, cu, msl, scale, ws=bm, bitmap_ready=bm is not None)
         bufs = ops.attn_bwd(t["dout"], qd, kd, vd, out, lse, idx, n, cu, msl, scale, 15,
                             (torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd),
                              torch.empty((ops._lib.load().dsa_attn_bwd_workspace_bytes(w.T, w.Hq, msl, 1),),
                                          dtype=torch.uint8, device=dev)))
         stage_ms = {
-            "index_topk": timed(lambda: ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k), it),
-            "attn_fwd": timed(lambda: ops.attn_fwd(qd, kd, vd, idx, n, cu, msl, scale), it),
+            "index_topk": timed(lambda: ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k, bitmap=bm), it),
+            "attn_fwd": timed(lambda: ops.attn_fwd(qd, kd, vd, idx, n, cu, msl, scale, ws=bm, bitmap_ready=bm is not None), it),
         }
-        for name, part in (("bwd_delta", 1), ("bwd_bitmap", 2), ("bwd_dq", 4), ("bwd_dkv", 8)):
+        # (part bits: 1 delta, 2 bitmap from the list, 4 query side, 8 key side)
+        for name, part in (("bwd_dq", 1 | 4), ("bwd_dkv", 8)):
             stage_ms[name] = timed(lambda: ops.attn_bwd(t["dout"], qd, kd, vd, out, lse, idx, n, cu, msl, scale, part, bufs), it)
+        # passes the step no longer runs at this workload, alone, for comparison
+        passes_alone = {name: timed(lambda: ops.attn_bwd(t["dout"], qd, kd, vd, out, lse, idx, n, cu, msl, scale, part, bufs), it)
+                        for name, part in (("delta_pass", 1), ("bitmap_from_list", 2), ("dq_reading_delta", 4))}
 
     # ---- roofline ----------------------------------------------------------------------------
     wk = w.work()
@@ -333,7 +342,7 @@ def main():
     # per stage: measured time against the stage's nominal roofline (the larger of flop / MFMA peak and bytes / HBM
     # peak, the bytes being those a row gather of the selected keys would move) and against its flop alone
     stage_time = {"index_topk": stage_ms["index_topk"], "attn_fwd": stage_ms["attn_fwd"],
-                  "attn_bwd": stage_ms["bwd_delta"] + stage_ms["bwd_bitmap"] + stage_ms["bwd_dq"] + stage_ms["bwd_dkv"]}
+                  "attn_bwd": stage_ms["bwd_dq"] + stage_ms["bwd_dkv"]}
     stage_work = {"index_topk": (wk["F1"], wk["B2"]), "attn_fwd": (wk["F3"], wk["B3"]), "attn_bwd": (wk["F4"], wk["B4"])}
     stage_roofline = {}
     for name, (flop, nbytes) in stage_work.items():
@@ -365,6 +374,7 @@ def main():
                      "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command, scaled by a 1 GiB copy (profiles/)",
                      "algorithmic_flop": dom_flop, "avg_ms": stage_ms[dom]},
         "stage_ms": stage_ms,
+        "passes_alone_ms": passes_alone,
         "ms_per_step_median": pct(0.5), "ms_per_step_p10": pct(0.1), "ms_per_step_p90": pct(0.9),
         "roofline_whole_op": {"compute_only_bound_ms": compute_bound_ms, "frac_compute_only": compute_bound_ms / ms_per_step,
                               "nominal_gather_roofline_ms": roof_total, "nominal_t_roof_ms": t_roof_ms, "stages": stage_roofline,
