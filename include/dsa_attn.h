@@ -321,6 +321,14 @@ int dsa_split_bf16_stack_qkv(const float *q, const float *k, const float *v, int
 int dsa_split_bf16_combine_qkv(const void *yq, const void *yk, const void *yv, int64_t rows_q, int64_t rows_kv, int D,
                                float *dq, float *dk, float *dv, void *stream);
 
+/*
+ * Three fp32 arrays of na, nb, nc elements rounded to bf16 (to nearest even, what tensor.to(torch.bfloat16) gives) by one
+ * launch: the indexer's three inputs when the caller holds them in fp32 (no reference counterpart: the reference runs
+ * under bf16 autocast).  Inputs 16-byte aligned, outputs 8-byte aligned.
+ */
+int dsa_round_bf16_x3(const float *a, const float *b, const float *c, int64_t na, int64_t nb, int64_t nc, void *ya, void *yb,
+                      void *yc, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

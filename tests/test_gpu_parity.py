@@ -159,6 +159,30 @@ def test_fp32_carrier_of_three_operands_equals_the_single_operand_launches():
     assert [x.shape[0] for x in e] == [0, 0, 0]
 
 
+def test_three_fp32_arrays_rounded_to_bf16_by_one_launch_equal_torch_casts():
+    """The indexer's inputs of an fp32 caller: same bits as tensor.to(torch.bfloat16) (round to nearest even, infinities,
+    signed zeros, subnormals, values that round up to the next power of two), NaN stays NaN; odd element counts."""
+    _log("fp32 -> bf16 x3")
+    g = torch.Generator(device=DEV).manual_seed(9)
+    a = torch.randn(333, 5, 32, device=DEV, generator=g)
+    b = torch.randn(333, 32, device=DEV, generator=g) * 1e-3
+    c = torch.randn(333, 5, device=DEV, generator=g) * 1e4
+    special = torch.tensor([0.0, -0.0, float("inf"), -float("inf"), 1.0 + 2.0 ** -8, 1.0 + 2.0 ** -9, 1.0 + 3 * 2.0 ** -9,
+                            1.99999988, 3.3895314e38, 1e-40, -1e-45, 65504.0], device=DEV)
+    c.view(-1)[:special.numel()] = special
+    c.view(-1)[-1] = float("nan")
+    ya, yb, yc = ops._as_bf16_x3(a, b, c)
+    for y, x in ((ya, a), (yb, b), (yc, c)):
+        want = x.to(torch.bfloat16)
+        assert y.shape == x.shape and y.dtype == torch.bfloat16 and y.is_contiguous()
+        assert torch.equal(torch.isnan(y), torch.isnan(want))
+        ok = ~torch.isnan(want)
+        assert torch.equal(y.view(torch.int16)[ok], want.view(torch.int16)[ok])
+    # anything but three fp32 tensors goes through the plain casts
+    h = ops._as_bf16_x3(a.half(), b, c)
+    assert torch.equal(h[0], a.half().to(torch.bfloat16)) and torch.equal(h[1], b.to(torch.bfloat16))
+
+
 @pytest.mark.parametrize("name,segs,K", [
     ("C2", (700, 333, 40, 0, 515, 204), 256),
     ("C3", (1100, 64, 600, 284), 512),

@@ -80,6 +80,7 @@ _SIGNATURES = {
     "dsa_sigmoid_gate_fwd": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_int, c_int, c_void_p, c_void_p]),
     "dsa_split_bf16_stack": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p]),
     "dsa_split_bf16_combine": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p]),
+    "dsa_round_bf16_x3": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "dsa_split_bf16_stack_qkv": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p, c_void_p,
                                          c_void_p]),
     "dsa_split_bf16_combine_qkv": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p,

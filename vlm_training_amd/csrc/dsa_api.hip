@@ -69,6 +69,8 @@ hipError_t dsa_launch_sigmoid_gate_fwd(const void *x, const void *gate, int64_t 
                                        int64_t rows, void *y, hipStream_t stream);
 hipError_t dsa_launch_split_stack(const float *x, int64_t rows, int D, int order, void *y, hipStream_t stream);
 hipError_t dsa_launch_split_combine(const void *y, int64_t rows, int D, int part, float *out, hipStream_t stream);
+hipError_t dsa_launch_round_bf16_x3(const float *a, const float *b, const float *c, int64_t na, int64_t nb, int64_t nc, void *ya,
+                                    void *yb, void *yc, hipStream_t stream);
 hipError_t dsa_launch_split_stack_qkv(const float *q, const float *k, const float *v, int64_t rows_q, int64_t rows_kv, int D, void *yq,
                                       void *yk, void *yv, hipStream_t stream);
 hipError_t dsa_launch_split_combine_qkv(const void *yq, const void *yk, const void *yv, int64_t rows_q, int64_t rows_kv, int D,
@@ -728,4 +730,15 @@ extern "C" int dsa_split_bf16_combine_qkv(const void *yq, const void *yk, const 
     if ((rows_q > 0 && (!yq || !dq)) || (rows_kv > 0 && (!yk || !yv || !dk || !dv))) return fail(DSA_ERR_ARG, "null tensor pointer");
     hipError_t e = dsa_launch_split_combine_qkv(yq, yk, yv, rows_q, rows_kv, D, dq, dk, dv, (hipStream_t)stream);
     return e == hipSuccess ? DSA_OK : hip_fail(e, "split/combine launch");
+}
+
+// ---- three fp32 arrays rounded to bf16 by one launch (the indexer's inputs of an fp32 caller) ----
+extern "C" int dsa_round_bf16_x3(const float *a, const float *b, const float *c, int64_t na, int64_t nb, int64_t nc, void *ya,
+                                 void *yb, void *yc, void *stream) {
+    if (na < 0 || nb < 0 || nc < 0) return fail(DSA_ERR_ARG, "negative element count");
+    if ((na > 0 && (!a || !ya)) || (nb > 0 && (!b || !yb)) || (nc > 0 && (!c || !yc))) return fail(DSA_ERR_ARG, "null tensor pointer");
+    if ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15) || (((uintptr_t)ya | (uintptr_t)yb | (uintptr_t)yc) & 7))
+        return fail(DSA_ERR_ARG, "inputs must be 16-byte aligned, outputs 8-byte aligned");
+    hipError_t e = dsa_launch_round_bf16_x3(a, b, c, na, nb, nc, ya, yb, yc, (hipStream_t)stream);
+    return e == hipSuccess ? DSA_OK : hip_fail(e, "bf16 rounding launch");
 }

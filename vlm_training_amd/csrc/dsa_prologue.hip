@@ -411,3 +411,38 @@ extern "C" hipError_t dsa_launch_split_combine_qkv(const void *yq, const void *y
                        (const bf16_t *)yv, rows_q, rows_kv, D, dq, dk, dv);
     return hipGetLastError();
 }
+
+// ---------------------------------------------------------------------------------------------------
+// fp32 -> bf16 (round to nearest even, the hardware conversion) of three arrays in one launch: the indexer's inputs of
+// an fp32 caller.  Four elements per thread; the last one to three of an array go one by one.
+// ---------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void round4_bf16(const float *__restrict__ x, int64_t i4, int64_t n, bf16_t *__restrict__ y) {
+    const int64_t i = i4 * 4;
+    if (i + 4 <= n) {
+        const f32x4 v = *reinterpret_cast<const f32x4 *>(x + i);
+        const u32x2 o = {pack2bf(v[0], v[1]), pack2bf(v[2], v[3])};
+        *reinterpret_cast<u32x2 *>(y + i) = o;
+    } else {
+        for (int64_t j = i; j < n; ++j) y[j] = (bf16_t)x[j];
+    }
+}
+__global__ __launch_bounds__(256) void dsa_round_bf16_x3_kernel(const float *__restrict__ a, const float *__restrict__ b,
+                                                                 const float *__restrict__ c, int64_t na, int64_t nb, int64_t nc,
+                                                                 bf16_t *__restrict__ ya, bf16_t *__restrict__ yb,
+                                                                 bf16_t *__restrict__ yc) {
+    const int64_t qa = (na + 3) / 4, qb = (nb + 3) / 4, qc = (nc + 3) / 4;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < qa + qb + qc; i += (int64_t)gridDim.x * 256) {
+        if (i < qa) round4_bf16(a, i, na, ya);
+        else if (i < qa + qb) round4_bf16(b, i - qa, nb, yb);
+        else round4_bf16(c, i - qa - qb, nc, yc);
+    }
+}
+extern "C" hipError_t dsa_launch_round_bf16_x3(const float *a, const float *b, const float *c, int64_t na, int64_t nb, int64_t nc,
+                                               void *ya, void *yb, void *yc, hipStream_t stream) {
+    const int64_t n4 = (na + 3) / 4 + (nb + 3) / 4 + (nc + 3) / 4;
+    if (n4 == 0) return hipSuccess;
+    const int nb_ = (int)((n4 + 255) / 256 > 8192 ? 8192 : (n4 + 255) / 256);
+    hipLaunchKernelGGL(dsa_round_bf16_x3_kernel, dim3(nb_), dim3(256), 0, stream, a, b, c, na, nb, nc, (bf16_t *)ya, (bf16_t *)yb,
+                       (bf16_t *)yc);
+    return hipGetLastError();
+}

@@ -36,6 +36,26 @@ def _as_bf16(t: torch.Tensor) -> torch.Tensor:
     return (t if t.dtype == torch.bfloat16 else t.to(torch.bfloat16)).contiguous()
 
 
+def _as_bf16_x3(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor):
+    """Three tensors to bf16; three fp32 ones by one launch instead of three casts."""
+    if not (a.dtype == b.dtype == c.dtype == torch.float32) or not (a.is_cuda and a.numel()):
+        return _as_bf16(a), _as_bf16(b), _as_bf16(c)
+    a, b, c = a.contiguous(), b.contiguous(), c.contiguous()
+    if (a.data_ptr() | b.data_ptr() | c.data_ptr()) & 15:
+        return _as_bf16(a), _as_bf16(b), _as_bf16(c)
+    # one buffer, each part on a 16-byte boundary
+    offs, total = [], 0
+    for t in (a, b, c):
+        offs.append(total)
+        total += (t.numel() + 7) // 8 * 8
+    buf = torch.empty((total,), dtype=torch.bfloat16, device=a.device)
+    ys = [buf[o:o + t.numel()].view(t.shape) for o, t in zip(offs, (a, b, c))]
+    rc = _lib.load().dsa_round_bf16_x3(_ptr(a), _ptr(b), _ptr(c), a.numel(), b.numel(), c.numel(), _ptr(ys[0]), _ptr(ys[1]),
+                                       _ptr(ys[2]), _stream(a.device))
+    _lib.check(rc, "dsa_round_bf16_x3")
+    return ys[0], ys[1], ys[2]
+
+
 def _check_cu(cu_seqlens: torch.Tensor, T: int, max_seqlen: Optional[int] = None):
     if cu_seqlens.dim() != 1 or cu_seqlens.numel() < 2:
         raise ValueError("cu_seqlens must be 1-D with at least two entries")
@@ -87,7 +107,7 @@ def indexer_scores(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen: int, index_scale
     ld = (max_seqlen + 31) // 32 * 32
     scores = torch.full((T, ld), float("-inf"), dtype=torch.float32, device=q_idx.device)
     lib = _lib.load()
-    qi, ki, wi = _as_bf16(q_idx), _as_bf16(k_idx), _as_bf16(w_idx)     # keep the casts alive over the launch
+    qi, ki, wi = _as_bf16_x3(q_idx, k_idx, w_idx)                      # keep the casts alive over the launch
     rc = lib.dsa_indexer_scores(_ptr(qi), _ptr(ki), _ptr(wi), _ptr(cu), T,
                                 cu.numel() - 1, Hi, Di, scale, _lib.DSA_DTYPE_BF16, 0, T, skip_dense_k, _ptr(scores), ld,
                                 _stream(q_idx.device))
@@ -132,7 +152,7 @@ def index_topk(q_idx, k_idx, w_idx, cu_seqlens, max_seqlen: int, top_k: int,
     n = torch.empty((T,), dtype=torch.int32, device=q_idx.device)
     ws_bytes = lib.dsa_index_topk_workspace_bytes(T, max_seqlen, top_k) if (max_seqlen > top_k or return_scores) else 0
     ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q_idx.device)
-    qi, ki, wi = _as_bf16(q_idx), _as_bf16(k_idx), _as_bf16(w_idx)     # keep the casts alive over the launch
+    qi, ki, wi = _as_bf16_x3(q_idx, k_idx, w_idx)                      # keep the casts alive over the launch
     if os.environ.get("DSA_DEBUG_NAN"):
         # the device ranks NaN above +inf without a word; with this switch (one device-to-host copy) it is an error,
         # as it is in the CPU restatement of the selection
@@ -186,7 +206,7 @@ def indexer_bwd(q_idx, k_idx, w_idx, idx, n, dscore, cu_seqlens, max_seqlen: int
         raise ValueError("dscore must be (T,K) fp32")
     scale = index_scale if index_scale is not None else (Di ** -0.5) * (Hi ** -0.5)
     lib = _lib.load()
-    qi, ki, wi = _as_bf16(q_idx), _as_bf16(k_idx), _as_bf16(w_idx)
+    qi, ki, wi = _as_bf16_x3(q_idx, k_idx, w_idx)
     d_kernel = next((d for d in (64, 128) if d >= Di), None)
     if d_kernel is not None and d_kernel != Di:          # e.g. 32-wide index heads: zero columns change no score
         pad = d_kernel - Di
