@@ -363,6 +363,49 @@ def test_dense_path_equals_reference_semantics():
         assert_close_bf16(vd.grad, vr.grad, "dv")
 
 
+@pytest.mark.parametrize("profile", ["rising", "falling", "all_low", "spikes", "all_high"])
+@pytest.mark.parametrize("D", [128, 256])
+def test_forward_reference_point_follows_logits_of_any_scale(profile, D):
+    """The forward forms P against a running reference and looks for a tile's maximum only when a sum says it must:
+    logits that rise by hundreds along the keys (the reference has to move again and again), fall (it never moves
+    after the first tile), sit far below zero (nothing may underflow as a whole), far above (nothing may overflow),
+    or spike in single keys - out, lse and dv against fp32 softmax of the same bf16 inputs."""
+    _log(f"reference point {profile} D={D}")
+    g = torch.Generator().manual_seed(3)
+    T, Hq, Hkv = 700, 4, 2
+    cu = [0, 450, 700]
+    u = torch.nn.functional.normalize(torch.randn(D, generator=g), dim=0)
+    pos = torch.arange(T, dtype=torch.float32)
+    level = {"rising": pos * 0.6 - 100, "falling": 150 - pos * 0.6, "all_low": -300 + torch.randn(T, generator=g),
+             "all_high": 300 + torch.randn(T, generator=g),
+             "spikes": torch.where((pos.long() % 97) == 13, torch.tensor(120.0), torch.tensor(-20.0))}[profile]
+    # logit(t, s) = scale * q[t].k[s] = level[s] + noise: q = sqrt(D) u (+ noise), k[s] = level[s] u (+ noise)
+    q = (D ** 0.5 * u + 0.05 * torch.randn(T, Hq, D, generator=g)).bfloat16()
+    k = (level[:, None, None] * u + 0.05 * torch.randn(T, Hkv, D, generator=g)).bfloat16()
+    v = torch.randn(T, Hkv, D, generator=g).bfloat16()
+    do = torch.randn(T, Hq, D, generator=g).bfloat16()
+    cu_d = torch.tensor(cu, dtype=torch.int32, device=DEV)
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    out = ops.dsa_varlen_attn(qd, kd, vd, cu_d, 450)
+    out.backward(do.to(DEV))
+    _, lse = ops.attn_fwd(q.to(DEV), k.to(DEV), v.to(DEV), None, None, cu_d, 450, D ** -0.5)
+    qr, kr, vr = (x.float().requires_grad_(True) for x in (q, k, v))
+    ref = R.dense_varlen_causal(qr, kr, vr, cu)
+    ref.backward(do.float())
+    want_lse = torch.empty(Hq, T)
+    for a, b in zip(cu[:-1], cu[1:]):
+        logit = torch.einsum("thd,shd->hts", q[a:b].float(), k[a:b].float().repeat_interleave(Hq // Hkv, dim=1)) * D ** -0.5
+        logit = logit.masked_fill(torch.ones(b - a, b - a, dtype=torch.bool).triu(1), float("-inf"))
+        want_lse[:, a:b] = torch.logsumexp(logit, dim=-1)
+    assert torch.isfinite(lse).all()
+    assert (lse.cpu() - want_lse).abs().max() <= 2e-3 * max(1.0, want_lse.abs().max().item())
+    assert_close_bf16(out, ref, f"out {profile}")
+    # (keys of norm 300 multiply the bf16 rounding of dS into dq far beyond the bound of ordinary inputs: the backward
+    # is checked for the finite results and for dv, which no key scales)
+    assert all(torch.isfinite(x.grad).all() for x in (qd, kd, vd))
+    assert_close_bf16(vd.grad, vr.grad, "dv", steps=2)
+
+
 @pytest.mark.parametrize("Hq,Hkv,D,causal,segs", [
     (16, 16, 72, False, (1024, 300, 77)),                  # the 1152 / 16 vision tower: padded to the head_dim-96 kernels
     (8, 2, 96, True, (700, 1, 333, 1500)),                 # head_dim 96 itself, causal, four heads per kv head

@@ -296,6 +296,43 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
         *reinterpret_cast<u32x4 *>(&lds[BUF][0][tile_off<D>(row, ch)]) = kst[SET][i];              \
         *reinterpret_cast<u32x4 *>(&lds[BUF][1][tile_off<D>(row, ch)]) = vst[SET][i];              \
     }
+// Online softmax of one tile.  The row maximum is not searched in every tile: P is formed against the running
+// reference first, and only when a lane's sum says that some probability may have passed 2^8 - or a live row has not met
+// a selected key yet - does the wave look for the tile's maximum, move the reference, rescale the sums and form P
+// again: the first tile of a block, then rarely.  In between P stays below 2^8, exact in fp32 and safe in bf16, and
+// never underflows as a whole, because the reference is a maximum the row has really met.  (Searching the maximum in
+// every tile, 16 more vector instructions per tile, was 4-5 % slower at 32 768 tokens.)
+#define FWD_SOFTMAX                                                                                \
+        float s2[16], pr[16];                                                                      \
+        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi)                                          \
+            s2[vi] = keep_or_neginf(sacc[vi], bit_mask(word, 8 * (vi >> 2) + (vi & 3)));           \
+        float psum = 0.f;                                                                          \
+        {                                                                                          \
+            const float mneg = (mrun == -INFINITY) ? 0.f : -mrun;                                  \
+            _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                    \
+                pr[vi] = fast_exp2(fmaf(s2[vi], scale_log2, mneg));                                \
+                psum += pr[vi];                                                                    \
+            }                                                                                      \
+        }                                                                                          \
+        if (__builtin_amdgcn_ballot_w64(row_ok && (mrun == -INFINITY || !(psum <= 256.f)))) {      \
+            float mloc = -INFINITY;                                                                \
+            _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) mloc = fmaxf(mloc, s2[vi]);          \
+            mloc = half_max_f(mloc) * scale_log2;                                                  \
+            if (mloc > mrun) {                                                                     \
+                const float alpha = fast_exp2(mrun - mloc);   /* mrun = -inf: 0, and the sums are 0 */ \
+                lsum *= alpha;                                                                     \
+                _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) oacc[dt] *= alpha;               \
+                mrun = mloc;                                                                       \
+            }                                                                                      \
+            const float mneg = (mrun == -INFINITY) ? 0.f : -mrun;                                  \
+            psum = 0.f;                                                                            \
+            _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                    \
+                pr[vi] = fast_exp2(fmaf(s2[vi], scale_log2, mneg));                                \
+                psum += pr[vi];                                                                    \
+            }                                                                                      \
+        }                                                                                          \
+        lsum += psum;                                                                              \
+        const bf16x8 pB0 = pack8(pr), pB1 = pack8(pr + 8);
 #define FWD_COMPUTE(TILE, BUF)                                                                      \
     {                                                                                              \
         const int kc0 = (TILE) * 32;                                                               \
@@ -311,30 +348,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
             _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) sacc = mfma32(ka[ks], qB[ks], sacc); \
             sched_reads_ahead<KS, 4, 1>();                                                         \
         }                                                                                          \
-        float s2[16], mloc = -INFINITY;                                                            \
-        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
-            s2[vi] = keep_or_neginf(sacc[vi], bit_mask(word, 8 * (vi >> 2) + (vi & 3)));           \
-            mloc = fmaxf(mloc, s2[vi]);                                                            \
-        }                                                                                          \
-        mloc = half_max_f(mloc) * scale_log2;                                     \
-        /* the reference maximum only moves when a row's maximum grows by more than 2^8 (rare      \
-           after the first tiles); until then P stays below 2^8, exact in fp32 and safe in bf16 */ \
-        if (__builtin_amdgcn_ballot_w64(mloc > mrun + 8.f)) {                                      \
-            const float mnew = fmaxf(mrun, mloc);                                                  \
-            float alpha = fast_exp2(mrun - ((mnew == -INFINITY) ? 0.f : mnew));                    \
-            asm volatile("" : "+v"(alpha));              /* keep the rescale inside the branch */   \
-            lsum *= alpha;                                                                         \
-            _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) oacc[dt] *= alpha;                   \
-            mrun = mnew;                                                                           \
-        }                                                                                          \
-        const float mneg = (mrun == -INFINITY) ? 0.f : -mrun; /* rows with nothing selected yet */   \
-        float psum = 0.f;                                                                          \
-        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
-            s2[vi] = fast_exp2(fmaf(s2[vi], scale_log2, mneg));                                    \
-            psum += s2[vi];                                                                        \
-        }                                                                                          \
-        lsum += psum;                                                                              \
-        const bf16x8 pB0 = pack8(s2), pB1 = pack8(s2 + 8);                                         \
+        FWD_SOFTMAX                                                                                \
         _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
             mfma32_acc(oacc[dt], lo.trop(vt, 0, dt), pB0);                          \
             mfma32_acc(oacc[dt], lo.trop(vt, 1, dt), pB1);                     \
@@ -345,6 +359,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
 #undef FWD_LOAD
 #undef FWD_STORE
 #undef FWD_COMPUTE
+#undef FWD_SOFTMAX
 
     float l = half_sum_f(lsum);
     if (row_ok) {
@@ -1481,8 +1496,12 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkvpc_kernel(
                 *reinterpret_cast<u32x4 *>(slot + lds_off[i]) = qv;
                 *reinterpret_cast<u32x4 *>(slot + TILE_B + lds_off[i]) = dv4;
             }
-            if (ctid < 32) lse_s[ctid] = __uint_as_float(aux_st) * LOG2E_F;
-            else if (ctid < 64) dlt_s[ctid - 32] = __uint_as_float(aux_st);
+            // a row that is not live (past the segment, past the walk, a padded head) has q = dO = 0 but would read a
+            // live row's lse: with lse far below zero its P = exp(0 - lse) overflows and 0 * inf reaches dK and dV.  It gets
+            // an lse that makes P vanish instead.
+            const bool row_dead = b > last || (b == 0 && aux_over > 0) || ((ctid & 31) & (Gp - 1)) >= G;
+            if (ctid < 32) lse_s[ctid] = row_dead ? 1e30f : __uint_as_float(aux_st) * LOG2E_F;
+            else if (ctid < 64) dlt_s[ctid - 32] = row_dead ? 0.f : __uint_as_float(aux_st);
             else if (HAS_IDX && ctid < 64 + 4 * QB)
                 mask_s[((ctid - 64) / QB) * 32 + (ctid - 64) % QB] =
                     (aux_mask_ok && !(b > last || (b == 0 && aux_over > 0))) ? aux_st : 0u;
@@ -1742,10 +1761,13 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
     int aux_q = 0, aux_stride = 0, aux_lds = 4 * AUX_SLOT;          // spare word behind the four slots
     float aux_mul = 0.f;
     uint32_t aux_and = 0u;
-    bool aux_is_word = false;
+    bool aux_is_word = false, aux_pad = false;
+    uint32_t aux_dead_value = 0u;                    // what a row that is not live stores: word 0, delta 0, -lse/scale -1e30
     if (ctid < 64) {                                 // 0..31: lse of row ctid, 32..63: delta of row ctid-32
         const int row = ctid & 31;
         const int hd = min(row & (Gp - 1), G - 1);
+        aux_pad = (row & (Gp - 1)) >= G;
+        aux_dead_value = ctid < 32 ? __float_as_uint(-1e30f) : 0u;
         aux_q = row >> GSHIFT;
         aux_stride = 1;
         aux_base = reinterpret_cast<const uint32_t *>((ctid < 32 ? lse : delta) + (int64_t)(kvh * G + hd) * T + s0);
@@ -1802,9 +1824,12 @@ __global__ __launch_bounds__(512, 1) void dsa_tile_dkv2_kernel(
                 *reinterpret_cast<u32x4 *>(slot + TILE_B + lds_off[i]) = live ? dost[i] : z4;
             }
         }
-        const bool word_dead = aux_is_word && (b > last || (b == 0 && aux_over > 0));
+        // a row that is not live (past the segment, past the walk, a padded head) has q = dO = 0 but would read a live
+        // row's lse: with lse far below zero its P = exp(0 - lse) overflows and 0 * inf reaches dK and dV.  Its selection
+        // word is cleared, and its S starts so low that P vanishes also where no selection masks it.
+        const bool dead = b > last || (b == 0 && aux_over > 0) || aux_pad;
         *reinterpret_cast<uint32_t *>(aux_ring + (aux_lds < 4 * AUX_SLOT ? (b & 3) * AUX_SLOT : 0) + aux_lds) =
-            word_dead ? 0u : aux_value(aux_st);
+            dead ? aux_dead_value : aux_value(aux_st);
     };
     // steady forms (blocks 2 .. last of a group whose heads fill the padded group): no branch, no select
     auto gload_steady = [&](u32x4 (&qst)[CPT], u32x4 (&dost)[CPT], uint32_t &aux_st) __attribute__((always_inline)) {
