@@ -666,9 +666,9 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
         float ds[16];                                                                              \
         _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
             const float dsv = __shfl(dl, 8 * (vi >> 2) + (vi & 3) + 4 * h, 64);   /* element vi is key column 8*(vi/4)+4h+vi%4 */ \
-            const float sv = sacc[vi];                                                             \
-            dwacc = fmaf(dsv, fmaxf(sv, 0.f), dwacc);                                              \
-            ds[vi] = sv > 0.f ? dsv * wrow_v : 0.f;                                                \
+            const float sv = sacc[vi];                   /* the row's weight multiplies the finished sum instead */ \
+            ds[vi] = sv > 0.f ? dsv : 0.f;                                                         \
+            dwacc = fmaf(ds[vi], sv, dwacc);             /* dscore * relu(s) */                     \
         }                                                                                          \
         const bf16x8 dB0 = pack8(ds), dB1 = pack8(ds + 8);                                         \
         _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
@@ -686,7 +686,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     if (row_ok) {
         bf16_t *op = dq_idx + ((int64_t)t * Hi + hrow) * D;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) store_c_tile(op + dt * 32, acc[dt], cscale, h);
+        for (int dt = 0; dt < DT; ++dt) store_c_tile(op + dt * 32, acc[dt], cscale * wrow_v, h);
         if (h == 0) dw[(int64_t)t * Hi + hrow] = dwt * cscale;
     }
 }
