@@ -2292,7 +2292,16 @@ extern "C" hipError_t dsa_launch_tile_mass(const void *q, const void *k, const f
 }
 // indexer backward: prefix table, query side (dq_idx, dw), key side (dk_idx).  D = indexer head_dim (64 or 128),
 // at most 64 indexer heads.
-#define IDXK_CHUNK 512                                   // queries per piece of a key tile's walk
+// Queries per piece of a key tile's walk in the indexer backward.  A piece is one workgroup and about 1.3 us per query:
+// the finer the pieces, the better a launch of few thousand of them balances over 512 workgroup slots (32 768 tokens:
+// 6.26 -> 5.95 ms with 256 instead of 512, 6.31 with 128; 8192 tokens: 0.44 -> 0.31 -> 0.25 ms), the more fp32 partial
+// sums (one (T, Di) plane per piece index).  Depends on T, and on the bound of the longest segment only where the
+// planes would pass 1.25 GiB.
+static int idxk_chunk(int T, int Di, int ldw) {
+    int c = T <= 16384 ? 128 : 256;
+    while ((size_t)((ldw * 32 + c - 1) / c) * T * Di * 4 > ((size_t)5 << 28) && c < (1 << 20)) c *= 2;
+    return c;
+}
 template <int D, int GS>
 static void launch_idx_bwd_i(hipStream_t stream, const void *q_idx, const void *k_idx, const void *w_idx, const float *dscore,
                              const uint32_t *bitmap, const int32_t *prefix, int ldw, const int32_t *cu, int N, int T, int Hi,
@@ -2302,14 +2311,16 @@ static void launch_idx_bwd_i(hipStream_t stream, const void *q_idx, const void *
     hipLaunchKernelGGL((dsa_tile_idxq_kernel<D, GS, NW>), gq, dim3(64 * NW), 0, stream, (const bf16_t *)q_idx,
                        (const bf16_t *)k_idx, (const bf16_t *)w_idx, dscore, bitmap, ldw, cu, N, T, Hi, K, cscale,
                        (bf16_t *)dq_idx, dw);
-    const dim3 gk((unsigned)((int64_t)T / 128 + N + 1), (unsigned)((ldw * 32 + IDXK_CHUNK - 1) / IDXK_CHUNK));
+    const int chunk = idxk_chunk(T, D, ldw);
+    const dim3 gk((unsigned)((int64_t)T / 128 + N + 1), (unsigned)((ldw * 32 + chunk - 1) / chunk));
     hipLaunchKernelGGL((dsa_tile_idxk_kernel<D, GS>), gk, dim3(256), 0, stream, (const bf16_t *)q_idx, (const bf16_t *)k_idx,
-                       (const bf16_t *)w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, IDXK_CHUNK, partial);
+                       (const bf16_t *)w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, chunk, partial);
     hipLaunchKernelGGL(dsa_idxk_reduce_kernel, dim3((unsigned)((T + 7) / 8)), dim3(256), 0, stream, partial, cu, N, T, D,
-                       IDXK_CHUNK, ldw * 32, (bf16_t *)dk_idx);
+                       chunk, ldw * 32, (bf16_t *)dk_idx);
 }
 extern "C" size_t dsa_indexer_bwd_partial_bytes(int T, int Di, int ldw) {
-    return (size_t)((ldw * 32 + IDXK_CHUNK - 1) / IDXK_CHUNK) * T * Di * 4;
+    const int chunk = idxk_chunk(T, Di, ldw);
+    return (size_t)((ldw * 32 + chunk - 1) / chunk) * T * Di * 4;
 }
 extern "C" hipError_t dsa_launch_indexer_bwd(const void *q_idx, const void *k_idx, const void *w_idx, const float *dscore,
                                              const uint32_t *bitmap, int32_t *prefix, int ldw, const int32_t *cu, int N,
