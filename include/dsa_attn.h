@@ -194,7 +194,7 @@ int dsa_get_tile_crossover(void);
  * on the first such call outside a capture) between a fork and a join event on the caller's stream, so that to the
  * caller the whole call is still ordered on the stream it passed; under stream capture the second stream joins the
  * capture through those events.  0: never (one stream).  2: for every launch size.  Results are the same bits in all
- * modes.
+ * modes.  dsa_indexer_bwd runs its query side and its key side the same way (mode 1: up to 16 384 tokens).
  */
 int dsa_set_bwd_overlap(int mode);
 int dsa_get_bwd_overlap(void);

@@ -989,8 +989,17 @@ def test_indexer_backward_matches_autograd_of_the_oracle(Hi, Di, K, segs):
     assert_close_bf16(dq, qi.grad, "dq_idx")
     assert_close_bf16(dk, ki.grad, "dk_idx")
     assert_close_bf16(dw, wi.grad, "dw")
-    dq2, dk2, dw2 = ops.indexer_bwd(d["q_idx"], d["k_idx"], d["w_idx"], idx, n, dscore.to(DEV), d["cu_seqlens"], w.max_seqlen)
-    assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dw, dw2)
+    # run to run, and with the query side on the library's second stream beside the key side or behind it: the same bits
+    old = ops.set_bwd_overlap(0)
+    try:
+        for mode in (0, 2, 1):
+            ops.set_bwd_overlap(mode)
+            dq2, dk2, dw2 = ops.indexer_bwd(d["q_idx"], d["k_idx"], d["w_idx"], idx, n, dscore.to(DEV), d["cu_seqlens"], w.max_seqlen)
+            tail = dq2.float().sum() + dk2.float().sum() + dw2.sum()      # queued right behind the call
+            assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dw, dw2), f"mode {mode}"
+            assert torch.isfinite(tail)
+    finally:
+        ops.set_bwd_overlap(old)
 
 
 def test_indexer_training_step_end_to_end():

@@ -32,7 +32,7 @@ hipError_t dsa_launch_gather_dq(const void *dout, const void *q, const void *k, 
 hipError_t dsa_launch_indexer_bwd(const void *q_idx, const void *k_idx, const void *w_idx, const float *dscore,
                                   const uint32_t *bitmap, int32_t *prefix, int ldw, const int32_t *cu, int N, int T, int Hi,
                                   int Di, int K, float cscale, void *dq_idx, void *dk_idx, float *dw, float *partial,
-                                  hipStream_t stream);
+                                  hipStream_t stream, hipStream_t stream_q);
 size_t dsa_indexer_bwd_partial_bytes(int T, int Di, int ldw);
 hipError_t dsa_launch_tile_mass(const void *q, const void *k, const float *lse, const uint32_t *bitmap, int ldw,
                                 const int32_t *n, const int32_t *cu, int N, int T, int Hq, int Hkv, int D, int K,
@@ -375,55 +375,6 @@ extern "C" int dsa_attn_mass(const void *q, const void *k, const float *lse, con
     return DSA_OK;
 }
 
-// ---- indexer backward: gradients of the selected scores w.r.t. the indexer's inputs --------------------
-extern "C" size_t dsa_indexer_bwd_workspace_bytes(int T, int Di, int max_seqlen) {
-    if (T <= 0) return 0;
-    const int ldw = bitmap_ldw(max_seqlen);                    // selection bitmap + slot prefix table + partial dk sums
-    return 2 * align_up((size_t)T * ldw * 4, 256) + align_up(dsa_indexer_bwd_partial_bytes(T, Di, ldw), 256);
-}
-
-extern "C" int dsa_indexer_bwd(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *idx, const int32_t *n,
-                               const float *dscore, const int32_t *cu, int T, int N, int Hi, int Di, int K, float scale,
-                               int dtype, int max_seqlen, void *dq_idx, void *dk_idx, float *dw, void *ws, size_t ws_bytes,
-                               void *stream) {
-    if (int rc = check_packed(T, N, cu)) return rc;
-    if (dtype != DSA_DTYPE_BF16) return fail(DSA_ERR_UNSUPPORTED, "indexer tensors must be bf16 (dtype code %d)", dtype);
-    if (Hi < 1 || Hi > 64) return fail(DSA_ERR_UNSUPPORTED, "Hi=%d: 1..64 indexer heads", Hi);
-    if (!(Di == 64 || Di == 128)) return fail(DSA_ERR_UNSUPPORTED, "Di=%d: the indexer backward covers 64 and 128", Di);
-    if (K < 1) return fail(DSA_ERR_ARG, "top_k=%d must be >= 1", K);
-    if (!q_idx || !k_idx || !w_idx || !idx || !n || !dscore || !dq_idx || !dk_idx || !dw) return fail(DSA_ERR_ARG, "null tensor pointer");
-    if (max_seqlen < 1 || max_seqlen > (T > 0 ? T : 1)) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
-    if (T == 0) return DSA_OK;
-    const size_t need = dsa_indexer_bwd_workspace_bytes(T, Di, max_seqlen);
-    if (!ws || ws_bytes < need) return fail(DSA_ERR_WORKSPACE, "indexer backward workspace: have %zu bytes, need %zu", ws_bytes, need);
-    const int ldw = bitmap_ldw(max_seqlen);
-    if ((size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);
-    hipStream_t st = (hipStream_t)stream;
-    const size_t bm = align_up((size_t)T * ldw * 4, 256);
-    uint32_t *bitmap = (uint32_t *)ws;
-    int32_t *prefix = (int32_t *)((char *)ws + bm);
-    float *partial = (float *)((char *)ws + 2 * bm);
-    hipError_t e = dsa_launch_bitmap(idx, n, cu, N, T, K, ldw, bitmap, st);
-    if (e != hipSuccess) return hip_fail(e, "bitmap launch");
-    e = dsa_launch_indexer_bwd(q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, Di, K, scale, dq_idx, dk_idx, dw,
-                               partial, st);
-    if (e != hipSuccess) return hip_fail(e, "indexer backward launch");
-    return DSA_OK;
-}
-
-extern "C" size_t dsa_attn_bwd_workspace_bytes(int T, int Hq, int max_seqlen, int has_idx) {
-    if (T <= 0) return 0;
-    size_t b = align_up((size_t)T * Hq * 4, 256);                                     // delta
-    if (has_idx) b += align_up((size_t)T * bitmap_ldw(max_seqlen) * 4, 256);          // selection bitmap
-    b += align_up(dsa_tile_dkv_partial_bytes(T), 256);                                // dK / dV of key-tile walks in pieces
-    return b + align_up(dsa_tile_order_bytes(T), 256);                                // launch order of the key tiles
-}
-
-extern "C" size_t dsa_attn_bwd_bitmap_offset(int T, int Hq) {
-    if (T <= 0 || Hq <= 0) return 0;
-    return align_up((size_t)T * Hq * 4, 256);
-}
-
 // ---- the query-side and the key-side pass of one backward side by side ----
 // Both read the same inputs and write different outputs, and a launch of few workgroups ends on its longest walks with
 // most CUs idle: the query side then runs on a second stream of the library's own (default priority, one per device,
@@ -469,6 +420,80 @@ static OverlapCtx *overlap_ctx(hipStream_t main_stream) {
         return nullptr;
     }
     return &c;
+}
+
+// ---- indexer backward: gradients of the selected scores w.r.t. the indexer's inputs --------------------
+extern "C" size_t dsa_indexer_bwd_workspace_bytes(int T, int Di, int max_seqlen) {
+    if (T <= 0) return 0;
+    const int ldw = bitmap_ldw(max_seqlen);                    // selection bitmap + slot prefix table + partial dk sums
+    return 2 * align_up((size_t)T * ldw * 4, 256) + align_up(dsa_indexer_bwd_partial_bytes(T, Di, ldw), 256);
+}
+
+extern "C" int dsa_indexer_bwd(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *idx, const int32_t *n,
+                               const float *dscore, const int32_t *cu, int T, int N, int Hi, int Di, int K, float scale,
+                               int dtype, int max_seqlen, void *dq_idx, void *dk_idx, float *dw, void *ws, size_t ws_bytes,
+                               void *stream) {
+    if (int rc = check_packed(T, N, cu)) return rc;
+    if (dtype != DSA_DTYPE_BF16) return fail(DSA_ERR_UNSUPPORTED, "indexer tensors must be bf16 (dtype code %d)", dtype);
+    if (Hi < 1 || Hi > 64) return fail(DSA_ERR_UNSUPPORTED, "Hi=%d: 1..64 indexer heads", Hi);
+    if (!(Di == 64 || Di == 128)) return fail(DSA_ERR_UNSUPPORTED, "Di=%d: the indexer backward covers 64 and 128", Di);
+    if (K < 1) return fail(DSA_ERR_ARG, "top_k=%d must be >= 1", K);
+    if (!q_idx || !k_idx || !w_idx || !idx || !n || !dscore || !dq_idx || !dk_idx || !dw) return fail(DSA_ERR_ARG, "null tensor pointer");
+    if (max_seqlen < 1 || max_seqlen > (T > 0 ? T : 1)) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
+    if (T == 0) return DSA_OK;
+    const size_t need = dsa_indexer_bwd_workspace_bytes(T, Di, max_seqlen);
+    if (!ws || ws_bytes < need) return fail(DSA_ERR_WORKSPACE, "indexer backward workspace: have %zu bytes, need %zu", ws_bytes, need);
+    const int ldw = bitmap_ldw(max_seqlen);
+    if ((size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);
+    hipStream_t st = (hipStream_t)stream;
+    const size_t bm = align_up((size_t)T * ldw * 4, 256);
+    uint32_t *bitmap = (uint32_t *)ws;
+    int32_t *prefix = (int32_t *)((char *)ws + bm);
+    float *partial = (float *)((char *)ws + 2 * bm);
+    hipError_t e = dsa_launch_bitmap(idx, n, cu, N, T, K, ldw, bitmap, st);
+    if (e != hipSuccess) return hip_fail(e, "bitmap launch");
+    // the query side (dq_idx, dw) and the key side (dk_idx) read the same inputs and write different outputs: side by
+    // side on two streams where dsa_set_bwd_overlap allows it, as the two passes of the attention backward
+    std::unique_lock<std::mutex> ov_lock;
+    OverlapCtx *ov = nullptr;
+    const int ov_mode = g_bwd_overlap.load(std::memory_order_relaxed);
+    // (mode 1: launches up to 16 384 tokens with T * max_seqlen * Hi * Di of at least 1e10 - 8192 tokens 0.24 -> 0.20 ms,
+    // 16 384 tokens 0.53 -> 0.48; at 32 768 tokens both sides fill the GPU alone and nothing is gained)
+    if (ov_mode == 2 || (ov_mode == 1 && T <= 16384 && (double)T * max_seqlen * Hi * Di >= 1e10)) {
+        ov_lock = std::unique_lock<std::mutex>(g_overlap_mu);
+        ov = overlap_ctx(st);
+        if (!ov) ov_lock.unlock();
+    }
+    hipStream_t sq = st;
+    if (ov) {
+        e = hipEventRecord(ov->fork, st);
+        if (e == hipSuccess) e = hipStreamWaitEvent(ov->aux, ov->fork, 0);
+        if (e != hipSuccess) return hip_fail(e, "fork to the second stream");
+        sq = ov->aux;
+    }
+    int rc = DSA_OK;
+    e = dsa_launch_indexer_bwd(q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, Di, K, scale, dq_idx, dk_idx, dw,
+                               partial, st, sq);
+    if (e != hipSuccess) rc = hip_fail(e, "indexer backward launch");
+    if (ov) {
+        e = hipEventRecord(ov->join, ov->aux);
+        if (e == hipSuccess) e = hipStreamWaitEvent(st, ov->join, 0);
+        if (e != hipSuccess && rc == DSA_OK) rc = hip_fail(e, "join of the second stream");
+    }
+    return rc;
+}
+
+extern "C" size_t dsa_attn_bwd_workspace_bytes(int T, int Hq, int max_seqlen, int has_idx) {
+    if (T <= 0) return 0;
+    size_t b = align_up((size_t)T * Hq * 4, 256);                                     // delta
+    if (has_idx) b += align_up((size_t)T * bitmap_ldw(max_seqlen) * 4, 256);          // selection bitmap
+    b += align_up(dsa_tile_dkv_partial_bytes(T), 256);                                // dK / dV of key-tile walks in pieces
+    return b + align_up(dsa_tile_order_bytes(T), 256);                                // launch order of the key tiles
+}
+
+extern "C" size_t dsa_attn_bwd_bitmap_offset(int T, int Hq) {
+    if (T <= 0 || Hq <= 0) return 0;
+    return align_up((size_t)T * Hq * 4, 256);
 }
 
 // the backward proper: every buffer named, so that the two entry points below differ only in where the buffers live

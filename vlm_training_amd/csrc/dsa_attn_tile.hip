@@ -2305,18 +2305,19 @@ static int idxk_chunk(int T, int Di, int ldw) {
 template <int D, int GS>
 static void launch_idx_bwd_i(hipStream_t stream, const void *q_idx, const void *k_idx, const void *w_idx, const float *dscore,
                              const uint32_t *bitmap, const int32_t *prefix, int ldw, const int32_t *cu, int N, int T, int Hi,
-                             int K, float cscale, void *dq_idx, void *dk_idx, float *dw, float *partial) {
+                             int K, float cscale, void *dq_idx, void *dk_idx, float *dw, float *partial, hipStream_t stream_q) {
     constexpr int NW = tile_waves<D>();
-    const dim3 gq((unsigned)((int64_t)T / ((32 * NW) >> GS) + N + 1));
-    hipLaunchKernelGGL((dsa_tile_idxq_kernel<D, GS, NW>), gq, dim3(64 * NW), 0, stream, (const bf16_t *)q_idx,
-                       (const bf16_t *)k_idx, (const bf16_t *)w_idx, dscore, bitmap, ldw, cu, N, T, Hi, K, cscale,
-                       (bf16_t *)dq_idx, dw);
+    // (the key side, the longer pass, is issued first: with two streams it gets the GPU first)
     const int chunk = idxk_chunk(T, D, ldw);
     const dim3 gk((unsigned)((int64_t)T / 128 + N + 1), (unsigned)((ldw * 32 + chunk - 1) / chunk));
     hipLaunchKernelGGL((dsa_tile_idxk_kernel<D, GS>), gk, dim3(256), 0, stream, (const bf16_t *)q_idx, (const bf16_t *)k_idx,
                        (const bf16_t *)w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, chunk, partial);
     hipLaunchKernelGGL(dsa_idxk_reduce_kernel, dim3((unsigned)((T + 7) / 8)), dim3(256), 0, stream, partial, cu, N, T, D,
                        chunk, ldw * 32, (bf16_t *)dk_idx);
+    const dim3 gq((unsigned)((int64_t)T / ((32 * NW) >> GS) + N + 1));
+    hipLaunchKernelGGL((dsa_tile_idxq_kernel<D, GS, NW>), gq, dim3(64 * NW), 0, stream_q, (const bf16_t *)q_idx,
+                       (const bf16_t *)k_idx, (const bf16_t *)w_idx, dscore, bitmap, ldw, cu, N, T, Hi, K, cscale,
+                       (bf16_t *)dq_idx, dw);
 }
 extern "C" size_t dsa_indexer_bwd_partial_bytes(int T, int Di, int ldw) {
     const int chunk = idxk_chunk(T, Di, ldw);
@@ -2325,15 +2326,15 @@ extern "C" size_t dsa_indexer_bwd_partial_bytes(int T, int Di, int ldw) {
 extern "C" hipError_t dsa_launch_indexer_bwd(const void *q_idx, const void *k_idx, const void *w_idx, const float *dscore,
                                              const uint32_t *bitmap, int32_t *prefix, int ldw, const int32_t *cu, int N,
                                              int T, int Hi, int Di, int K, float cscale, void *dq_idx, void *dk_idx,
-                                             float *dw, float *partial, hipStream_t stream) {
+                                             float *dw, float *partial, hipStream_t stream, hipStream_t stream_q) {
     if (Hi < 1 || Hi > 64 || !(Di == 64 || Di == 128)) return hipErrorInvalidValue;
     hipLaunchKernelGGL(dsa_bitmap_prefix_kernel, dim3(T), dim3(64), 0, stream, bitmap, ldw, prefix);
     if (Di == 128) {
-        if (Hi > 32) launch_idx_bwd_i<128, 6>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw, partial);
-        else launch_idx_bwd_i<128, 5>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw, partial);
+        if (Hi > 32) launch_idx_bwd_i<128, 6>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw, partial, stream_q);
+        else launch_idx_bwd_i<128, 5>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw, partial, stream_q);
     } else {
-        if (Hi > 32) launch_idx_bwd_i<64, 6>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw, partial);
-        else launch_idx_bwd_i<64, 5>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw, partial);
+        if (Hi > 32) launch_idx_bwd_i<64, 6>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw, partial, stream_q);
+        else launch_idx_bwd_i<64, 5>(stream, q_idx, k_idx, w_idx, dscore, bitmap, prefix, ldw, cu, N, T, Hi, K, cscale, dq_idx, dk_idx, dw, partial, stream_q);
     }
     return hipGetLastError();
 }
