@@ -11,9 +11,7 @@
 
 extern "C" {
 hipError_t dsa_launch_topk(const float *scores, int64_t ld, int row_begin, int row_end, const int32_t *cu, int N,
-                           int K, int max_row, int32_t *idx, int32_t *n, uint32_t *bitmap, int ldw, hipStream_t stream);
-hipError_t dsa_launch_gather_scores(const float *scores, int64_t ld, int row_begin, int row_end, const int32_t *cu, int N,
-                                    int K, const int32_t *idx, const int32_t *n, float *sel, hipStream_t stream);
+                           int K, int max_row, int32_t *idx, int32_t *n, uint32_t *bitmap, int ldw, float *sel, hipStream_t stream);
 hipError_t dsa_launch_indexer_kl(const float *sel, const float *mass, const int32_t *n, int T, int K, float grad_scale,
                                  float *loss, float *dscore, hipStream_t stream);
 hipError_t dsa_launch_indexer(const void *q_idx, const void *k_idx, const void *w_idx, const int32_t *cu, int N,
@@ -126,7 +124,7 @@ extern "C" int dsa_topk_from_scores(const float *scores, int64_t ld, int row_beg
     if (!scores || !idx || !n) return fail(DSA_ERR_ARG, "null tensor pointer");
     if (K < 1) return fail(DSA_ERR_ARG, "top_k=%d must be >= 1", K);
     if (row_begin < 0 || row_end > T || row_begin > row_end) return fail(DSA_ERR_ARG, "bad row range [%d,%d)", row_begin, row_end);
-    hipError_t e = dsa_launch_topk(scores, ld, row_begin, row_end, cu, N, K, (int)ld, idx, n, nullptr, 0, (hipStream_t)stream);
+    hipError_t e = dsa_launch_topk(scores, ld, row_begin, row_end, cu, N, K, (int)ld, idx, n, nullptr, 0, nullptr, (hipStream_t)stream);
     return e == hipSuccess ? DSA_OK : hip_fail(e, "top-k launch");
 }
 
@@ -166,12 +164,8 @@ static int index_topk_impl(const void *q_idx, const void *k_idx, const void *w_i
             if (rc) return rc;
         }
         hipError_t e = dsa_launch_topk((const float *)ws, ld, (int)r0, r1, cu, N, K, max_seqlen, idx, n, bitmap,
-                                       bitmap_ldw(max_seqlen), (hipStream_t)stream);
+                                       bitmap_ldw(max_seqlen), sel_scores, (hipStream_t)stream);
         if (e != hipSuccess) return hip_fail(e, "top-k launch");
-        if (sel_scores) {
-            e = dsa_launch_gather_scores((const float *)ws, ld, (int)r0, r1, cu, N, K, idx, n, sel_scores, (hipStream_t)stream);
-            if (e != hipSuccess) return hip_fail(e, "score gather launch");
-        }
     }
     return DSA_OK;
 }

@@ -10,6 +10,8 @@
 //      output offset, so the result comes out ascending and deterministic without sorting.
 //
 // Rows up to TOPK_LDS_CAP keys are read from HBM once and kept in LDS as keys.
+// With a sel_out pointer the kernel also writes the scores of the selected keys beside their indices (the key it ranks
+// by is the score, bit for bit, but for the sign of a zero).
 //
 // With a bitmap pointer the kernel also leaves the row's inverted selection (bit c of the row's ldw words = "key column c
 // of the segment is selected", what dsa_bitmap_kernel builds from the finished list): the compaction's ballots are those
@@ -20,6 +22,10 @@
 #define TOPK_LDS_CAP 8192
 #define TOPK_BINS 2048                                  // 11-bit digits (the last pass uses 1024 of them)
 
+// the score a key stands for (-0.0 comes back as +0.0: score_key folds the two)
+__device__ __forceinline__ float key_score(uint32_t k) {
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
 __device__ __forceinline__ uint32_t score_key(float x) {
     uint32_t u = __float_as_uint(x);
     if (u == 0x80000000u) u = 0u;                       // -0.0 ties with +0.0
@@ -34,7 +40,7 @@ template <bool CACHED>
 __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
     const float *__restrict__ scores, int64_t ld, int row_begin, const int32_t *__restrict__ cu, int N, int K, int lds_keys,
     int only, int skip_upto, int32_t *__restrict__ idx_out, int32_t *__restrict__ n_out, uint32_t *__restrict__ bitmap,
-    int ldw) {
+    int ldw, float *__restrict__ sel_out) {
     __shared__ uint32_t hist[TOPK_BINS];
     __shared__ uint32_t wave_tot[4];
     __shared__ uint32_t sel_digit, sel_remaining;
@@ -53,8 +59,12 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
     if (only == 2 && nvalid <= skip_upto) return;
 
     uint32_t *brow = bitmap ? bitmap + (int64_t)t * ldw : nullptr;
+    float *srow = sel_out ? sel_out + (int64_t)t * K : nullptr;   // the scores of the selected keys, slot by slot (0 past n)
+    const float *row = scores + (int64_t)(t - row_begin) * ld;
     if (nvalid <= K) {
         for (int i = tid; i < K; i += TOPK_THREADS) orow[i] = (i < nvalid) ? (s0 + i) : -1;
+        if (srow)
+            for (int i = tid; i < K; i += TOPK_THREADS) srow[i] = (i < nvalid) ? row[i] : 0.f;
         if (tid == 0) n_out[t] = nvalid;
         if (brow)
             for (int w = tid; w < ldw; w += TOPK_THREADS) {
@@ -63,7 +73,6 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
             }
         return;
     }
-    const float *row = scores + (int64_t)(t - row_begin) * ld;
     const bool cached = CACHED && nvalid <= lds_keys;    // a row beyond the stated longest one is read from memory each pass
     for (int i = tid; i < TOPK_BINS; i += TOPK_THREADS) hist[i] = 0u;
     __syncthreads();
@@ -203,7 +212,10 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
             // exactly K keys are taken when every score orders (the radix passes count them); NaN scores can break the
             // count, hence the bound on the slot
             const uint32_t slot = out_pos + (uint32_t)__popcll(b_take & lt_mask);
-            if (take && slot < (uint32_t)K) orow[slot] = s0 + i;
+            if (take && slot < (uint32_t)K) {
+                orow[slot] = s0 + i;
+                if (srow) srow[slot] = key_score(kk[u]);
+            }
             if (brow && lane < 2) {                     // the ballot is the two bitmap words of these 64 columns
                 const int w = ((base + u * 64) >> 5) + lane;
                 if (w < ldw) brow[w] = (uint32_t)(b_take >> (32 * lane));
@@ -219,37 +231,26 @@ __global__ __launch_bounds__(TOPK_THREADS) void dsa_topk_rows_kernel(
 
 extern "C" hipError_t dsa_launch_topk(const float *scores, int64_t ld, int row_begin, int row_end,
                                       const int32_t *cu, int N, int K, int max_row, int32_t *idx, int32_t *n,
-                                      uint32_t *bitmap, int ldw, hipStream_t stream) {
+                                      uint32_t *bitmap, int ldw, float *sel, hipStream_t stream) {
     const int rows = row_end - row_begin;
     if (rows <= 0) return hipSuccess;
     if (max_row <= TOPK_LDS_CAP) {
         hipLaunchKernelGGL(dsa_topk_rows_kernel<true>, dim3(rows), dim3(TOPK_THREADS), (size_t)((max_row + 3) & ~3) * 4, stream,
-                           scores, ld, row_begin, cu, N, K, (max_row + 3) & ~3, 0, 0, idx, n, bitmap, ldw);
+                           scores, ld, row_begin, cu, N, K, (max_row + 3) & ~3, 0, 0, idx, n, bitmap, ldw, sel);
     } else {
         hipLaunchKernelGGL(dsa_topk_rows_kernel<true>, dim3(rows), dim3(TOPK_THREADS), (size_t)TOPK_LDS_CAP * 4, stream, scores,
-                           ld, row_begin, cu, N, K, TOPK_LDS_CAP, 1, 0, idx, n, bitmap, ldw);
+                           ld, row_begin, cu, N, K, TOPK_LDS_CAP, 1, 0, idx, n, bitmap, ldw, sel);
         hipLaunchKernelGGL(dsa_topk_rows_kernel<false>, dim3(rows), dim3(TOPK_THREADS), 16, stream, scores, ld, row_begin, cu,
-                           N, K, 0, 2, TOPK_LDS_CAP, idx, n, bitmap, ldw);
+                           N, K, 0, 2, TOPK_LDS_CAP, idx, n, bitmap, ldw, sel);
     }
     return hipGetLastError();
 }
 
 // ------------------------------------------------------------------------------------------------
-// Indexer scores of the selected keys, sel[t,j] = score of key idx[t,j] (0 for j >= n[t]), picked out of
-// the chunk's score rows after its top-k; and the KL divergence of the indexer's distribution over the
-// selected keys from a target distribution (the attention mass), with its gradient w.r.t. the scores.
+// The KL divergence of the indexer's distribution over the selected keys (their scores sel[t,j], 0 for j >= n[t], come
+// out of the selection kernel's compaction) from a target distribution (the attention mass), with its gradient w.r.t.
+// the scores.
 // ------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void dsa_gather_scores_kernel(const float *__restrict__ scores, int64_t ld, int row_begin,
-                                                                 const int32_t *__restrict__ cu, int N, int K,
-                                                                 const int32_t *__restrict__ idx,
-                                                                 const int32_t *__restrict__ nsel, float *__restrict__ sel) {
-    const int t = row_begin + blockIdx.x;
-    const int s0 = cu[find_segment(cu, N, t)], nt = nsel[t];
-    const float *row = scores + (int64_t)(t - row_begin) * ld;
-    const int32_t *irow = idx + (int64_t)t * K;
-    float *orow = sel + (int64_t)t * K;
-    for (int j = threadIdx.x; j < K; j += 256) orow[j] = j < nt ? row[irow[j] - s0] : 0.f;
-}
 
 // block-wide reductions over 256 threads (4 waves)
 __device__ __forceinline__ float block_max_256(float v, float *red) {
@@ -297,14 +298,6 @@ __global__ __launch_bounds__(256) void dsa_indexer_kl_kernel(const float *__rest
     if (threadIdx.x == 0) loss[t] = nt > 0 ? acc : 0.f;
 }
 
-extern "C" hipError_t dsa_launch_gather_scores(const float *scores, int64_t ld, int row_begin, int row_end,
-                                               const int32_t *cu, int N, int K, const int32_t *idx, const int32_t *n,
-                                               float *sel, hipStream_t stream) {
-    if (row_end <= row_begin) return hipSuccess;
-    hipLaunchKernelGGL(dsa_gather_scores_kernel, dim3(row_end - row_begin), dim3(256), 0, stream, scores, ld, row_begin, cu, N,
-                       K, idx, n, sel);
-    return hipGetLastError();
-}
 extern "C" hipError_t dsa_launch_indexer_kl(const float *sel, const float *mass, const int32_t *n, int T, int K,
                                             float grad_scale, float *loss, float *dscore, hipStream_t stream) {
     if (T <= 0) return hipSuccess;
