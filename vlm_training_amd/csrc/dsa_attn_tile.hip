@@ -599,6 +599,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
     constexpr int NBUF = 2, NT = NW * 64, Gp = 1 << GSHIFT, QBW = (NW * 32) >> GSHIFT;
     static_assert(LOADS >= 1 && GSHIFT >= 5, "a wave's 32 rows are heads of one query");
     __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][TILE_B];
+    __shared__ __attribute__((aligned(16))) float dl_s[NW][32];      // per wave: the gradients of the current tile's 32 keys
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, h = lane >> 5, j = lane & 31;
     LaneOffsets<D> lo;
@@ -663,12 +664,17 @@ __global__ __launch_bounds__(NW * 64, (D <= 128 && NW == 4) ? 2 : 1) void dsa_ti
             _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) sacc = mfma32(ka[ks], qB[ks], sacc); \
             sched_reads_ahead<KS, 4, 1>();                                                         \
         }                                                                                          \
+        /* the wave's 32 gradients go through its own 128 bytes of LDS: one write and four 16-byte reads per lane     \
+           (element vi is key column 8*(vi/4) + 4h + vi%4) instead of sixteen lane permutes */      \
+        if (h == 0) dl_s[wv][j] = dl;                                                              \
         float ds[16];                                                                              \
-        _Pragma("unroll") for (int vi = 0; vi < 16; ++vi) {                                        \
-            const float dsv = __shfl(dl, 8 * (vi >> 2) + (vi & 3) + 4 * h, 64);   /* element vi is key column 8*(vi/4)+4h+vi%4 */ \
-            const float sv = sacc[vi];                   /* the row's weight multiplies the finished sum instead */ \
-            ds[vi] = sv > 0.f ? dsv : 0.f;                                                         \
-            dwacc = fmaf(ds[vi], sv, dwacc);             /* dscore * relu(s) */                     \
+        _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {                                         \
+            const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&dl_s[wv][8 * g4 + 4 * h]);          \
+            _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                        \
+                const float sv = sacc[4 * g4 + e];       /* the row's weight multiplies the finished sum instead */ \
+                ds[4 * g4 + e] = sv > 0.f ? d4[e] : 0.f;                                           \
+                dwacc = fmaf(ds[4 * g4 + e], sv, dwacc); /* dscore * relu(s) */                     \
+            }                                                                                      \
         }                                                                                          \
         const bf16x8 dB0 = pack8(ds), dB1 = pack8(ds + 8);                                         \
         _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                        \
