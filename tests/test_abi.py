@@ -68,6 +68,19 @@ def test_argument_errors_are_reported_not_thrown():
     assert rc == -1 and b"cu_seqlens" in lib.dsa_last_error()
     with pytest.raises(ValueError):
         _lib.check(rc, "dsa_attn_fwd")
+    # the entry points that read or leave a selection bitmap, and the small ones beside them: refused before any launch
+    import ctypes
+    cu = (ctypes.c_int32 * 2)(0, 8)
+    rc = lib.dsa_attn_fwd_saved_bitmap(None, None, None, None, None, cu, 8, 1, 4, 2, 64, 0, 1.0, 0, 8, 1, None, None, None, 0, None)
+    assert rc == -1 and b"idx is null" in lib.dsa_last_error()
+    one = ctypes.c_int32(0)
+    rc = lib.dsa_index_topk_bitmap(None, None, None, cu, 8, 1, 4, 64, 4, 1.0, 0, 8, ctypes.byref(one), ctypes.byref(one), None,
+                                   None, 0, None, 0, None)
+    assert rc == -3 and b"selection bitmap" in lib.dsa_last_error()
+    assert lib.dsa_round_bf16_x3(None, None, None, 4, 0, 0, None, None, None, None) == -1
+    assert lib.dsa_round_bf16_x3(None, None, None, 0, 0, 0, None, None, None, None) == 0       # nothing to do
+    assert lib.dsa_split_bf16_stack_qkv(None, None, None, 0, 0, 64, None, None, None, None) == 0
+    assert lib.dsa_split_bf16_combine_qkv(None, None, None, 4, 0, 64, None, None, None, None) == -1
 
 
 def test_cpu_tensors_are_refused_loudly():
