@@ -298,9 +298,77 @@ __global__ __launch_bounds__(256) void dsa_indexer_kl_kernel(const float *__rest
     if (threadIdx.x == 0) loss[t] = nt > 0 ? acc : 0.f;
 }
 
+// The same for rows of at most 256 * NV scores (K a multiple of 4, rows 16-byte aligned): one wave per row, the row read
+// once with all its 16-byte loads in flight and held in registers, reductions inside the wave - no pass over the row
+// waits for another and no barrier (the kernel above reads the scores three times and meets at three barriers).
+template <int NV>
+__global__ __launch_bounds__(256) void dsa_indexer_kl_rows_kernel(const float *__restrict__ sel, const float *__restrict__ mass,
+                                                                   const int32_t *__restrict__ nsel, int T, int K,
+                                                                   float grad_scale, float *__restrict__ loss,
+                                                                   float *__restrict__ dscore) {
+    const int lane = threadIdx.x & 63, t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= T) return;                                  // (whole waves; nothing below synchronises the workgroup)
+    const int nt = nsel[t], K4 = K >> 2;
+    const float4 *irow = reinterpret_cast<const float4 *>(sel + (int64_t)t * K);
+    const float4 *prow = reinterpret_cast<const float4 *>(mass + (int64_t)t * K);
+    float s[NV][4], p[NV][4];
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int i4 = lane + 64 * u;
+        const float4 a = irow[min(i4, K4 - 1)], b = prow[min(i4, K4 - 1)];
+        s[u][0] = a.x; s[u][1] = a.y; s[u][2] = a.z; s[u][3] = a.w;
+        p[u][0] = b.x; p[u][1] = b.y; p[u][2] = b.z; p[u][3] = b.w;
+    }
+    float m = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < NV; ++u)
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            if (4 * (lane + 64 * u) + c < nt) m = fmaxf(m, s[u][c]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    float z = 0.f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u)
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            if (4 * (lane + 64 * u) + c < nt) z += __expf(s[u][c] - m);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) z += __shfl_xor(z, off, 64);
+    const float lse = m + __logf(z);
+    float acc = 0.f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int i4 = lane + 64 * u;
+        float g[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            g[c] = 0.f;
+            if (4 * i4 + c < nt) {
+                const float logq = s[u][c] - lse;
+                if (p[u][c] > 0.f) acc += p[u][c] * (__logf(p[u][c]) - logq);
+                g[c] = (__expf(logq) - p[u][c]) * grad_scale;
+            }
+        }
+        if (dscore && i4 < K4) reinterpret_cast<float4 *>(dscore + (int64_t)t * K)[i4] = make_float4(g[0], g[1], g[2], g[3]);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if (lane == 0) loss[t] = nt > 0 ? acc : 0.f;
+}
+
 extern "C" hipError_t dsa_launch_indexer_kl(const float *sel, const float *mass, const int32_t *n, int T, int K,
                                             float grad_scale, float *loss, float *dscore, hipStream_t stream) {
     if (T <= 0) return hipSuccess;
-    hipLaunchKernelGGL(dsa_indexer_kl_kernel, dim3(T), dim3(256), 0, stream, sel, mass, n, K, grad_scale, loss, dscore);
+    const bool rows16 = K % 4 == 0 && ((reinterpret_cast<uintptr_t>(sel) | reinterpret_cast<uintptr_t>(mass) |
+                                        reinterpret_cast<uintptr_t>(dscore)) & 15) == 0;
+    const dim3 grid((unsigned)((T + 3) / 4));
+#define KL_ROWS(NV) hipLaunchKernelGGL(dsa_indexer_kl_rows_kernel<NV>, grid, dim3(256), 0, stream, sel, mass, n, T, K, grad_scale, loss, dscore)
+    if (rows16 && K <= 256) KL_ROWS(1);
+    else if (rows16 && K <= 512) KL_ROWS(2);
+    else if (rows16 && K <= 1024) KL_ROWS(4);
+    else if (rows16 && K <= 2048) KL_ROWS(8);
+    else hipLaunchKernelGGL(dsa_indexer_kl_kernel, dim3(T), dim3(256), 0, stream, sel, mass, n, K, grad_scale, loss, dscore);
+#undef KL_ROWS
     return hipGetLastError();
 }
