@@ -165,15 +165,19 @@ def indexer_target_stage(w, t, iters):
     and the indexer backward (query side 4*Hi*Di, key side 4*Hi*Di flop per causal pair of a visited tile)."""
     from vlm_training_amd import ops
     cu, msl, scale = t["cu_seqlens"], w.max_seqlen, w.D ** -0.5
-    idx, n, sel = ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k, return_scores=True)
-    out, lse = ops.attn_fwd(t["q"], t["k"], t["v"], idx, n, cu, msl, scale)
-    ms = timed(lambda: ops.attn_mass(t["q"], t["k"], lse, idx, n, cu, msl, scale), iters)
+    # as the operator runs them: the selection kernel leaves the bitmap (and the selected scores), forward and mass read it
+    lib = ops._lib.load()
+    bm = torch.empty((max(lib.dsa_attn_fwd_workspace_bytes(w.T, msl, 1), 4),), dtype=torch.uint8, device=t["q"].device) \
+        if lib.dsa_get_tile_crossover() > 0 else None
+    idx, n, sel = ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k, return_scores=True, bitmap=bm)
+    out, lse = ops.attn_fwd(t["q"], t["k"], t["v"], idx, n, cu, msl, scale, ws=bm, bitmap_ready=bm is not None)
+    ms = timed(lambda: ops.attn_mass(t["q"], t["k"], lse, idx, n, cu, msl, scale, bitmap=bm), iters)
     P, S = w.pair_counts()
     res = {"attn_mass": {"ms": ms, "selected_pair_TFLOP/s": 2.0 * w.Hq * w.D * S / ms / 1e9,
                          "partial_table_GB/s": 2.0 * w.Hkv * 4 * S / ms / 1e6}}
-    mass = ops.attn_mass(t["q"], t["k"], lse, idx, n, cu, msl, scale)
+    mass = ops.attn_mass(t["q"], t["k"], lse, idx, n, cu, msl, scale, bitmap=bm)
     res["index_topk_with_scores_ms"] = timed(
-        lambda: ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k, return_scores=True), iters)
+        lambda: ops.index_topk(t["q_idx"], t["k_idx"], t["w_idx"], cu, msl, w.top_k, return_scores=True, bitmap=bm), iters)
     res["indexer_kl_ms"] = timed(lambda: ops.indexer_kl(sel, mass, n), iters)
     loss, dscore = ops.indexer_kl(sel, mass, n)
     res["mean_kl"] = float(loss.mean())

@@ -174,6 +174,14 @@ int dsa_attn_mass(const void *q, const void *k, const float *lse, const int32_t 
                   const int32_t *cu_seqlens, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
                   int dtype, int max_seqlen, float *mass, void *ws, size_t ws_bytes, void *stream);
 size_t dsa_attn_mass_workspace_bytes(int T, int N, int Hq, int Hkv, int D, int K, int max_seqlen);
+/* dsa_attn_mass reading the selection bitmap that dsa_index_topk_bitmap or a forward left (the same idx, n, cu_seqlens
+ * and max_seqlen) instead of building its own; ws then holds only what dsa_attn_mass_workspace_bytes() asks for beyond
+ * dsa_attn_fwd_workspace_bytes(T, max_seqlen, 1) - nothing at all where one workgroup holds every kv head (ws may be
+ * NULL then). */
+int dsa_attn_mass_saved_bitmap(const void *q, const void *k, const float *lse, const int32_t *idx, const int32_t *n,
+                               const int32_t *cu_seqlens, int T, int N, int Hq, int Hkv, int D, int K,
+                               float softmax_scale, int dtype, int max_seqlen, float *mass, const void *bitmap,
+                               size_t bitmap_bytes, void *ws, size_t ws_bytes, void *stream);
 
 /*
  * Tuning knob (process-wide, no reference counterpart): query rows whose position in their segment is

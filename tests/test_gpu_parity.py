@@ -910,6 +910,11 @@ def test_attention_mass_matches_the_oracle(Hq, Hkv, D, K, segs):
     assert float(mass[pad].abs().sum()) == 0.0
     again = ops.attn_mass(d["q"], d["k"], lse, idx, n, d["cu_seqlens"], w.max_seqlen, scale)
     assert torch.equal(mass, again)                       # fixed summation order: bit-identical from run to run
+    # with the bitmap the selection kernel left instead of one built here: the same bits
+    bm = torch.empty((ops._lib.load().dsa_attn_fwd_workspace_bytes(w.T, w.max_seqlen, 1),), dtype=torch.uint8, device=DEV)
+    idx2, n2 = ops.index_topk(d["q_idx"], d["k_idx"], d["w_idx"], d["cu_seqlens"], w.max_seqlen, K, bitmap=bm)
+    assert torch.equal(idx2, idx) and torch.equal(n2, n)
+    assert torch.equal(ops.attn_mass(d["q"], d["k"], lse, idx, n, d["cu_seqlens"], w.max_seqlen, scale, bitmap=bm), mass)
 
 
 def test_operator_returns_the_mass_beside_the_output_and_stays_differentiable():

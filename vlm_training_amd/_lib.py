@@ -50,6 +50,9 @@ _SIGNATURES = {
     "dsa_attn_fwd_saved_bitmap": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                           c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                           c_size_t, c_void_p]),
+    "dsa_attn_mass_saved_bitmap": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                           c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p,
+                                           c_size_t, c_void_p]),
     "dsa_set_bwd_overlap": (c_int, [c_int]),
     "dsa_get_bwd_overlap": (c_int, []),
     "dsa_attn_bwd_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),

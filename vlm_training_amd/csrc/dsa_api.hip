@@ -348,25 +348,48 @@ extern "C" size_t dsa_attn_mass_workspace_bytes(int T, int N, int Hq, int Hkv, i
     return align_up((size_t)T * bitmap_ldw(max_seqlen) * 4, 256) + (g > 1 ? align_up((size_t)g * T * K * 4, 256) : 0);
 }
 
-extern "C" int dsa_attn_mass(const void *q, const void *k, const float *lse, const int32_t *idx, const int32_t *n,
-                             const int32_t *cu, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
-                             int dtype, int max_seqlen, float *mass, void *ws, size_t ws_bytes, void *stream) {
+// saved_bitmap != NULL: the bitmap of idx/n exists already (left by dsa_index_topk_bitmap or a forward) and is only read;
+// ws then holds the partial tables alone
+static int attn_mass_run(const void *q, const void *k, const float *lse, const int32_t *idx, const int32_t *n, const int32_t *cu,
+                         int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale, int dtype, int max_seqlen, float *mass,
+                         const void *saved_bitmap, size_t saved_bytes, void *ws, size_t ws_bytes, void *stream) {
     if (int rc = check_attn(T, N, cu, Hq, Hkv, D, K, dtype, idx, n)) return rc;
     if (!q || !k || !lse || !idx || !n || !mass) return fail(DSA_ERR_ARG, "null tensor pointer");
     if (max_seqlen < 1 || max_seqlen > (T > 0 ? T : 1)) return fail(DSA_ERR_ARG, "max_seqlen=%d outside [1,T=%d]", max_seqlen, T);
     if (T == 0) return DSA_OK;
-    const size_t need = dsa_attn_mass_workspace_bytes(T, N, Hq, Hkv, D, K, max_seqlen);
-    if (!ws || ws_bytes < need) return fail(DSA_ERR_WORKSPACE, "mass workspace: have %zu bytes, need %zu", ws_bytes, need);
     const int ldw = bitmap_ldw(max_seqlen);
+    const size_t bm = align_up((size_t)T * ldw * 4, 256);
+    const size_t need = dsa_attn_mass_workspace_bytes(T, N, Hq, Hkv, D, K, max_seqlen) - (saved_bitmap ? bm : 0);
+    if (need && (!ws || ws_bytes < need)) return fail(DSA_ERR_WORKSPACE, "mass workspace: have %zu bytes, need %zu", ws_bytes, need);
+    if (saved_bitmap && saved_bytes < bm) return fail(DSA_ERR_WORKSPACE, "selection bitmap: have %zu bytes, need %zu", saved_bytes, bm);
     if ((size_t)ldw * 4 > 64 * 1024) return fail(DSA_ERR_UNSUPPORTED, "max_seqlen=%d: selection bitmap row exceeds 64 KiB of LDS", max_seqlen);
     hipStream_t st = (hipStream_t)stream;
-    uint32_t *bitmap = (uint32_t *)ws;
-    float *partial = (float *)((char *)ws + align_up((size_t)T * ldw * 4, 256));
-    hipError_t e = dsa_launch_bitmap(idx, n, cu, N, T, K, ldw, bitmap, st);
-    if (e != hipSuccess) return hip_fail(e, "bitmap launch");
+    const uint32_t *bitmap = saved_bitmap ? (const uint32_t *)saved_bitmap : (const uint32_t *)ws;
+    float *partial = (float *)((char *)ws + (saved_bitmap ? 0 : bm));
+    hipError_t e = hipSuccess;
+    if (!saved_bitmap) {
+        e = dsa_launch_bitmap(idx, n, cu, N, T, K, ldw, (uint32_t *)ws, st);
+        if (e != hipSuccess) return hip_fail(e, "bitmap launch");
+    }
     e = dsa_launch_tile_mass(q, k, lse, bitmap, ldw, n, cu, N, T, Hq, Hkv, D, K, softmax_scale, partial, mass, st);
     if (e != hipSuccess) return hip_fail(e, "attention mass launch");
     return DSA_OK;
+}
+
+extern "C" int dsa_attn_mass(const void *q, const void *k, const float *lse, const int32_t *idx, const int32_t *n,
+                             const int32_t *cu, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
+                             int dtype, int max_seqlen, float *mass, void *ws, size_t ws_bytes, void *stream) {
+    return attn_mass_run(q, k, lse, idx, n, cu, T, N, Hq, Hkv, D, K, softmax_scale, dtype, max_seqlen, mass, nullptr, 0, ws,
+                         ws_bytes, stream);
+}
+
+extern "C" int dsa_attn_mass_saved_bitmap(const void *q, const void *k, const float *lse, const int32_t *idx, const int32_t *n,
+                                          const int32_t *cu, int T, int N, int Hq, int Hkv, int D, int K, float softmax_scale,
+                                          int dtype, int max_seqlen, float *mass, const void *bitmap, size_t bitmap_bytes,
+                                          void *ws, size_t ws_bytes, void *stream) {
+    if (!bitmap) return fail(DSA_ERR_ARG, "null selection bitmap");
+    return attn_mass_run(q, k, lse, idx, n, cu, T, N, Hq, Hkv, D, K, softmax_scale, dtype, max_seqlen, mass, bitmap,
+                         bitmap_bytes, ws, ws_bytes, stream);
 }
 
 // ---- the query-side and the key-side pass of one backward side by side ----

@@ -311,10 +311,13 @@ def attn_fwd(q, k, v, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: float,
     return out, lse
 
 
-def attn_mass(q, k, lse, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: Optional[float] = None) -> torch.Tensor:
+def attn_mass(q, k, lse, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: Optional[float] = None,
+              bitmap=None) -> torch.Tensor:
     """Head-averaged attention probability of every selected key, (T, K) fp32, rows summing to one: the target
     of the KL loss that trains the indexer.  ``lse`` (Hq, T) is the forward's second output for the same
-    q, k, idx.  Nothing here is differentiable (the target is detached in DSA's objective)."""
+    q, k, idx.  ``bitmap``: the selection bitmap of this idx/n and max_seqlen, if the caller holds it (the forward's
+    workspace), so that none is built here.  Nothing here is differentiable (the target is detached in DSA's
+    objective)."""
     _require_cuda(q, k, lse, idx, n, cu_seqlens)
     T, Hq, D = q.shape
     Hkv, K = k.shape[1], idx.shape[1]
@@ -327,6 +330,14 @@ def attn_mass(q, k, lse, idx, n, cu_seqlens, max_seqlen: int, softmax_scale: Opt
     qb, kb = _as_bf16(q), _as_bf16(k)
     mass = torch.empty((T, K), dtype=torch.float32, device=q.device)
     ws_bytes = lib.dsa_attn_mass_workspace_bytes(T, cu.numel() - 1, Hq, Hkv, D, K, max_seqlen)
+    if bitmap is not None:
+        ws_bytes -= lib.dsa_attn_fwd_workspace_bytes(T, max_seqlen, 1)       # the partial tables alone (often nothing)
+        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=q.device) if ws_bytes else None
+        rc = lib.dsa_attn_mass_saved_bitmap(_ptr(qb), _ptr(kb), _ptr(lse.contiguous()), _ptr(idx), _ptr(n), _ptr(cu), T,
+                                            cu.numel() - 1, Hq, Hkv, D, K, scale, _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(mass),
+                                            _ptr(bitmap), bitmap.numel(), _ptr(ws), ws_bytes, _stream(q.device))
+        _lib.check(rc, "dsa_attn_mass_saved_bitmap")
+        return mass
     ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=q.device)
     rc = lib.dsa_attn_mass(_ptr(qb), _ptr(kb), _ptr(lse.contiguous()), _ptr(idx), _ptr(n), _ptr(cu), T, cu.numel() - 1, Hq,
                            Hkv, D, K, scale, _lib.DSA_DTYPE_BF16, max_seqlen, _ptr(mass), _ptr(ws), ws_bytes,
@@ -468,7 +479,7 @@ class _DsaVarlenAttn(torch.autograd.Function):
         if not want_mass:
             return res
         # from the very operands and log-sum-exp of the forward, so that every row sums to one
-        mass = attn_mass(qb, kb, lse, idx, n, cu_seqlens, int(max_seqlen), softmax_scale)
+        mass = attn_mass(qb, kb, lse, idx, n, cu_seqlens, int(max_seqlen), softmax_scale, bitmap=fwd_ws)
         ctx.mark_non_differentiable(mass)
         return res, mass
 
